@@ -1,0 +1,213 @@
+// Host side of the C ABI declared in include/fdb.h: argument validation, the integer delta
+// table, and dispatch to the device launchers.  No device memory is allocated here.
+#include <math.h>
+#include <stdint.h>
+#include <string.h>
+
+#include <hip/hip_runtime_api.h>
+
+#include "../../include/fdb.h"
+#include "fdb_kernels.h"
+
+namespace {
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int qk_elem_size(int dtype) {
+  switch (dtype) {
+    case FDB_F32: return 4;
+    case FDB_BF16:
+    case FDB_F16: return 2;
+    case FDB_FP8_E4M3: return 1;
+    default: return 0;
+  }
+}
+int v_elem_size(int dtype) { return dtype == FDB_F32 ? 4 : 2; }
+
+// DeBERTa's signed log bucket (transformers modeling_deberta_v2.py:56-69), evaluated in fp32 in
+// the same operation order as the eager code: ceil(log(a/mid) / log((max-1)/mid) * (mid-1)) + mid.
+int32_t log_bucket(int32_t r, int32_t bucket_size, int32_t max_position) {
+  const int32_t mid = bucket_size / 2;
+  const int32_t a = r < 0 ? -r : r;
+  if (a <= mid) return r;  // |r| < mid is mapped to mid-1 <= mid, |r| == mid stays: both take the identity branch
+  const float num = logf((float)a / (float)mid);
+  const float den = logf((float)(max_position - 1) / (float)mid);
+  const float pos = ceilf(num / den * (float)(mid - 1)) + (float)mid;
+  const int32_t bkt = (int32_t)pos;
+  return r < 0 ? -bkt : bkt;
+}
+
+int32_t delta_of(int32_t r, int32_t position_buckets, int32_t max_position) {
+  int32_t span, rel;
+  if (position_buckets > 0) {
+    span = position_buckets;
+    rel = log_bucket(r, position_buckets, max_position);
+  } else {
+    span = max_position;
+    rel = r;
+  }
+  int64_t d = (int64_t)rel + span;
+  if (d < 0) d = 0;
+  if (d > 2 * (int64_t)span - 1) d = 2 * (int64_t)span - 1;
+  return (int32_t)d;
+}
+
+bool lut_config_ok(int32_t position_buckets, int32_t max_position) {
+  if (max_position < 1) return false;
+  if (position_buckets > 0) {
+    const int32_t mid = position_buckets / 2;
+    if (position_buckets > 16383) return false;
+    if (mid < 2) return false;                 // log zone degenerates (mid-1 == 0)
+    if (max_position - 1 <= mid) return false; // log((max-1)/mid) <= 0: eager divides by it
+  } else if (max_position > 16383) {
+    return false;
+  }
+  return true;
+}
+
+constexpr int32_t kRadiusCap = 1 << 22;
+
+}  // namespace
+
+extern "C" {
+
+int fdb_version(void) { return FDB_VERSION; }
+
+const char* fdb_strerror(int code) {
+  switch (code) {
+    case FDB_OK: return "ok";
+    case FDB_ERR_NULL: return "required pointer is NULL";
+    case FDB_ERR_DTYPE: return "unknown dtype";
+    case FDB_ERR_HEAD_DIM: return "unsupported head_dim (supported: 32, 64, 128)";
+    case FDB_ERR_ALIGN: return "pointer or stride is not 16-byte aligned";
+    case FDB_ERR_SHAPE: return "batch/heads/max_seqlen/total_tokens invalid";
+    case FDB_ERR_SPAN: return "att_span/lut_radius/delta_lut invalid while a position term is present";
+    case FDB_ERR_SCALE: return "fp8 dtype needs q_scale, k_scale and a scale for each position tensor";
+    case FDB_ERR_WORKLIST: return "cu_seqlens given without a work-list buffer";
+    case FDB_ERR_LUT_ARGS: return "invalid position_buckets/max_position/radius/out for the delta table";
+    case FDB_ERR_UNSUPPORTED: return "dtype/head_dim combination not built";
+    default: break;
+  }
+  if (code > 0) return hipGetErrorString((hipError_t)code);
+  return "unknown error";
+}
+
+int32_t fdb_tile_rows(void) { return FDB_BM; }
+
+int32_t fdb_worklist_max_tiles(int32_t total_tokens, int32_t batch) {
+  if (total_tokens < 0 || batch < 0) return 0;
+  // sum_b ceil(L_b / BM) <= floor(T / BM) + batch
+  int64_t n = (int64_t)total_tokens / FDB_BM + batch;
+  if (n > INT32_MAX) n = INT32_MAX;
+  return (int32_t)n;
+}
+
+int64_t fdb_worklist_ints(int32_t total_tokens, int32_t batch) {
+  return 2 + 2 * (int64_t)fdb_worklist_max_tiles(total_tokens, batch);
+}
+
+int fdb_attn_check(const fdb_attn_args* a) {
+  if (!a) return FDB_ERR_NULL;
+  if (!a->q || !a->k || !a->v || !a->out) return FDB_ERR_NULL;
+  const int qsz = qk_elem_size(a->dtype);
+  if (qsz == 0) return FDB_ERR_DTYPE;
+  const int vsz = v_elem_size(a->dtype);
+  if (a->head_dim != 32 && a->head_dim != 64 && a->head_dim != 128) return FDB_ERR_HEAD_DIM;
+  if (a->dtype == FDB_F32 && a->head_dim == 128) return FDB_ERR_UNSUPPORTED;
+  if (a->batch < 1 || a->heads < 1 || a->heads > 65535 || a->max_seqlen < 1 || a->total_tokens < 1)
+    return FDB_ERR_SHAPE;
+  if (!a->cu_seqlens && (int64_t)a->batch * a->max_seqlen != a->total_tokens) return FDB_ERR_SHAPE;
+  if (a->cu_seqlens && !a->worklist) return FDB_ERR_WORKLIST;
+  const bool has_pos = a->pos_key || a->pos_query;
+  if (has_pos && (a->att_span < 1 || a->lut_radius < 1 || !a->delta_lut)) return FDB_ERR_SPAN;
+  if (a->dtype == FDB_FP8_E4M3) {
+    if (!a->q_scale || !a->k_scale) return FDB_ERR_SCALE;
+    if (a->pos_key && !a->pk_scale) return FDB_ERR_SCALE;
+    if (a->pos_query && !a->pq_scale) return FDB_ERR_SCALE;
+  }
+  if (!aligned16(a->q) || !aligned16(a->k) || !aligned16(a->v) || !aligned16(a->out)) return FDB_ERR_ALIGN;
+  if ((a->pos_key && !aligned16(a->pos_key)) || (a->pos_query && !aligned16(a->pos_query))) return FDB_ERR_ALIGN;
+  const int64_t qk_strides[] = {a->q_stride_b, a->q_stride_t, a->q_stride_h, a->k_stride_b, a->k_stride_t,
+                                a->k_stride_h, a->pos_key ? a->pk_stride_h : 0, a->pos_key ? a->pk_stride_r : 0,
+                                a->pos_query ? a->pq_stride_h : 0, a->pos_query ? a->pq_stride_r : 0};
+  for (int64_t s : qk_strides)
+    if ((s * qsz) % 16 != 0) return FDB_ERR_ALIGN;
+  const int64_t v_strides[] = {a->v_stride_b, a->v_stride_t, a->v_stride_h, a->o_stride_b, a->o_stride_t, a->o_stride_h};
+  for (int64_t s : v_strides)
+    if ((s * vsz) % 16 != 0) return FDB_ERR_ALIGN;
+  return FDB_OK;
+}
+
+int fdb_attn_fwd(const fdb_attn_args* a, void* stream) {
+  const int rc = fdb_attn_check(a);
+  if (rc != FDB_OK) return rc;
+  FdbKParams p;
+  memset(&p, 0, sizeof(p));
+  p.q = (const char*)a->q;
+  p.k = (const char*)a->k;
+  p.v = (const char*)a->v;
+  p.pk = (const char*)a->pos_key;
+  p.pq = (const char*)a->pos_query;
+  p.out = (char*)a->out;
+  p.lse = a->lse;
+  p.cu = a->cu_seqlens;
+  p.wl = a->worklist;
+  p.lut = a->delta_lut;
+  p.qs = a->q_scale; p.ks = a->k_scale; p.pks = a->pk_scale; p.pqs = a->pq_scale;
+  p.q_sb = a->q_stride_b; p.q_st = a->q_stride_t; p.q_sh = a->q_stride_h;
+  p.k_sb = a->k_stride_b; p.k_st = a->k_stride_t; p.k_sh = a->k_stride_h;
+  p.v_sb = a->v_stride_b; p.v_st = a->v_stride_t; p.v_sh = a->v_stride_h;
+  p.o_sb = a->o_stride_b; p.o_st = a->o_stride_t; p.o_sh = a->o_stride_h;
+  p.pk_sh = a->pk_stride_h; p.pk_sr = a->pk_stride_r;
+  p.pq_sh = a->pq_stride_h; p.pq_sr = a->pq_stride_r;
+  p.B = a->batch; p.H = a->heads; p.L = a->max_seqlen;
+  p.tiles_per_seq = (a->max_seqlen + FDB_BM - 1) / FDB_BM;
+  p.R = a->lut_radius > 0 ? a->lut_radius : 1;
+  p.r_neg = -p.R; p.r_pos = p.R;
+  p.causal = a->causal ? 1 : 0;
+  p.scale_log2 = a->sm_scale * 1.4426950408889634f;
+  int64_t grid_x = a->cu_seqlens ? fdb_worklist_max_tiles(a->total_tokens, a->batch)
+                                 : (int64_t)a->batch * p.tiles_per_seq;
+  if (grid_x < 1 || grid_x > INT32_MAX) return FDB_ERR_SHAPE;
+  return fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, stream);
+}
+
+int fdb_build_worklist(const int32_t* cu_seqlens, int32_t batch, int32_t total_tokens, int32_t* worklist,
+                       void* stream) {
+  if (!cu_seqlens || !worklist) return FDB_ERR_NULL;
+  if (batch < 1 || total_tokens < 0) return FDB_ERR_SHAPE;
+  return fdb_launch_worklist(cu_seqlens, batch, worklist, fdb_worklist_max_tiles(total_tokens, batch), stream);
+}
+
+int32_t fdb_delta_lut_radius(int32_t position_buckets, int32_t max_position) {
+  if (!lut_config_ok(position_buckets, max_position)) return FDB_ERR_LUT_ARGS;
+  const int32_t span = position_buckets > 0 ? position_buckets : max_position;
+  // delta is non-decreasing in r; find where each side reaches its clamp value
+  int32_t r = 1;
+  while (r < kRadiusCap && !(delta_of(r, position_buckets, max_position) == 2 * span - 1 &&
+                             delta_of(-r, position_buckets, max_position) == 0))
+    ++r;
+  return r;
+}
+
+int fdb_delta_lut(int32_t position_buckets, int32_t max_position, int32_t radius, int16_t* out) {
+  if (!out || radius < 1 || radius > kRadiusCap || !lut_config_ok(position_buckets, max_position))
+    return FDB_ERR_LUT_ARGS;
+  for (int32_t r = -radius; r <= radius; ++r) out[r + radius] = (int16_t)delta_of(r, position_buckets, max_position);
+  return FDB_OK;
+}
+
+int fdb_quant_e4m3_per_head(const void* x, int64_t x_stride_t, int64_t x_stride_h, void* y, int64_t y_stride_t,
+                            int64_t y_stride_h, float* scale, uint32_t* absmax_ws, int32_t tokens, int32_t heads,
+                            int32_t head_dim, void* stream) {
+  if (!x || !y || !scale || !absmax_ws) return FDB_ERR_NULL;
+  if (head_dim != 32 && head_dim != 64 && head_dim != 128) return FDB_ERR_HEAD_DIM;
+  if (tokens < 1 || heads < 1 || heads > 65535) return FDB_ERR_SHAPE;
+  if (!aligned16(x) || (reinterpret_cast<uintptr_t>(y) & 7u) || (x_stride_t * 2) % 16 || (x_stride_h * 2) % 16 ||
+      y_stride_t % 8 || y_stride_h % 8)
+    return FDB_ERR_ALIGN;
+  return fdb_launch_quant(x, x_stride_t, x_stride_h, y, y_stride_t, y_stride_h, scale, absmax_ws, tokens, heads,
+                          head_dim, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,137 @@
+// Small helper kernels around the fused attention: the varlen q-tile work-list built on the
+// device from cu_seqlens (the reference builds it in a Python loop with one host sync per
+// sequence, src/flashdeberta/ops/flash_attention_varlen.py:71-83) and the per-head absmax ->
+// OCP e4m3 quantisation of the FP8 Q/K variant.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "fdb_kernels.h"
+
+namespace {
+
+constexpr int kWlThreads = 256;
+
+// wl[0] = number of tiles, wl[1] = 0, then (sequence, first row) pairs in sequence order.
+__global__ __launch_bounds__(kWlThreads) void fdb_worklist_kernel(const int32_t* __restrict__ cu, int32_t batch,
+                                                                  int32_t* __restrict__ wl, int32_t max_tiles) {
+  __shared__ int32_t part[kWlThreads];
+  const int t = threadIdx.x;
+  const int per = (batch + kWlThreads - 1) / kWlThreads;
+  const int b_lo = min(batch, t * per), b_hi = min(batch, b_lo + per);
+  int32_t cnt = 0;
+  for (int b = b_lo; b < b_hi; ++b) cnt += (max(cu[b + 1] - cu[b], 0) + FDB_BM - 1) / FDB_BM;
+  part[t] = cnt;
+  __syncthreads();
+  // exclusive scan over 256 partial counts (Hillis-Steele)
+  for (int off = 1; off < kWlThreads; off <<= 1) {
+    int32_t add = (t >= off) ? part[t - off] : 0;
+    __syncthreads();
+    part[t] += add;
+    __syncthreads();
+  }
+  int32_t pos = part[t] - cnt;
+  if (t == kWlThreads - 1) {
+    wl[0] = min(part[t], max_tiles);
+    wl[1] = 0;
+  }
+  for (int b = b_lo; b < b_hi; ++b) {
+    const int len = max(cu[b + 1] - cu[b], 0);
+    for (int m0 = 0; m0 < len; m0 += FDB_BM, ++pos)
+      if (pos < max_tiles) {
+        wl[2 + 2 * pos] = b;
+        wl[3 + 2 * pos] = m0;
+      }
+  }
+}
+
+__global__ void fdb_fill_u32(uint32_t* p, int n, uint32_t v) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __builtin_bit_cast(float, (uint32_t)b << 16); }
+
+// grid (token blocks, heads); each thread owns 8 consecutive d of one token.
+template <int D>
+__global__ __launch_bounds__(256) void fdb_absmax_kernel(const uint16_t* __restrict__ x, int64_t st, int64_t sh,
+                                                         uint32_t* __restrict__ absmax, int32_t tokens) {
+  constexpr int CPT = D / 8;  // 16-byte chunks per token row
+  const int h = blockIdx.y;
+  float m = 0.f;
+  for (int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; c < (int64_t)tokens * CPT;
+       c += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t t = c / CPT;
+    const int cc = (int)(c % CPT);
+    const uint4 raw = *(const uint4*)(x + t * st + h * sh + cc * 8);
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      m = fmaxf(m, fabsf(bf16_bits_to_f32((uint16_t)(w[e] & 0xffffu))));
+      m = fmaxf(m, fabsf(bf16_bits_to_f32((uint16_t)(w[e] >> 16))));
+    }
+  }
+  for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+  if ((threadIdx.x & 63) == 0) atomicMax(absmax + h, __builtin_bit_cast(uint32_t, m));  // m >= 0: bit order = value order
+}
+
+template <int D>
+__global__ __launch_bounds__(256) void fdb_quant_kernel(const uint16_t* __restrict__ x, int64_t st, int64_t sh,
+                                                        uint8_t* __restrict__ y, int64_t yst, int64_t ysh,
+                                                        const uint32_t* __restrict__ absmax, float* __restrict__ scale,
+                                                        int32_t tokens) {
+  constexpr int CPT = D / 8;
+  const int h = blockIdx.y;
+  const float amax = fmaxf(__builtin_bit_cast(float, absmax[h]), 1e-12f);
+  const float sc = amax / 448.0f;
+  if (blockIdx.x == 0 && threadIdx.x == 0) scale[h] = sc;
+  for (int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; c < (int64_t)tokens * CPT;
+       c += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t t = c / CPT;
+    const int cc = (int)(c % CPT);
+    const uint4 raw = *(const uint4*)(x + t * st + h * sh + cc * 8);
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+    float f[8];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      f[2 * e] = fminf(fmaxf(bf16_bits_to_f32((uint16_t)(w[e] & 0xffffu)) / sc, -448.f), 448.f);
+      f[2 * e + 1] = fminf(fmaxf(bf16_bits_to_f32((uint16_t)(w[e] >> 16)) / sc, -448.f), 448.f);
+    }
+    uint32_t outw[2];
+    // two e4m3 bytes per conversion: low half of the word first, then the high half
+    outw[0] = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], 0, false);
+    outw[0] = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], outw[0], true);
+    outw[1] = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], 0, false);
+    outw[1] = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], outw[1], true);
+    *(uint2*)(y + t * yst + h * ysh + cc * 8) = uint2{outw[0], outw[1]};
+  }
+}
+
+}  // namespace
+
+int fdb_launch_worklist(const int32_t* cu, int32_t batch, int32_t* wl, int32_t max_tiles, void* stream) {
+  hipLaunchKernelGGL(fdb_worklist_kernel, dim3(1), dim3(kWlThreads), 0, (hipStream_t)stream, cu, batch, wl, max_tiles);
+  return (int)hipGetLastError();
+}
+
+int fdb_launch_quant(const void* x, int64_t x_st, int64_t x_sh, void* y, int64_t y_st, int64_t y_sh, float* scale,
+                     uint32_t* absmax_ws, int32_t tokens, int32_t heads, int32_t head_dim, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  hipLaunchKernelGGL(fdb_fill_u32, dim3((heads + 255) / 256), dim3(256), 0, stream, absmax_ws, heads, 0u);
+  const int64_t chunks = (int64_t)tokens * head_dim / 8;
+  int gx = (int)((chunks + 255) / 256);
+  if (gx > 1024) gx = 1024;
+  if (gx < 1) gx = 1;
+#define FDB_Q(DD)                                                                                              \
+  hipLaunchKernelGGL(fdb_absmax_kernel<DD>, dim3(gx, heads), dim3(256), 0, stream, (const uint16_t*)x, x_st,   \
+                     x_sh, absmax_ws, tokens);                                                                 \
+  hipLaunchKernelGGL(fdb_quant_kernel<DD>, dim3(gx, heads), dim3(256), 0, stream, (const uint16_t*)x, x_st,    \
+                     x_sh, (uint8_t*)y, y_st, y_sh, absmax_ws, scale, tokens);
+  switch (head_dim) {
+    case 32: FDB_Q(32) break;
+    case 64: FDB_Q(64) break;
+    case 128: FDB_Q(128) break;
+    default: return -3;
+  }
+#undef FDB_Q
+  return (int)hipGetLastError();
+}

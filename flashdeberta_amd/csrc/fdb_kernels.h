@@ -1,0 +1,44 @@
+// Internal interface between the host-side C ABI (fdb_api.cpp) and the device code
+// (fdb_attn.hip, fdb_aux.hip).  Not installed; the public contract is include/fdb.h.
+#pragma once
+#include <stdint.h>
+
+// Query rows per workgroup (4 waves x 32 rows) and keys per main-loop iteration.
+#define FDB_BM 128
+#define FDB_BN 64
+
+struct FdbKParams {
+  const char* q;
+  const char* k;
+  const char* v;
+  const char* pk;  // K_r, NULL when the content->position term is absent
+  const char* pq;  // Q_r, NULL when the position->content term is absent
+  char* out;
+  float* lse;
+  const int32_t* cu;   // cu_seqlens or NULL
+  const int32_t* wl;   // work-list (varlen only)
+  const int16_t* lut;  // delta LUT, index r + R
+  const float* qs;     // fp8 dequant scales per head (NULL otherwise)
+  const float* ks;
+  const float* pks;
+  const float* pqs;
+  int64_t q_sb, q_st, q_sh;
+  int64_t k_sb, k_st, k_sh;
+  int64_t v_sb, v_st, v_sh;
+  int64_t o_sb, o_st, o_sh;
+  int64_t pk_sh, pk_sr;
+  int64_t pq_sh, pq_sr;
+  int32_t B, H, L, tiles_per_seq;
+  int32_t R;        // LUT radius
+  int32_t r_neg;    // delta(r) == delta(-R) for every r <= r_neg
+  int32_t r_pos;    // delta(r) == delta(+R) for every r >= r_pos
+  int32_t causal;
+  float scale_log2; // sm_scale * log2(e)
+};
+
+// Launchers return the hipError_t of the launch as int.
+int fdb_launch_attn(const FdbKParams& p, int dtype, int head_dim, int grid_x, void* stream);
+int fdb_launch_worklist(const int32_t* cu, int32_t batch, int32_t* wl, int32_t max_tiles, void* stream);
+int fdb_launch_quant(const void* x, int64_t x_st, int64_t x_sh, void* y, int64_t y_st, int64_t y_sh,
+                     float* scale, uint32_t* absmax_ws, int32_t tokens, int32_t heads, int32_t head_dim,
+                     void* stream);

@@ -1,0 +1,223 @@
+"""Operators of the disentangled-attention forward on MI355X.
+
+Counterparts in the reference (src/flashdeberta/ops/):
+  flash_attention_with_disentangled        flash_attention.py:1088-1091
+  flash_attention_with_disentangled_varlen flash_attention_varlen.py:485-511
+The reference ops take the pre-multiplied bias tensors Q.K_r^T and K.Q_r^T ([B,H,L,2S], built by
+src/flashdeberta/model.py:189-192 / :210-214).  Here those products are fused into the kernel, so
+the ops take the factors K_r / Q_r ([H, 2S, D], the projected relative embeddings) instead.
+"""
+import ctypes
+import math
+
+import numpy as np
+import torch
+
+from . import _lib
+from ._lib import FdbAttnArgs, check, lib
+
+_DTYPES = {torch.float32: _lib.FDB_F32, torch.bfloat16: _lib.FDB_BF16, torch.float16: _lib.FDB_F16}
+_FP8 = torch.float8_e4m3fn
+
+_lut_host_cache = {}
+_lut_dev_cache = {}
+
+
+def att_span(position_buckets, max_relative_positions):
+    """S of the reference (flash_attention.py:1045): buckets if bucketing is on, else the max distance."""
+    return position_buckets if position_buckets > 0 else max_relative_positions
+
+
+def delta_lut_host(position_buckets, max_relative_positions):
+    """(int16 numpy array of delta(r) for r = -R..R, R).  Pure host code (no GPU needed)."""
+    key = (int(position_buckets), int(max_relative_positions))
+    hit = _lut_host_cache.get(key)
+    if hit is not None:
+        return hit
+    radius = lib.fdb_delta_lut_radius(*key)
+    if radius < 1:
+        raise ValueError("unsupported relative-position config position_buckets=%d max_relative_positions=%d: %s"
+                         % (key[0], key[1], _lib.strerror(radius)))
+    out = np.empty(2 * radius + 1, dtype=np.int16)
+    check(lib.fdb_delta_lut(key[0], key[1], radius, out.ctypes.data_as(ctypes.c_void_p)), "fdb_delta_lut")
+    _lut_host_cache[key] = (out, radius)
+    return out, radius
+
+
+def delta_lut_device(position_buckets, max_relative_positions, device):
+    key = (int(position_buckets), int(max_relative_positions), torch.device(device))
+    hit = _lut_dev_cache.get(key)
+    if hit is None:
+        host, radius = delta_lut_host(position_buckets, max_relative_positions)
+        hit = (torch.from_numpy(host).to(device), radius)
+        _lut_dev_cache[key] = hit
+    return hit
+
+
+def _stream_ptr(device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _pos_arg(x, H, D, span, name):
+    """K_r / Q_r as [H, 2S, D] (a leading singleton batch dim as produced by the module is dropped)."""
+    if x is None:
+        return None
+    if x.dim() == 4 and x.shape[0] == 1:
+        x = x[0]
+    if x.dim() != 3 or x.shape[0] != H or x.shape[2] != D or x.shape[1] < 2 * span:
+        raise ValueError("%s must be the projected relative embeddings [H=%d, >=2S=%d, D=%d], got %s. "
+                         "(The pre-multiplied [B,H,L,2S] bias tensors of the reference op are not an input here: "
+                         "the product is fused into the kernel.)" % (name, H, 2 * span, D, tuple(x.shape)))
+    if x.stride(2) != 1:
+        x = x.contiguous()
+    return x
+
+
+def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seqlens=None, max_seqlen=None,
+                               sm_scale=None, position_buckets=0, max_relative_positions=0, causal=False,
+                               return_lse=False, q_scale=None, k_scale=None, pos_key_scale=None,
+                               pos_query_scale=None, out=None):
+    """Fused forward.  Layouts (strides are free except a unit stride on D):
+         fixed length : q, k, v  [B, L, H, D]   -> out [B, L, H, D] (contiguous: a free view of [B, L, H*D])
+         packed varlen: q, k, v  [T, H, D] + cu_seqlens int32 [B+1] (+ max_seqlen upper bound) -> out [T, H, D]
+       pos_key = K_r, pos_query = Q_r: [H, 2S, D] or None (term absent).  sm_scale defaults to
+       1/sqrt(D * (1 + #position terms)) as the reference module computes it (src/flashdeberta/model.py:151-157).
+       fp8: q/k/pos_* are torch.float8_e4m3fn with float32 per-head scales; v is bfloat16.
+    """
+    if not q.is_cuda:
+        raise RuntimeError("disentangled_attention_fwd runs on the GPU only; got device %s" % q.device)
+    varlen = cu_seqlens is not None
+    if varlen:
+        if q.dim() != 3:
+            raise ValueError("with cu_seqlens, q/k/v must be [T, H, D]")
+        T, H, D = q.shape
+        B = cu_seqlens.numel() - 1
+        L = int(max_seqlen) if max_seqlen is not None else T
+        if cu_seqlens.dtype != torch.int32 or not cu_seqlens.is_cuda:
+            raise ValueError("cu_seqlens must be an int32 tensor on the GPU")
+    else:
+        if q.dim() != 4:
+            raise ValueError("q/k/v must be [B, L, H, D] (or [T, H, D] with cu_seqlens)")
+        B, L, H, D = q.shape
+        T = B * L
+    if k.shape != q.shape or v.shape != q.shape:
+        raise ValueError("q, k, v must have the same shape (self-attention): %s %s %s"
+                         % (tuple(q.shape), tuple(k.shape), tuple(v.shape)))
+    fp8 = q.dtype == _FP8
+    if fp8:
+        if k.dtype != _FP8 or v.dtype != torch.bfloat16:
+            raise ValueError("fp8 path: q and k float8_e4m3fn, v bfloat16")
+        dt = _lib.FDB_FP8_E4M3
+    else:
+        if q.dtype not in _DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
+            raise ValueError("unsupported dtypes %s %s %s" % (q.dtype, k.dtype, v.dtype))
+        dt = _DTYPES[q.dtype]
+    q, k, v = [x if x.stride(-1) == 1 else x.contiguous() for x in (q, k, v)]
+    span = att_span(position_buckets, max_relative_positions)
+    pos_key = _pos_arg(pos_key, H, D, span, "pos_key")
+    pos_query = _pos_arg(pos_query, H, D, span, "pos_query")
+    for pname, x in (("pos_key", pos_key), ("pos_query", pos_query)):
+        if x is not None and x.dtype != q.dtype:
+            raise ValueError("%s dtype %s does not match q dtype %s" % (pname, x.dtype, q.dtype))
+    n_terms = 1 + (pos_key is not None) + (pos_query is not None)
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(D * n_terms)
+
+    a = FdbAttnArgs()
+    keep = []
+    if pos_key is not None or pos_query is not None:
+        lut, radius = delta_lut_device(position_buckets, max_relative_positions, q.device)
+        a.delta_lut, a.lut_radius, a.att_span = lut.data_ptr(), radius, span
+    if out is None:
+        out = torch.empty(q.shape, dtype=v.dtype, device=q.device)
+    elif out.shape != q.shape or out.dtype != v.dtype or out.stride(-1) != 1:
+        raise ValueError("out must have q's shape, v's dtype and a unit stride on D")
+    lse = torch.empty((T, H), dtype=torch.float32, device=q.device) if return_lse else None
+    a.q, a.k, a.v, a.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
+    a.pos_key, a.pos_query = (_ptr(pos_key) or ctypes.c_void_p()).value, (_ptr(pos_query) or ctypes.c_void_p()).value
+    a.lse = lse.data_ptr() if lse is not None else None
+    if varlen:
+        for n, x in (("q", q), ("k", k), ("v", v), ("o", out)):
+            setattr(a, n + "_stride_b", 0)
+            setattr(a, n + "_stride_t", x.stride(0))
+            setattr(a, n + "_stride_h", x.stride(1))
+        wl = torch.empty(int(lib.fdb_worklist_ints(T, B)), dtype=torch.int32, device=q.device)
+        keep.append(wl)
+        check(lib.fdb_build_worklist(_ptr(cu_seqlens), B, T, _ptr(wl), _stream_ptr(q.device)), "fdb_build_worklist")
+        a.cu_seqlens, a.worklist = cu_seqlens.data_ptr(), wl.data_ptr()
+    else:
+        for n, x in (("q", q), ("k", k), ("v", v), ("o", out)):
+            setattr(a, n + "_stride_b", x.stride(0))
+            setattr(a, n + "_stride_t", x.stride(1))
+            setattr(a, n + "_stride_h", x.stride(2))
+    if pos_key is not None:
+        a.pk_stride_h, a.pk_stride_r = pos_key.stride(0), pos_key.stride(1)
+    if pos_query is not None:
+        a.pq_stride_h, a.pq_stride_r = pos_query.stride(0), pos_query.stride(1)
+    if fp8:
+        scales = {"q_scale": q_scale, "k_scale": k_scale, "pk_scale": pos_key_scale, "pq_scale": pos_query_scale}
+        for n, s in scales.items():
+            if s is not None:
+                if s.dtype != torch.float32 or s.numel() != H or not s.is_cuda:
+                    raise ValueError("%s must be a float32 GPU tensor with one entry per head" % n)
+                s = s.contiguous()
+                keep.append(s)
+                setattr(a, n, s.data_ptr())
+    a.batch, a.heads, a.head_dim, a.max_seqlen, a.total_tokens = B, H, D, L, T
+    a.dtype, a.causal, a.sm_scale = dt, int(bool(causal)), float(sm_scale)
+    with torch.cuda.device(q.device):
+        check(lib.fdb_attn_fwd(ctypes.byref(a), _stream_ptr(q.device)), "fdb_attn_fwd")
+    return (out, lse) if return_lse else out
+
+
+def flash_attention_with_disentangled(q, k, v, k_pos, q_pos, causal=False, sm_scale=None,
+                                      position_buckets=0, max_relative_distance=0):
+    """Same call shape as the reference op (flash_attention.py:1088-1091): q, k, v [B, H, L, D],
+    returns [B, H, L, D].  k_pos / q_pos are K_r / Q_r [H, 2S, D] (see the module docstring).
+    As in the reference, sm_scale=None means 1/sqrt(D) (flash_attention.py:1042-1043)."""
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(q.shape[-1])
+    o = disentangled_attention_fwd(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), k_pos, q_pos,
+                                   sm_scale=sm_scale, position_buckets=position_buckets,
+                                   max_relative_positions=max_relative_distance, causal=causal)
+    return o.transpose(1, 2)
+
+
+def flash_attention_with_disentangled_varlen(q, k, v, q_pos, k_pos, cu_seqlens_q, cu_seqlens_k,
+                                             max_seqlen_q, max_seqlen_k, causal=False, sm_scale=None,
+                                             position_buckets=0, max_relative_distance=0):
+    """Same call shape as the reference op (flash_attention_varlen.py:485-511): q, k, v [T, H, D].
+    Positional order follows the reference: the 4th argument feeds the content->position term
+    (K_r), the 5th the position->content term (Q_r) (flash_attention_varlen.py:445,470).
+    Self-attention only: cu_seqlens_q must equal cu_seqlens_k."""
+    if cu_seqlens_q is not cu_seqlens_k and not torch.equal(cu_seqlens_q, cu_seqlens_k):
+        raise ValueError("self-attention only: cu_seqlens_q and cu_seqlens_k must match")
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(q.shape[-1])
+    return disentangled_attention_fwd(q, k, v, q_pos, k_pos, cu_seqlens=cu_seqlens_q.to(torch.int32),
+                                      max_seqlen=max(int(max_seqlen_q), int(max_seqlen_k)), sm_scale=sm_scale,
+                                      position_buckets=position_buckets,
+                                      max_relative_positions=max_relative_distance, causal=causal)
+
+
+def quantize_e4m3_per_head(x):
+    """x: bf16 [..., H, D] on the GPU -> (float8_e4m3fn tensor of the same shape, float32 scales [H]);
+    scale[h] = max(absmax over everything but h, 1e-12) / 448, y = e4m3_rne(x / scale[h])."""
+    if not x.is_cuda or x.dtype != torch.bfloat16:
+        raise ValueError("quantize_e4m3_per_head expects a bfloat16 GPU tensor")
+    H, D = x.shape[-2], x.shape[-1]
+    x3 = x.reshape(-1, H, D)
+    if x3.stride(2) != 1:
+        x3 = x3.contiguous()
+    y = torch.empty(x3.shape, dtype=torch.uint8, device=x.device)
+    scale = torch.empty(H, dtype=torch.float32, device=x.device)
+    ws = torch.empty(H, dtype=torch.int32, device=x.device)
+    with torch.cuda.device(x.device):
+        check(lib.fdb_quant_e4m3_per_head(_ptr(x3), x3.stride(0), x3.stride(1), _ptr(y), y.stride(0), y.stride(1),
+                                          _ptr(scale), _ptr(ws), x3.shape[0], H, D, _stream_ptr(x.device)),
+              "fdb_quant_e4m3_per_head")
+    return y.view(_FP8).reshape(x.shape), scale

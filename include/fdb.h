@@ -1,0 +1,155 @@
+/*
+ * fdb.h -- C ABI of the MI355X (gfx950) disentangled-attention forward library.
+ *
+ * The library is a plain shared object (libfdb_hip.so): C linkage, raw device pointers,
+ * integer sizes and strides, no C++ or torch types in any signature.  It never allocates or
+ * frees device memory and keeps no pointer after a call returns; every buffer, including the
+ * output, the optional log-sum-exp, the varlen work-list and the delta look-up table, is
+ * owned by the caller.  All launches are asynchronous on the stream passed in.
+ *
+ * Reference interfaces replaced (paths relative to the FlashDeBERTa repository):
+ *   fdb_attn_fwd           <- flash_attention_with_disentangled
+ *                             (src/flashdeberta/ops/flash_attention.py:1088-1091, kernel :146-300,
+ *                             launcher :421-488) and flash_attention_with_disentangled_varlen
+ *                             (src/flashdeberta/ops/flash_attention_varlen.py:485-511, kernel :85-225,
+ *                             launcher :349-440), plus the two bias GEMMs the module runs before
+ *                             them (src/flashdeberta/model.py:189-192 and :210-214), which are
+ *                             fused here: the entry point takes the projected relative embeddings
+ *                             K_r / Q_r [H, 2S, D] rather than their [B,H,L,2S] products.
+ *   fdb_build_worklist     <- get_mid (src/flashdeberta/ops/flash_attention_varlen.py:71-83), the
+ *                             per-q-tile (sequence, first row) list; built on the device.
+ *   fdb_delta_lut          <- the log-bucket arithmetic evaluated per score element in the kernels
+ *                             (flash_attention.py:236-254, flash_attention_varlen.py:174-186), i.e.
+ *                             make_log_bucket_position of transformers' modeling_deberta_v2.py:56-69
+ *                             followed by clamp(. + S, 0, 2S-1) (:318, :336); host-side, integers out.
+ *   fdb_quant_e4m3_per_head   no reference counterpart (FP8 Q/K variant).
+ */
+#ifndef FDB_H_
+#define FDB_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FDB_VERSION 1
+
+/* element types of q/k/pos_key/pos_query (v and out: see fdb_attn_args.dtype) */
+enum fdb_dtype {
+  FDB_F32 = 0,      /* everything fp32, fp32 MFMA                                   */
+  FDB_BF16 = 1,     /* everything bf16, fp32 accumulate                             */
+  FDB_F16 = 2,      /* everything fp16, fp32 accumulate                             */
+  FDB_FP8_E4M3 = 3  /* q,k,pos_key,pos_query OCP e4m3 + per-head scales; v,out bf16 */
+};
+
+/* return codes: 0 ok, negative = invalid argument, positive = hipError_t of the launch */
+enum fdb_status {
+  FDB_OK = 0,
+  FDB_ERR_NULL = -1,        /* required pointer is NULL                                   */
+  FDB_ERR_DTYPE = -2,       /* dtype not one of fdb_dtype                                  */
+  FDB_ERR_HEAD_DIM = -3,    /* head_dim not supported (supported: 32, 64, 128)             */
+  FDB_ERR_ALIGN = -4,       /* pointer or stride not 16-byte aligned                       */
+  FDB_ERR_SHAPE = -5,       /* batch/heads/seqlen/total_tokens not positive or inconsistent */
+  FDB_ERR_SPAN = -6,        /* att_span <= 0 or lut_radius < 1 with a position term present */
+  FDB_ERR_SCALE = -7,       /* fp8 dtype without the needed scale vectors                  */
+  FDB_ERR_WORKLIST = -8,    /* cu_seqlens given without a work-list buffer                 */
+  FDB_ERR_LUT_ARGS = -9,    /* fdb_delta_lut: bad bucket/max_position/radius/out           */
+  FDB_ERR_UNSUPPORTED = -10 /* combination not built                                       */
+};
+
+/*
+ * One forward call.  Logical tensors (S = att_span):
+ *   q, k, v, out : element (b, l, h, d) at  base + b*stride_b + (tok0_b + l)*stride_t + h*stride_h + d
+ *                  fixed length (cu_seqlens == NULL): tok0_b = 0, 0 <= l < max_seqlen
+ *                  packed varlen (cu_seqlens != NULL): tok0_b = cu_seqlens[b], stride_b ignored,
+ *                                                      0 <= l < cu_seqlens[b+1]-cu_seqlens[b]
+ *   pos_key  (K_r): element (h, r, d) at base + h*pk_stride_h + r*pk_stride_r + d, 0 <= r < 2S
+ *   pos_query(Q_r): likewise with pq_stride_*
+ *   score(i,j) = sm_scale * ( q_i.k_j + q_i.K_r[delta(i-j)] + k_j.Q_r[delta(i-j)] ),
+ *   delta(r) = delta_lut[clamp(r, -lut_radius, lut_radius) + lut_radius]; a NULL pos pointer
+ *   drops that term.  out_i = sum_j softmax_j(score(i,.)) v_j ; lse_i = log sum_j exp(score(i,j)).
+ * Strides are in elements.  The last dimension has unit stride.
+ */
+typedef struct fdb_attn_args {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* pos_key;     /* K_r or NULL (no content->position term)  */
+  const void* pos_query;   /* Q_r or NULL (no position->content term)  */
+  void* out;
+  float* lse;              /* [B*max_seqlen*H] (fixed) / [T*H] (varlen), token-major, or NULL */
+  const int32_t* cu_seqlens; /* device int32[batch+1] or NULL                                 */
+  int32_t* worklist;       /* device int32[fdb_worklist_ints(...)], filled by fdb_build_worklist */
+  const int16_t* delta_lut;  /* device int16[2*lut_radius+1] from fdb_delta_lut, or NULL if no pos term */
+  const float* q_scale;    /* fp8 only: device float[heads] dequant scales               */
+  const float* k_scale;
+  const float* pk_scale;
+  const float* pq_scale;
+  int64_t q_stride_b, q_stride_t, q_stride_h;
+  int64_t k_stride_b, k_stride_t, k_stride_h;
+  int64_t v_stride_b, v_stride_t, v_stride_h;
+  int64_t o_stride_b, o_stride_t, o_stride_h;
+  int64_t pk_stride_h, pk_stride_r;
+  int64_t pq_stride_h, pq_stride_r;
+  int32_t batch;
+  int32_t heads;
+  int32_t head_dim;
+  int32_t max_seqlen;      /* fixed: the sequence length; varlen: upper bound on any length */
+  int32_t total_tokens;    /* varlen: cu_seqlens[batch]; fixed: batch*max_seqlen            */
+  int32_t att_span;        /* S: position_buckets if > 0 else max_relative_positions        */
+  int32_t lut_radius;
+  int32_t dtype;           /* enum fdb_dtype                                                 */
+  int32_t causal;          /* nonzero: key j visible to query i only if j <= i               */
+  float sm_scale;
+} fdb_attn_args;
+
+int fdb_version(void);
+const char* fdb_strerror(int code);
+
+/* Host-only validation of an argument block (what fdb_attn_fwd checks before launching). */
+int fdb_attn_check(const fdb_attn_args* a);
+
+/* Enqueue the fused forward on `stream` (a hipStream_t). */
+int fdb_attn_fwd(const fdb_attn_args* a, void* stream);
+
+/* Number of int32 the varlen work-list needs for (total_tokens, batch): 2 ints per possible
+ * q-tile plus a header.  Depends on shapes only, so no device sync is needed to size it. */
+int64_t fdb_worklist_ints(int32_t total_tokens, int32_t batch);
+
+/* Upper bound on q-tiles for (total_tokens, batch); the grid of the varlen launch. */
+int32_t fdb_worklist_max_tiles(int32_t total_tokens, int32_t batch);
+
+/* Rows of one q-tile (the work-list granularity). */
+int32_t fdb_tile_rows(void);
+
+/* Enqueue the device-side work-list construction from cu_seqlens. */
+int fdb_build_worklist(const int32_t* cu_seqlens, int32_t batch, int32_t total_tokens,
+                       int32_t* worklist, void* stream);
+
+/*
+ * Host: fill out[0 .. 2*radius] with delta(r) for r = -radius .. radius, where
+ *   position_buckets > 0 : delta = clamp(log_bucket(r; position_buckets, max_position) + S, 0, 2S-1), S = position_buckets
+ *   otherwise            : delta = clamp(r + S, 0, 2S-1), S = max_position
+ * fdb_delta_lut_radius returns the smallest radius beyond which delta is constant on both sides.
+ */
+int32_t fdb_delta_lut_radius(int32_t position_buckets, int32_t max_position);
+int fdb_delta_lut(int32_t position_buckets, int32_t max_position, int32_t radius, int16_t* out);
+
+/*
+ * Per-head absmax quantisation to OCP e4m3: for each head h,
+ *   scale[h] = max(absmax over all tokens and d of x[:, h, :], tiny) / 448,
+ *   y = e4m3_rne(x / scale[h]).
+ * x: bf16 element (t, h, d) at x + t*x_stride_t + h*x_stride_h + d, t < tokens; y: same indexing
+ * with y strides, one byte per element.  absmax_ws: device uint32[heads] scratch owned by the caller.
+ */
+int fdb_quant_e4m3_per_head(const void* x, int64_t x_stride_t, int64_t x_stride_h,
+                            void* y, int64_t y_stride_t, int64_t y_stride_h,
+                            float* scale, uint32_t* absmax_ws,
+                            int32_t tokens, int32_t heads, int32_t head_dim, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FDB_H_ */
