@@ -17,7 +17,7 @@ FDB_F32, FDB_BF16, FDB_F16, FDB_FP8_E4M3 = 0, 1, 2, 3
 class FdbAttnArgs(ctypes.Structure):
     _fields_ = (
         [(n, ctypes.c_void_p) for n in (
-            "q", "k", "v", "pos_key", "pos_query", "out", "lse", "cu_seqlens", "worklist", "delta_lut",
+            "q", "k", "v", "pos_key", "pos_query", "out", "lse", "cu_seqlens", "worklist", "seq_start", "seq_len", "delta_lut",
             "q_scale", "k_scale", "pk_scale", "pq_scale")]
         + [(n, ctypes.c_int64) for n in (
             "q_stride_b", "q_stride_t", "q_stride_h", "k_stride_b", "k_stride_t", "k_stride_h",
@@ -30,7 +30,7 @@ class FdbAttnArgs(ctypes.Structure):
 
 
 EXPORTS = (
-    "fdb_version", "fdb_strerror", "fdb_attn_check", "fdb_attn_fwd", "fdb_worklist_ints",
+    "fdb_version", "fdb_attn_args_size", "fdb_strerror", "fdb_attn_check", "fdb_attn_fwd", "fdb_worklist_ints",
     "fdb_worklist_max_tiles", "fdb_tile_rows", "fdb_build_worklist", "fdb_delta_lut_radius", "fdb_delta_lut",
     "fdb_quant_e4m3_per_head",
 )
@@ -44,6 +44,10 @@ def _load():
     lib = ctypes.CDLL(LIB_PATH)
     vp, i32, i64 = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64
     lib.fdb_version.restype = ctypes.c_int
+    lib.fdb_attn_args_size.restype = ctypes.c_size_t
+    if lib.fdb_attn_args_size() != ctypes.sizeof(FdbAttnArgs):
+        raise ImportError("flashdeberta_amd: %s was built from a different include/fdb.h (struct size %d, binding %d); rebuild it"
+                          % (LIB_PATH, lib.fdb_attn_args_size(), ctypes.sizeof(FdbAttnArgs)))
     lib.fdb_strerror.restype = ctypes.c_char_p
     lib.fdb_strerror.argtypes = [ctypes.c_int]
     lib.fdb_attn_check.restype = ctypes.c_int

@@ -73,6 +73,8 @@ extern "C" {
 
 int fdb_version(void) { return FDB_VERSION; }
 
+size_t fdb_attn_args_size(void) { return sizeof(fdb_attn_args); }
+
 const char* fdb_strerror(int code) {
   switch (code) {
     case FDB_OK: return "ok";
@@ -153,6 +155,8 @@ int fdb_attn_fwd(const fdb_attn_args* a, void* stream) {
   p.cu = a->cu_seqlens;
   p.wl = a->worklist;
   p.lut = a->delta_lut;
+  p.seq_start = a->cu_seqlens ? nullptr : a->seq_start;
+  p.seq_len = a->cu_seqlens ? nullptr : a->seq_len;
   p.qs = a->q_scale; p.ks = a->k_scale; p.pks = a->pk_scale; p.pqs = a->pq_scale;
   p.q_sb = a->q_stride_b; p.q_st = a->q_stride_t; p.q_sh = a->q_stride_h;
   p.k_sb = a->k_stride_b; p.k_st = a->k_stride_t; p.k_sh = a->k_stride_h;

@@ -204,8 +204,9 @@ __global__ __launch_bounds__(kThreads, 1) void fdb_attn_kernel(const FdbKParams 
   } else {
     b = blockIdx.x / p.tiles_per_seq;
     m0 = (blockIdx.x % p.tiles_per_seq) * FDB_BM;
-    tok0 = 0;
-    Lb = p.L;
+    tok0 = p.seq_start ? min(max(p.seq_start[b], 0), p.L) : 0;
+    Lb = p.seq_len ? min(max(p.seq_len[b], 0), p.L - tok0) : p.L;
+    if (m0 >= Lb) return;
     qo = b * p.q_sb; ko = b * p.k_sb; vo = b * p.v_sb; oo = b * p.o_sb;
   }
   const char* qb = p.q + (qo + (int64_t)tok0 * p.q_st + (int64_t)h * p.q_sh) * QT::SZ;
@@ -388,7 +389,7 @@ __global__ __launch_bounds__(kThreads, 1) void fdb_attn_kernel(const FdbKParams 
                    o_acc[d][4 * q4 + 2] * inv, o_acc[d][4 * q4 + 3] * inv);
       }
     if (p.lse && g == 0) {
-      const int64_t tok = p.cu ? (int64_t)tok0 + i : (int64_t)b * p.L + i;
+      const int64_t tok = p.cu ? (int64_t)tok0 + i : (int64_t)b * p.L + tok0 + i;
       p.lse[tok * p.H + h] = (m_run + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
     }
   }

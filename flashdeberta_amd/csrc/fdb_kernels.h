@@ -17,6 +17,8 @@ struct FdbKParams {
   float* lse;
   const int32_t* cu;   // cu_seqlens or NULL
   const int32_t* wl;   // work-list (varlen only)
+  const int32_t* seq_start;  // padded fixed layout: first real token / number of real tokens per row (or NULL)
+  const int32_t* seq_len;
   const int16_t* lut;  // delta LUT, index r + R
   const float* qs;     // fp8 dequant scales per head (NULL otherwise)
   const float* ks;

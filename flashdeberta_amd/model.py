@@ -1,0 +1,171 @@
+"""Drop-in attention module and the `_attn_implementation` switch.
+
+Counterparts in the reference (src/flashdeberta/model.py):
+  FlashDisentangledSelfAttention   :97-252   same constructor, parameters and forward signature
+  DEBERTA_SELF_ATTENTION_CLASSES   :254-257  {"eager", "flash_attention_2"}
+  FlashDebertaV2Model              :394-496  here a thin subclass of transformers' DebertaV2Model
+The eager entry is transformers' own DisentangledSelfAttention, exactly as in the reference.
+Forward / inference only (the reference's varlen path has no backward either,
+src/flashdeberta/ops/flash_attention_varlen.py:480-483).
+"""
+import math
+
+import torch
+from torch import nn
+from transformers.models.deberta_v2.modeling_deberta_v2 import (
+    DebertaV2Config,
+    DebertaV2Model,
+    DisentangledSelfAttention,
+)
+
+from . import ops
+from .padding import key_padding_mask, seq_bounds
+
+
+class FlashDisentangledSelfAttention(DisentangledSelfAttention):
+    """Same parameters as the eager module (query_proj, key_proj, value_proj[, pos_key_proj,
+    pos_query_proj]), so `load_state_dict(eager.state_dict())` works (reference tests/attention.py:60).
+
+    fp8_qk=True quantises Q, K and the projected relative embeddings to OCP e4m3 with per-head
+    absmax scales before the kernel (bf16 inputs only)."""
+
+    def __init__(self, config, fp8_qk=None):
+        super().__init__(config)
+        self.fp8_qk = bool(getattr(config, "fp8_qk", False)) if fp8_qk is None else bool(fp8_qk)
+
+    def _pos_layers(self, rel_embeddings):
+        """K_r, Q_r as [H, 2S, D] views of the projected relative embeddings
+        (reference model.py:159-177; the slice to 2S rows is transformers modeling_deberta_v2.py:295)."""
+        if not self.relative_attention or rel_embeddings is None:
+            return None, None
+        H, D = self.num_attention_heads, self.attention_head_size
+        span = self.pos_ebd_size
+        rel = self.pos_dropout(rel_embeddings)[0:2 * span]
+
+        def heads(x):  # [2S, H*D] -> [H, 2S, D] without a copy
+            return x.view(x.shape[0], H, D).transpose(0, 1)
+
+        pos_key = pos_query = None
+        if self.share_att_key:
+            if "c2p" in self.pos_att_type:
+                pos_key = heads(self.key_proj(rel))
+            if "p2c" in self.pos_att_type:
+                pos_query = heads(self.query_proj(rel))
+        else:
+            if "c2p" in self.pos_att_type:
+                pos_key = heads(self.pos_key_proj(rel))
+            if "p2c" in self.pos_att_type:
+                pos_query = heads(self.pos_query_proj(rel))
+        return pos_key, pos_query
+
+    def forward(self, hidden_states, attention_mask, output_attentions=False, query_states=None,
+                relative_pos=None, rel_embeddings=None):
+        """-> (context [B, L, H*D], None).  `relative_pos` is ignored: the bucketed relative
+        position is an integer table inside the kernel.  Attention probabilities are never
+        materialised, so `output_attentions` yields None like the reference (model.py:252)."""
+        if self.training and torch.is_grad_enabled() and hidden_states.requires_grad:
+            raise RuntimeError("FlashDisentangledSelfAttention is forward-only; use the eager implementation to train")
+        if query_states is None:
+            query_states = hidden_states
+        B, L, _ = hidden_states.shape
+        H, D = self.num_attention_heads, self.attention_head_size
+
+        q = self.query_proj(query_states).view(B, L, H, D)
+        k = self.key_proj(hidden_states).view(B, L, H, D)
+        v = self.value_proj(hidden_states).view(B, L, H, D)
+        pos_key, pos_query = self._pos_layers(rel_embeddings)
+
+        scale_factor = 1 + ("c2p" in self.pos_att_type and pos_key is not None) + \
+            ("p2c" in self.pos_att_type and pos_query is not None)
+        if not self.relative_attention:
+            scale_factor = 1 + ("c2p" in self.pos_att_type) + ("p2c" in self.pos_att_type)  # model.py:151-157
+        sm_scale = 1.0 / math.sqrt(D * scale_factor)
+
+        seq_start = seq_len = None
+        out = None
+        if attention_mask is not None:
+            seq_start, seq_len = seq_bounds(key_padding_mask(attention_mask))
+            out = torch.zeros((B, L, H, D), dtype=v.dtype, device=v.device)  # padded rows stay zero
+
+        kw = {}
+        if self.fp8_qk:
+            if q.dtype != torch.bfloat16:
+                raise ValueError("fp8_qk needs bfloat16 activations")
+            q, kw["q_scale"] = ops.quantize_e4m3_per_head(q)
+            k, kw["k_scale"] = ops.quantize_e4m3_per_head(k)
+            if pos_key is not None:
+                pos_key, kw["pos_key_scale"] = ops.quantize_e4m3_per_head(pos_key.transpose(0, 1))
+                pos_key = pos_key.transpose(0, 1)
+            if pos_query is not None:
+                pos_query, kw["pos_query_scale"] = ops.quantize_e4m3_per_head(pos_query.transpose(0, 1))
+                pos_query = pos_query.transpose(0, 1)
+
+        ctx = ops.disentangled_attention_fwd(
+            q, k, v, pos_key, pos_query, sm_scale=sm_scale,
+            position_buckets=self.position_buckets if self.relative_attention else 0,
+            max_relative_positions=self.max_relative_positions if self.relative_attention else 0,
+            seq_start=seq_start, seq_len=seq_len, out=out, **kw)
+        return (ctx.view(B, L, H * D), None)
+
+
+DEBERTA_SELF_ATTENTION_CLASSES = {
+    "eager": DisentangledSelfAttention,
+    "flash_attention_2": FlashDisentangledSelfAttention,
+}
+
+
+def patch_model(model, attn_implementation="flash_attention_2", fp8_qk=False, skip_dense_position_tensors=True):
+    """Swap every `layer.attention.self` of a transformers DebertaV2 model (bare or with a head)
+    for the class the key selects, keeping the weights.  With skip_dense_position_tensors the
+    encoder also stops building the [1, L, L] int64 relative-position tensor and the [B, 1, L, L]
+    mask (transformers modeling_deberta_v2.py:601-626), which the fused path never reads."""
+    cls = DEBERTA_SELF_ATTENTION_CLASSES[attn_implementation]
+    encoder = None
+    for mod in model.modules():
+        if mod.__class__.__name__ == "DebertaV2Encoder" or hasattr(mod, "rel_embeddings") and hasattr(mod, "layer"):
+            encoder = mod
+            break
+    if encoder is None:
+        raise ValueError("no DebertaV2 encoder found in %s" % type(model).__name__)
+    config = model.config
+    for layer in encoder.layer:
+        old = layer.attention.self
+        if type(old) is cls:
+            continue
+        new = cls(config, fp8_qk=fp8_qk) if cls is FlashDisentangledSelfAttention else cls(config)
+        new.load_state_dict(old.state_dict())
+        p = next(old.parameters())
+        new.to(device=p.device, dtype=p.dtype)
+        new.train(old.training)
+        layer.attention.self = new
+    flash = cls is FlashDisentangledSelfAttention
+    if flash and skip_dense_position_tensors:
+        encoder.get_rel_pos = lambda hidden_states, query_states=None, relative_pos=None: relative_pos
+        encoder.get_attention_mask = lambda attention_mask: attention_mask
+    else:
+        encoder.__dict__.pop("get_rel_pos", None)
+        encoder.__dict__.pop("get_attention_mask", None)
+    return model
+
+
+class FlashDebertaV2Model(DebertaV2Model):
+    """DebertaV2Model whose attention follows `config._attn_implementation` in
+    {"eager", "flash_attention_2"}; unset means "flash_attention_2", the reference's default
+    (model.py:61-62).  transformers' own check would treat "flash_attention_2" as a request for
+    the flash-attn package, so the two keys are resolved here instead."""
+
+    def _check_and_adjust_attn_implementation(self, attn_implementation, is_init_check=False, **kwargs):
+        if attn_implementation is None:
+            return "flash_attention_2"
+        if attn_implementation in DEBERTA_SELF_ATTENTION_CLASSES:
+            return attn_implementation
+        raise ValueError("attn_implementation must be one of %s, got %r"
+                         % (sorted(DEBERTA_SELF_ATTENTION_CLASSES), attn_implementation))
+
+    def __init__(self, config):
+        super().__init__(config)
+        patch_model(self, self.config._attn_implementation, fp8_qk=bool(getattr(config, "fp8_qk", False)))
+
+
+__all__ = ["FlashDisentangledSelfAttention", "DEBERTA_SELF_ATTENTION_CLASSES", "FlashDebertaV2Model",
+           "DebertaV2Config", "patch_model"]

@@ -79,13 +79,16 @@ def _pos_arg(x, H, D, span, name):
 
 def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seqlens=None, max_seqlen=None,
                                sm_scale=None, position_buckets=0, max_relative_positions=0, causal=False,
-                               return_lse=False, q_scale=None, k_scale=None, pos_key_scale=None,
+                               return_lse=False, seq_start=None, seq_len=None, q_scale=None, k_scale=None, pos_key_scale=None,
                                pos_query_scale=None, out=None):
     """Fused forward.  Layouts (strides are free except a unit stride on D):
          fixed length : q, k, v  [B, L, H, D]   -> out [B, L, H, D] (contiguous: a free view of [B, L, H*D])
          packed varlen: q, k, v  [T, H, D] + cu_seqlens int32 [B+1] (+ max_seqlen upper bound) -> out [T, H, D]
        pos_key = K_r, pos_query = Q_r: [H, 2S, D] or None (term absent).  sm_scale defaults to
        1/sqrt(D * (1 + #position terms)) as the reference module computes it (src/flashdeberta/model.py:151-157).
+       padded batches (fixed layout only): seq_start / seq_len int32 [B] GPU tensors give each row's real
+       tokens [seq_start, seq_start+seq_len); only those rows of `out` are written, so pass a zeroed `out`
+       (or ignore the padded rows).  Either may be None (0 / L).
        fp8: q/k/pos_* are torch.float8_e4m3fn with float32 per-head scales; v is bfloat16.
     """
     if not q.is_cuda:
@@ -154,6 +157,13 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
             setattr(a, n + "_stride_b", x.stride(0))
             setattr(a, n + "_stride_t", x.stride(1))
             setattr(a, n + "_stride_h", x.stride(2))
+        for n, x in (("seq_start", seq_start), ("seq_len", seq_len)):
+            if x is not None:
+                if x.dtype != torch.int32 or not x.is_cuda or x.numel() != B:
+                    raise ValueError("%s must be an int32 GPU tensor with one entry per batch row" % n)
+                x = x.contiguous()
+                keep.append(x)
+                setattr(a, n, x.data_ptr())
     if pos_key is not None:
         a.pk_stride_h, a.pk_stride_r = pos_key.stride(0), pos_key.stride(1)
     if pos_query is not None:

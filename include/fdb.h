@@ -62,7 +62,11 @@ enum fdb_status {
 /*
  * One forward call.  Logical tensors (S = att_span):
  *   q, k, v, out : element (b, l, h, d) at  base + b*stride_b + (tok0_b + l)*stride_t + h*stride_h + d
- *                  fixed length (cu_seqlens == NULL): tok0_b = 0, 0 <= l < max_seqlen
+ *                  fixed length (cu_seqlens == NULL): tok0_b = 0, 0 <= l < max_seqlen; with seq_start /
+ *                                                      seq_len (padded batches) the real tokens of row b are
+ *                                                      l in [seq_start[b], seq_start[b]+seq_len[b]), they
+ *                                                      attend only to each other with positions counted
+ *                                                      from seq_start[b]; other rows of `out` are not written
  *                  packed varlen (cu_seqlens != NULL): tok0_b = cu_seqlens[b], stride_b ignored,
  *                                                      0 <= l < cu_seqlens[b+1]-cu_seqlens[b]
  *   pos_key  (K_r): element (h, r, d) at base + h*pk_stride_h + r*pk_stride_r + d, 0 <= r < 2S
@@ -82,6 +86,8 @@ typedef struct fdb_attn_args {
   float* lse;              /* [B*max_seqlen*H] (fixed) / [T*H] (varlen), token-major, or NULL */
   const int32_t* cu_seqlens; /* device int32[batch+1] or NULL                                 */
   int32_t* worklist;       /* device int32[fdb_worklist_ints(...)], filled by fdb_build_worklist */
+  const int32_t* seq_start; /* fixed layout only, device int32[batch] or NULL: first real token of each row */
+  const int32_t* seq_len;   /* fixed layout only, device int32[batch] or NULL: number of real tokens        */
   const int16_t* delta_lut;  /* device int16[2*lut_radius+1] from fdb_delta_lut, or NULL if no pos term */
   const float* q_scale;    /* fp8 only: device float[heads] dequant scales               */
   const float* k_scale;
@@ -106,6 +112,8 @@ typedef struct fdb_attn_args {
 } fdb_attn_args;
 
 int fdb_version(void);
+/* sizeof(fdb_attn_args) as the library was built: lets a foreign-language binding check its struct mirror. */
+size_t fdb_attn_args_size(void);
 const char* fdb_strerror(int code);
 
 /* Host-only validation of an argument block (what fdb_attn_fwd checks before launching). */

@@ -1,0 +1,189 @@
+"""CPU tests of the C-ABI library: it loads, exports every symbol include/fdb.h declares, its
+host-side logic (delta table, work-list sizing, argument validation, error strings) behaves, and
+the python mirror of the reference interface is wired.  No kernel is launched here."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from flashdeberta_amd import _lib, ops
+from flashdeberta_amd._lib import FdbAttnArgs, lib
+from oracle import disentangled_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "fdb.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    body = text[text.index("} fdb_attn_args;"):]
+    return sorted(set(re.findall(r"\b(fdb_[a-z0-9_]+)\s*\(", body)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared_functions()
+    assert len(names) >= 10
+    for n in names:
+        assert hasattr(lib, n), "libfdb_hip.so does not export %s" % n
+    assert sorted(_lib.EXPORTS) == names
+
+
+def test_struct_mirror_and_version():
+    assert lib.fdb_attn_args_size() == ctypes.sizeof(FdbAttnArgs)
+    assert lib.fdb_version() == 1
+    assert lib.fdb_tile_rows() == 128
+
+
+@pytest.mark.parametrize("pb,mr", [(256, 512), (32, 64), (64, 512), (16, 40), (0, 512), (0, 24), (128, 256)])
+def test_delta_lut_bit_exact_vs_oracle(pb, mr):
+    lut, R = ops.delta_lut_host(pb, mr)
+    ref = O.delta_table(pb, mr, R)
+    assert lut.dtype == np.int16 and len(lut) == 2 * R + 1
+    assert (lut.astype(np.int64) == ref).all()
+    # beyond the radius delta is constant: the table's ends are the clamp values on both sides
+    wide = O.delta_table(pb, mr, 4 * R + 100)
+    c = 3 * R + 100
+    assert (wide[:c] == lut[0]).all() and (wide[-c:] == lut[-1]).all()
+    span = pb if pb > 0 else mr
+    assert lut[0] == 0 and lut[-1] == 2 * span - 1
+    # tight: one step inside the radius at least one side has not reached its clamp value yet
+    assert lut[1] != lut[0] or lut[-2] != lut[-1]
+
+
+def test_delta_lut_rejects_degenerate_configs():
+    assert lib.fdb_delta_lut_radius(2, 512) == -9      # mid - 1 == 0
+    assert lib.fdb_delta_lut_radius(256, 100) == -9    # log((max-1)/mid) <= 0
+    assert lib.fdb_delta_lut_radius(0, 0) == -9
+    buf = np.zeros(8, dtype=np.int16)
+    assert lib.fdb_delta_lut(256, 512, 0, buf.ctypes.data_as(ctypes.c_void_p)) == -9
+    assert lib.fdb_delta_lut(256, 512, 3, None) == -9
+    with pytest.raises(ValueError):
+        ops.delta_lut_host(2, 512)
+
+
+def test_worklist_sizing():
+    assert lib.fdb_worklist_max_tiles(1000, 4) == 1000 // 128 + 4
+    assert lib.fdb_worklist_ints(1000, 4) == 2 + 2 * (1000 // 128 + 4)
+    rng = np.random.default_rng(0)
+    for _ in range(50):
+        lens = rng.integers(0, 700, size=rng.integers(1, 40))
+        tiles = int(sum((l + 127) // 128 for l in lens))
+        assert tiles <= lib.fdb_worklist_max_tiles(int(lens.sum()), len(lens))
+
+
+def _good_args():
+    a = FdbAttnArgs()
+    a.q = a.k = a.v = a.out = 0x1000
+    a.pos_key = a.pos_query = 0x2000
+    a.delta_lut = 0x3000
+    for n in ("q", "k", "v", "o"):
+        setattr(a, n + "_stride_b", 512 * 768)
+        setattr(a, n + "_stride_t", 768)
+        setattr(a, n + "_stride_h", 64)
+    a.pk_stride_h = a.pq_stride_h = 64
+    a.pk_stride_r = a.pq_stride_r = 768
+    a.batch, a.heads, a.head_dim, a.max_seqlen, a.total_tokens = 2, 12, 64, 512, 1024
+    a.att_span, a.lut_radius, a.dtype, a.sm_scale = 256, 512, _lib.FDB_BF16, 0.0721
+    return a
+
+
+def test_argument_validation_codes():
+    chk = lambda a: lib.fdb_attn_check(ctypes.byref(a))
+    assert chk(_good_args()) == 0
+    a = _good_args(); a.q = None; assert chk(a) == -1
+    a = _good_args(); a.dtype = 9; assert chk(a) == -2
+    a = _good_args(); a.head_dim = 48; assert chk(a) == -3
+    a = _good_args(); a.k = 0x1008; assert chk(a) == -4
+    a = _good_args(); a.q_stride_t = 772; assert chk(a) == -4            # 772 * 2 bytes is not a multiple of 16
+    a = _good_args(); a.total_tokens = 1000; assert chk(a) == -5         # != batch * max_seqlen without cu_seqlens
+    a = _good_args(); a.heads = 0; assert chk(a) == -5
+    a = _good_args(); a.delta_lut = None; assert chk(a) == -6
+    a = _good_args(); a.att_span = 0; assert chk(a) == -6
+    a = _good_args(); a.dtype = _lib.FDB_FP8_E4M3; assert chk(a) == -7   # no scales
+    a = _good_args(); a.cu_seqlens = 0x4000; assert chk(a) == -8          # no work-list
+    a = _good_args(); a.dtype = _lib.FDB_F32; a.head_dim = 128; assert chk(a) == -10
+    a = _good_args(); a.pos_key = a.pos_query = None; a.delta_lut = None; a.att_span = 0; assert chk(a) == 0
+    assert lib.fdb_attn_check(None) == -1
+    # launching with bad arguments returns the same code without touching the GPU
+    a = _good_args(); a.head_dim = 48
+    assert lib.fdb_attn_fwd(ctypes.byref(a), None) == -3
+    assert lib.fdb_build_worklist(None, 1, 1, None, None) == -1
+    assert lib.fdb_quant_e4m3_per_head(None, 0, 0, None, 0, 0, None, None, 1, 1, 64, None) == -1
+
+
+def test_error_strings_and_python_mapping():
+    for code in range(-10, 1):
+        assert _lib.strerror(code) not in ("", "unknown error")
+    with pytest.raises(ValueError):
+        _lib.check(-3, "x")
+    with pytest.raises(RuntimeError):
+        _lib.check(1, "x")
+
+
+def test_ops_reject_cpu_tensors_and_bad_shapes():
+    q = torch.zeros(1, 8, 2, 64)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        ops.disentangled_attention_fwd(q, q, q)
+
+
+def test_module_is_state_dict_compatible_with_eager():
+    from transformers.models.deberta_v2.modeling_deberta_v2 import DisentangledSelfAttention
+
+    from flashdeberta_amd import DEBERTA_SELF_ATTENTION_CLASSES, FlashDisentangledSelfAttention
+
+    class Cfg:  # the plain config object of the reference's tests/attention.py:6-18
+        hidden_size, num_attention_heads = 128, 2
+        attention_probs_dropout_prob = hidden_dropout_prob = 0.1
+        pos_att_type = ["c2p", "p2c"]
+        relative_attention, position_buckets, max_relative_positions = True, 32, 64
+        max_position_embeddings, share_att_key = 512, False
+
+    eager = DisentangledSelfAttention(Cfg())
+    flash = FlashDisentangledSelfAttention(Cfg())
+    res = flash.load_state_dict(eager.state_dict())
+    assert not res.missing_keys and not res.unexpected_keys
+    assert DEBERTA_SELF_ATTENTION_CLASSES["eager"] is DisentangledSelfAttention
+    assert DEBERTA_SELF_ATTENTION_CLASSES["flash_attention_2"] is FlashDisentangledSelfAttention
+    pk, pq = flash._pos_layers(torch.randn(64, 128))
+    assert pk.shape == (2, 64, 64) and pq.shape == (2, 64, 64)
+
+
+def test_switch_builds_both_implementations():
+    from transformers.models.deberta_v2.modeling_deberta_v2 import DebertaV2Model, DisentangledSelfAttention
+
+    from flashdeberta_amd import DebertaV2Config, FlashDebertaV2Model, FlashDisentangledSelfAttention, patch_model
+
+    kw = dict(vocab_size=50, hidden_size=128, num_hidden_layers=2, num_attention_heads=2, intermediate_size=128,
+              relative_attention=True, pos_att_type="p2c|c2p", position_buckets=32, max_relative_positions=64,
+              share_att_key=True, norm_rel_ebd="layer_norm", position_biased_input=False)
+    m = FlashDebertaV2Model(DebertaV2Config(**kw))
+    assert all(type(l.attention.self) is FlashDisentangledSelfAttention for l in m.encoder.layer)
+    m = FlashDebertaV2Model(DebertaV2Config(attn_implementation="eager", **kw))
+    assert all(type(l.attention.self) is DisentangledSelfAttention for l in m.encoder.layer)
+    hf = DebertaV2Model(DebertaV2Config(**kw))
+    w = hf.encoder.layer[1].attention.self.query_proj.weight.clone()
+    patch_model(hf)
+    assert type(hf.encoder.layer[1].attention.self) is FlashDisentangledSelfAttention
+    assert torch.equal(hf.encoder.layer[1].attention.self.query_proj.weight, w)
+    patch_model(hf, "eager")
+    assert type(hf.encoder.layer[1].attention.self) is DisentangledSelfAttention
+    with pytest.raises(ValueError):
+        FlashDebertaV2Model(DebertaV2Config(attn_implementation="sdpa", **kw))
+
+
+def test_padding_helpers():
+    from flashdeberta_amd.padding import get_unpad_data, key_padding_mask, pad_input, seq_bounds, unpad_input
+
+    m = torch.tensor([[1, 1, 1, 0, 0], [0, 0, 1, 1, 1], [1, 1, 1, 1, 1]])
+    ext = m[:, None, None, :] * m[:, None, :, None]
+    assert torch.equal(key_padding_mask(ext), m.bool()) and torch.equal(key_padding_mask(m), m.bool())
+    s, n = seq_bounds(m.bool())
+    assert s.tolist() == [0, 2, 0] and n.tolist() == [3, 3, 5]
+    idx, cu, mx = get_unpad_data(m.bool())
+    ref_idx, ref_cu, ref_mx = O.unpad_data(m.numpy())
+    assert idx.tolist() == ref_idx.tolist() and cu.tolist() == ref_cu.tolist() and int(mx) == ref_mx
+    x = torch.arange(15.0).view(3, 5, 1)
+    assert torch.equal(pad_input(unpad_input(x, idx), idx, 3, 5), x * m[:, :, None])

@@ -1,0 +1,390 @@
+"""GPU parity tests: the HIP path, called through the C ABI, against the CPU oracle on the same
+seeded inputs, against the golden vectors, and -- at full size -- through properties that do not
+need the oracle.  Tolerances (max-abs against an fp32/fp64 reference) are the ones the task
+states: fp32 <= 1e-4, bf16 <= 2e-2, fp8 <= 6e-2; fp16 is held to 5e-3.  On unit-scale "stress"
+inputs the same bounds are applied to max|err| / max|ref|."""
+import glob
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from flashdeberta_amd import ops
+from oracle import disentangled_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+TOL = {torch.float32: 1e-4, torch.bfloat16: 2e-2, torch.float16: 5e-3}
+FP8_TOL = 6e-2
+
+
+def _inputs(B, L, H, D, pb, mr, dtype, seed, scale, c2p=True, p2c=True):
+    g = torch.Generator().manual_seed(seed)
+    S = ops.att_span(pb, mr)
+    q, k, v = [(torch.randn(B, L, H, D, generator=g) * scale).to(dtype) for _ in range(3)]
+    pk = (torch.randn(H, 2 * S, D, generator=g) * scale).to(dtype) if c2p else None
+    pq = (torch.randn(H, 2 * S, D, generator=g) * scale).to(dtype) if p2c else None
+    return q, k, v, pk, pq
+
+
+def _np(x):
+    return None if x is None else x.float().numpy().astype(np.float64)
+
+
+def _oracle_blhd(q, k, v, pk, pq, pb, mr, **kw):
+    t = lambda x: _np(x).transpose(0, 2, 1, 3)
+    r = O.disentangled_attention(t(q), t(k), t(v), _np(pk), _np(pq), pb, mr, **kw)
+    if isinstance(r, tuple):
+        return r[0].transpose(0, 2, 1, 3), r[1].transpose(0, 2, 1)
+    return r.transpose(0, 2, 1, 3)
+
+
+def _dev(x):
+    return None if x is None else x.cuda()
+
+
+def _check(out, ref, tol, what=""):
+    o = out.float().cpu().numpy()
+    assert not np.isnan(o).any(), what
+    err = np.abs(o - ref).max()
+    bound = tol * max(1.0, np.abs(ref).max())
+    assert err <= bound, "%s max-abs err %.3e > %.3e (ref max %.3e)" % (what, err, bound, np.abs(ref).max())
+    return err
+
+
+# ---- operator vs oracle ------------------------------------------------------------------------
+CASES = [
+    # B, L, H, D, buckets, max_rel, c2p, p2c
+    (1, 64, 1, 64, 32, 64, False, False),
+    (1, 64, 2, 64, 32, 64, True, False),
+    (1, 64, 2, 64, 32, 64, False, True),
+    (2, 200, 2, 64, 32, 64, True, True),      # ragged tail in both tile dimensions
+    (1, 129, 1, 64, 32, 64, True, True),      # one row past a q-tile
+    (3, 1, 2, 64, 32, 64, True, True),        # single token
+    (1, 700, 2, 64, 256, 512, True, True),    # v3 buckets: linear + log zone + both saturations
+    (1, 1300, 1, 64, 256, 512, True, True),
+    (2, 200, 2, 64, 0, 48, True, True),       # no bucketing, clamp at +-48
+    (2, 150, 3, 32, 32, 64, True, True),
+    (2, 150, 2, 128, 32, 64, True, True),
+    (1, 300, 2, 64, 64, 512, True, True),     # wide log zone (max_rel >> buckets)
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "B%dL%dH%dD%d_b%d_m%d_%d%d" % c)
+@pytest.mark.parametrize("scale", [0.02, 1.0], ids=["n002", "unit"])
+def test_operator_matches_oracle(case, dtype, scale):
+    B, L, H, D, pb, mr, c2p, p2c = case
+    if dtype == torch.float32 and D == 128:
+        pytest.skip("fp32 with head_dim 128 is not built (LDS budget)")
+    if scale == 0.02 and D != 64:
+        pytest.skip("small-scale inputs only at the model's head_dim")
+    q, k, v, pk, pq = _inputs(B, L, H, D, pb, mr, dtype, 1000 + L, scale, c2p, p2c)
+    ref, ref_lse = _oracle_blhd(q, k, v, pk, pq, pb, mr, return_lse=True)
+    out, lse = ops.disentangled_attention_fwd(_dev(q), _dev(k), _dev(v), _dev(pk), _dev(pq), position_buckets=pb,
+                                              max_relative_positions=mr, return_lse=True)
+    _check(out, ref, TOL[dtype], "out")
+    _check(lse.view(B, L, H), ref_lse, 4 * TOL[dtype], "lse")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_causal(dtype):
+    q, k, v, pk, pq = _inputs(2, 200, 2, 64, 32, 64, dtype, 7, 1.0)
+    ref = _oracle_blhd(q, k, v, pk, pq, 32, 64, causal=True)
+    out = ops.disentangled_attention_fwd(_dev(q), _dev(k), _dev(v), _dev(pk), _dev(pq), position_buckets=32,
+                                         max_relative_positions=64, causal=True)
+    _check(out, ref, TOL[dtype])
+
+
+def test_strided_inputs_and_reference_call_shape():
+    # [B, H, L, D] tensors as the reference op takes them (flash_attention.py:1088) and a fused qkv buffer
+    B, L, H, D = 2, 160, 2, 64
+    q, k, v, pk, pq = _inputs(B, L, H, D, 32, 64, torch.bfloat16, 11, 1.0)
+    ref = _oracle_blhd(q, k, v, pk, pq, 32, 64)
+    bh = lambda x: x.cuda().permute(0, 2, 1, 3).contiguous()
+    out = ops.flash_attention_with_disentangled(bh(q), bh(k), bh(v), _dev(pk), _dev(pq), False, 1 / np.sqrt(3 * D), 32, 64)
+    assert out.shape == (B, H, L, D)
+    _check(out.permute(0, 2, 1, 3), ref, TOL[torch.bfloat16])
+    qkv = torch.stack([q, k, v], dim=2).cuda()  # [B, L, 3, H, D]: token stride 3*H*D
+    out = ops.disentangled_attention_fwd(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], _dev(pk), _dev(pq),
+                                         position_buckets=32, max_relative_positions=64)
+    _check(out, ref, TOL[torch.bfloat16])
+
+
+# ---- delta indices are bit-exact inside the kernel ----------------------------------------------
+@pytest.mark.parametrize("pb,mr,L", [(256, 512, 1200), (32, 64, 300), (0, 40, 130)])
+@pytest.mark.parametrize("term", ["c2p", "p2c"])
+def test_delta_indices_bit_exact(pb, mr, L, term):
+    """Encode delta in the position term (score = c * delta / 32) and read the probabilities of a
+    64-key window through a one-hot V: delta(i, j) = 32 * (log P_ij + lse_i) / c exactly recovers
+    the index the kernel used for every (i, j)."""
+    D, S = 64, ops.att_span(pb, mr)
+    ramp = torch.zeros(1, 2 * S, D)
+    ramp[0, :, 0] = torch.arange(2 * S) / 32.0
+    e0 = torch.zeros(1, L, 1, D)
+    e0[..., 0] = 1.0
+    zero = torch.zeros(1, L, 1, D)
+    q, k = (e0, zero) if term == "c2p" else (zero, e0)
+    pk, pq = (ramp, None) if term == "c2p" else (None, ramp)
+    c = 1.0 / np.sqrt(2 * D)
+    want = O.delta_table(pb, mr, L)  # index r + L
+    got = np.empty((L, L), dtype=np.int64)
+    for j0 in range(0, L, D):
+        v = torch.zeros(1, L, 1, D)
+        n = min(D, L - j0)
+        v[0, j0:j0 + n, 0, :n] = torch.eye(n)
+        out, lse = ops.disentangled_attention_fwd(q.cuda(), k.cuda(), v.cuda(), _dev(pk), _dev(pq), position_buckets=pb,
+                                                  max_relative_positions=mr, return_lse=True)
+        p = out[0, :, 0, :n].double().cpu().numpy()
+        sc = np.log(p) + lse[:, 0].double().cpu().numpy()[:, None]
+        got[:, j0:j0 + n] = np.rint(sc * 32.0 / c).astype(np.int64)
+    i, j = np.meshgrid(np.arange(L), np.arange(L), indexing="ij")
+    assert (got == want[i - j + L]).all()
+
+
+# ---- packed varlen and padded batches ------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_varlen_matches_per_sequence_oracle(dtype):
+    lens = [5, 128, 1, 129, 300, 64, 257]
+    H, D, pb, mr = 2, 64, 32, 64
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    T = int(cu[-1])
+    g = torch.Generator().manual_seed(5)
+    q, k, v = [torch.randn(T, H, D, generator=g).to(dtype) for _ in range(3)]
+    pk, pq = [torch.randn(H, 2 * pb, D, generator=g).to(dtype) for _ in range(2)]
+    ref = O.disentangled_attention_varlen(_np(q), _np(k), _np(v), cu, _np(pk), _np(pq), pb, mr)
+    cu_t = torch.from_numpy(cu).cuda()
+    out = ops.disentangled_attention_fwd(q.cuda(), k.cuda(), v.cuda(), pk.cuda(), pq.cuda(), cu_seqlens=cu_t,
+                                         max_seqlen=max(lens), position_buckets=pb, max_relative_positions=mr)
+    _check(out, ref, TOL[dtype])
+    # reference call shape of the varlen op; order of the two position tensors as in the reference
+    out2 = ops.flash_attention_with_disentangled_varlen(q.cuda(), k.cuda(), v.cuda(), pk.cuda(), pq.cuda(), cu_t, cu_t,
+                                                        max(lens), max(lens), False, 1 / np.sqrt(3 * D), pb, mr)
+    assert torch.equal(out, out2)
+    # order independence: reversing the sequences permutes the result
+    order = list(range(len(lens)))[::-1]
+    perm = np.concatenate([np.arange(cu[b], cu[b + 1]) for b in order])
+    cu_r = torch.from_numpy(np.concatenate([[0], np.cumsum([lens[b] for b in order])]).astype(np.int32)).cuda()
+    out3 = ops.disentangled_attention_fwd(q[perm].cuda(), k[perm].cuda(), v[perm].cuda(), pk.cuda(), pq.cuda(),
+                                          cu_seqlens=cu_r, max_seqlen=max(lens), position_buckets=pb,
+                                          max_relative_positions=mr)
+    assert torch.equal(out3, out[torch.from_numpy(perm).cuda()])
+
+
+def test_worklist_on_device():
+    from flashdeberta_amd._lib import lib
+    import ctypes
+    rng = np.random.default_rng(3)
+    for B in (1, 7, 300, 1000):
+        lens = rng.integers(0, 600, size=B)
+        cu = torch.from_numpy(np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)).cuda()
+        T = int(lens.sum())
+        wl = torch.full((int(lib.fdb_worklist_ints(T, B)),), -7, dtype=torch.int32, device="cuda")
+        rc = lib.fdb_build_worklist(ctypes.c_void_p(cu.data_ptr()), B, T, ctypes.c_void_p(wl.data_ptr()),
+                                    ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0
+        w = wl.cpu().numpy()
+        want = [(b, m0) for b in range(B) for m0 in range(0, int(lens[b]), 128)]
+        assert w[0] == len(want)
+        assert w[2:2 + 2 * len(want)].reshape(-1, 2).tolist() == [list(x) for x in want]
+
+
+@pytest.mark.parametrize("side", ["right", "left"])
+def test_padded_batch_matches_packed(side):
+    B, L, H, D, pb, mr = 3, 200, 2, 64, 32, 64
+    lens = [200, 77, 130]
+    q, k, v, pk, pq = _inputs(B, L, H, D, pb, mr, torch.bfloat16, 21, 1.0)
+    start = [0, 0, 0] if side == "right" else [L - n for n in lens]
+    out = torch.zeros(B, L, H, D, dtype=torch.bfloat16, device="cuda")
+    ops.disentangled_attention_fwd(q.cuda(), k.cuda(), v.cuda(), pk.cuda(), pq.cuda(), position_buckets=pb,
+                                   max_relative_positions=mr, out=out,
+                                   seq_start=torch.tensor(start, dtype=torch.int32, device="cuda"),
+                                   seq_len=torch.tensor(lens, dtype=torch.int32, device="cuda"))
+    for b in range(B):
+        sl = slice(start[b], start[b] + lens[b])
+        ref = _oracle_blhd(q[b:b + 1, sl], k[b:b + 1, sl], v[b:b + 1, sl], pk, pq, pb, mr)
+        _check(out[b:b + 1, sl], ref, TOL[torch.bfloat16])
+        rest = torch.ones(L, dtype=torch.bool)
+        rest[sl] = False
+        assert (out[b, rest.cuda()] == 0).all()
+
+
+# ---- fp8 Q/K ---------------------------------------------------------------------------------------
+def _outliers(x, g):
+    m = torch.rand(x.shape, generator=g) < 0.01
+    return torch.where(m, x * 20, x)
+
+
+def test_fp8_quantisation_bit_exact():
+    g = torch.Generator().manual_seed(9)
+    x = _outliers(torch.randn(700, 12, 64, generator=g) * 0.02, g).to(torch.bfloat16)
+    y, s = ops.quantize_e4m3_per_head(x.cuda())
+    ref_y, ref_s = O.quantize_e4m3_per_head(x.float().numpy())
+    assert np.array_equal(s.cpu().numpy(), ref_s)
+    assert np.array_equal(y.view(torch.uint8).cpu().numpy(), O.e4m3_encode(ref_y))
+    # a strided view (one head-major slice of a wider buffer)
+    wide = torch.zeros(700, 12, 128, dtype=torch.bfloat16)
+    wide[..., :64] = x
+    y2, s2 = ops.quantize_e4m3_per_head(wide.cuda()[..., :64])
+    assert torch.equal(y2.view(torch.uint8), y.view(torch.uint8)) and torch.equal(s2, s)
+
+
+@pytest.mark.parametrize("L,pb,mr", [(300, 32, 64), (1100, 256, 512)])
+def test_fp8_attention(L, pb, mr):
+    B, H, D = 2, 3, 64
+    g = torch.Generator().manual_seed(13)
+    q, k, v, pk, pq = _inputs(B, L, H, D, pb, mr, torch.bfloat16, 14, 0.02)
+    q, k = _outliers(q.float(), g).to(torch.bfloat16), _outliers(k.float(), g).to(torch.bfloat16)
+    q8, qs = ops.quantize_e4m3_per_head(q.cuda())
+    k8, ks = ops.quantize_e4m3_per_head(k.cuda())
+    pk8, pks = ops.quantize_e4m3_per_head(pk.cuda().transpose(0, 1))
+    pq8, pqs = ops.quantize_e4m3_per_head(pq.cuda().transpose(0, 1))
+    out = ops.disentangled_attention_fwd(q8, k8, v.cuda(), pk8.transpose(0, 1), pq8.transpose(0, 1), position_buckets=pb,
+                                         max_relative_positions=mr, q_scale=qs, k_scale=ks, pos_key_scale=pks,
+                                         pos_query_scale=pqs)
+    # (a) tight: the oracle on the de-quantised operands
+    dq = lambda y, s: y.float().cpu() * s.cpu()[:, None]
+    ref_dq = _oracle_blhd(dq(q8, qs), dq(k8, ks), v, dq(pk8, pks).transpose(0, 1), dq(pq8, pqs).transpose(0, 1), pb, mr)
+    _check(out, ref_dq, TOL[torch.bfloat16], "vs de-quantised oracle")
+    # (b) the stated bound against the unquantised reference
+    ref = _oracle_blhd(q, k, v, pk, pq, pb, mr)
+    _check(out, ref, FP8_TOL, "vs unquantised oracle")
+    # unit-scale inputs: same bounds, relative
+    q, k, v, pk, pq = _inputs(1, L, 2, D, pb, mr, torch.bfloat16, 15, 1.0)
+    q8, qs = ops.quantize_e4m3_per_head(q.cuda())
+    k8, ks = ops.quantize_e4m3_per_head(k.cuda())
+    pk8, pks = ops.quantize_e4m3_per_head(pk.cuda().transpose(0, 1))
+    pq8, pqs = ops.quantize_e4m3_per_head(pq.cuda().transpose(0, 1))
+    out = ops.disentangled_attention_fwd(q8, k8, v.cuda(), pk8.transpose(0, 1), pq8.transpose(0, 1), position_buckets=pb,
+                                         max_relative_positions=mr, q_scale=qs, k_scale=ks, pos_key_scale=pks,
+                                         pos_query_scale=pqs)
+    ref_dq = _oracle_blhd(dq(q8, qs), dq(k8, ks), v, dq(pk8, pks).transpose(0, 1), dq(pq8, pqs).transpose(0, 1), pb, mr)
+    _check(out, ref_dq, TOL[torch.bfloat16], "unit scale vs de-quantised oracle")
+
+
+# ---- module: golden vectors and the live eager class ---------------------------------------------------
+def _module_from_golden(g, dtype=torch.float32):
+    from flashdeberta_amd import FlashDisentangledSelfAttention
+
+    B, L, hid, H, pb, mr, c2p, p2c, share = g["meta"].tolist()
+
+    class Cfg:
+        hidden_size, num_attention_heads = hid, H
+        attention_probs_dropout_prob = hidden_dropout_prob = 0.1
+        pos_att_type = (["c2p"] if c2p else []) + (["p2c"] if p2c else [])
+        relative_attention, position_buckets, max_relative_positions = True, pb, mr
+        max_position_embeddings, share_att_key = 512, bool(share)
+
+    m = FlashDisentangledSelfAttention(Cfg()).eval()
+    m.load_state_dict({k[2:]: torch.from_numpy(g[k]) for k in g.files if k.startswith("w.")})
+    return m.to("cuda", dtype)
+
+
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "[a-f]_*.npz"))), ids=os.path.basename)
+@pytest.mark.parametrize("mask_form", ["2d", "4d"])
+def test_module_matches_golden(path, mask_form):
+    g = np.load(path)
+    m = _module_from_golden(g)
+    mask = torch.from_numpy(g["mask"].astype(np.int64)).cuda()
+    am = mask if mask_form == "2d" else (mask[:, None, None, :] * mask[:, None, :, None])
+    with torch.no_grad():
+        out = m(torch.from_numpy(g["hidden"]).cuda(), am, rel_embeddings=torch.from_numpy(g["rel_embeddings"]).cuda())[0]
+    valid = g["mask"].astype(bool)[:, :, None]
+    ref = np.where(valid, g["out"], 0)  # padded rows: zeros here, unspecified in eager
+    _check(out, ref, 2e-4, "module fp32 vs golden")  # projections run in fp32 GEMMs on both sides
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("share", [True, False])
+def test_module_matches_live_eager(dtype, share):
+    from transformers.models.deberta_v2.modeling_deberta_v2 import DisentangledSelfAttention
+
+    from flashdeberta_amd import FlashDisentangledSelfAttention
+
+    class Cfg:
+        hidden_size, num_attention_heads = 256, 4
+        attention_probs_dropout_prob = hidden_dropout_prob = 0.1
+        pos_att_type = ["c2p", "p2c"]
+        relative_attention, position_buckets, max_relative_positions = True, 256, 512
+        max_position_embeddings, share_att_key = 512, share
+
+    torch.manual_seed(3)
+    eager = DisentangledSelfAttention(Cfg()).eval()
+    flash = FlashDisentangledSelfAttention(Cfg()).eval()
+    flash.load_state_dict(eager.state_dict())
+    B, L = 2, 640
+    hidden = torch.randn(B, L, 256)
+    rel = torch.randn(512, 256)
+    mask = torch.ones(B, L)
+    mask[1, 500:] = 0
+    ext = mask[:, None, None, :] * mask[:, None, :, None]
+    with torch.no_grad():
+        ref = eager(hidden, ext, rel_embeddings=rel)[0].numpy()  # fp32 eager on the host
+        out = flash.to("cuda", dtype)(hidden.cuda().to(dtype), mask.cuda(), rel_embeddings=rel.cuda().to(dtype))[0]
+    ref = np.where(mask.bool().numpy()[:, :, None], ref, 0)
+    _check(out, ref, 2e-4 if dtype == torch.float32 else 3e-2)
+
+
+def test_patched_encoder_matches_eager_encoder():
+    from transformers.models.deberta_v2.modeling_deberta_v2 import DebertaV2Config, DebertaV2Model
+
+    from flashdeberta_amd import patch_model
+
+    torch.manual_seed(4)
+    cfg = DebertaV2Config(vocab_size=1000, hidden_size=768, num_hidden_layers=2, num_attention_heads=12,
+                          intermediate_size=3072, relative_attention=True, pos_att_type="p2c|c2p", position_buckets=256,
+                          share_att_key=True, norm_rel_ebd="layer_norm", position_biased_input=False,
+                          max_position_embeddings=512, hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0)
+    model = DebertaV2Model(cfg).eval().cuda().to(torch.bfloat16)
+    ids = torch.randint(0, 1000, (4, 512), device="cuda")
+    mask = torch.ones(4, 512, dtype=torch.long, device="cuda")
+    mask[2, 300:] = 0
+    with torch.no_grad():
+        ref = model(input_ids=ids, attention_mask=mask).last_hidden_state.float()
+        patch_model(model)
+        out = model(input_ids=ids, attention_mask=mask).last_hidden_state.float()
+    valid = mask.bool()[:, :, None]
+    err = ((out - ref).abs() * valid).max().item()
+    assert err < 0.1, err  # two bf16 encoder layers; hidden states are O(1) after LayerNorm
+
+
+# ---- full-size properties (metric shape: v3-base heads, seq 4096, bf16) ----------------------------------
+def test_full_size_properties():
+    B, L, H, D, pb, mr = 1, 4096, 12, 64, 256, 512
+    q, k, v, pk, pq = [_dev(x) for x in _inputs(B, L, H, D, pb, mr, torch.bfloat16, 31, 1.0)]
+    run = lambda q, k, v, pk=pk, pq=pq: ops.disentangled_attention_fwd(q, k, v, pk, pq, position_buckets=pb,
+                                                                        max_relative_positions=mr)
+    out = run(q, k, v)
+    # V = 1  =>  O = 1 (probabilities sum to one)
+    ones = run(q, k, torch.ones_like(v)).float()
+    assert (ones - 1).abs().max().item() < 1e-2
+    # permuting heads permutes the output
+    perm = torch.randperm(H, device="cuda")
+    outp = run(q[:, :, perm].contiguous(), k[:, :, perm].contiguous(), v[:, :, perm].contiguous(), pk[perm], pq[perm])
+    assert torch.equal(outp, out[:, :, perm])
+    # linear in V
+    v2 = torch.randn_like(v)
+    lin = run(q, k, v + v2).float() - out.float() - run(q, k, v2).float()
+    assert lin.abs().max().item() < 3e-2
+    # all K_r rows equal: a per-query constant, invisible to the soft-max
+    pk_const = pk[:, :1].expand_as(pk).contiguous()
+    a = run(q, k, v, pk_const, pq).float()
+    b = run(q, k, v, torch.zeros_like(pk), pq).float()
+    assert (a - b).abs().max().item() < 2e-2
+    # two heads against the oracle
+    ref = _oracle_blhd(q[:, :, :2].cpu(), k[:, :, :2].cpu(), v[:, :, :2].cpu(), pk[:2].cpu(), pq[:2].cpu(), pb, mr)
+    _check(out[:, :, :2], ref, TOL[torch.bfloat16])
+
+
+def test_bad_arguments_raise():
+    q = torch.zeros(1, 8, 2, 48, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="head_dim"):
+        ops.disentangled_attention_fwd(q, q, q)
+    q = torch.zeros(1, 8, 2, 64, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="projected relative embeddings"):
+        ops.disentangled_attention_fwd(q, q, q, torch.zeros(1, 2, 8, 64, device="cuda", dtype=torch.bfloat16)[0, :, :, :32],
+                                       None, position_buckets=32, max_relative_positions=64)
+    with pytest.raises(ValueError):
+        ops.disentangled_attention_fwd(q, q, q.float())
