@@ -1,0 +1,160 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused disentangled-attention forward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
+
+A step is one launch of the fused kernel over one batch of synthetic, HBM-resident inputs.
+Default workload = the shape the headline metric is quoted on: DeBERTa-v3-base attention
+(12 heads x 64), sequence 4096, bf16, batch 8, position_buckets 256.  Prints ONE JSON line.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0, "fp32": 157.3}
+
+WORKLOADS = {
+    # name: (B, L, H, D, dtype, kind)
+    "v3base_L4096_B8_bf16": (8, 4096, 12, 64, "bf16", "fixed"),
+    "v3base_L4096_B1_bf16": (1, 4096, 12, 64, "bf16", "fixed"),
+    "v3base_L512_B8_bf16": (8, 512, 12, 64, "bf16", "fixed"),
+    "v3large_L4096_B1_bf16": (1, 4096, 16, 64, "bf16", "fixed"),
+    "v3base_varlen64_bf16": (64, 2048, 12, 64, "bf16", "varlen"),
+    "v3base_L8192_B4_fp8": (4, 8192, 12, 64, "fp8", "fixed"),
+    "v3base_L512_B1_fp32": (1, 512, 12, 64, "fp32", "fixed"),
+}
+S2 = 512  # 2 * position_buckets
+
+
+def flops(lens, H, D, pos=True):
+    """Algorithmic FLOPs: QK^T + PV (4 L^2 D) plus each position product once (4 L 2S D), per head."""
+    return sum(H * (4 * l * l * D + (4 * l * S2 * D if pos else 0)) for l in lens)
+
+
+def make_inputs(name, device):
+    from flashdeberta_amd import ops
+    B, L, H, D, dt, kind = WORKLOADS[name]
+    g = torch.Generator(device=device).manual_seed(1234)
+    tdt = {"bf16": torch.bfloat16, "fp8": torch.bfloat16, "fp32": torch.float32}[dt]
+    rnd = lambda *s: (torch.randn(*s, device=device, generator=g) * 0.02).to(tdt)
+    pk, pq = rnd(H, S2, D), rnd(H, S2, D)
+    kw = dict(position_buckets=256, max_relative_positions=512)
+    if kind == "varlen":
+        u = torch.rand(B, generator=torch.Generator().manual_seed(1004))
+        lens = torch.exp(math.log(32) + u * (math.log(2048) - math.log(32))).round().to(torch.int64).tolist()
+        T = sum(lens)
+        q, k, v = rnd(T, H, D), rnd(T, H, D), rnd(T, H, D)
+        cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32, device=device)
+        kw.update(cu_seqlens=cu, max_seqlen=max(lens))
+    else:
+        lens = [L] * B
+        q, k, v = rnd(B, L, H, D), rnd(B, L, H, D), rnd(B, L, H, D)
+    if dt == "fp8":
+        m = torch.rand(q.shape, device=device, generator=g) < 0.01
+        q = torch.where(m, q * 20, q)
+        m = torch.rand(k.shape, device=device, generator=g) < 0.01
+        k = torch.where(m, k * 20, k)
+        q, kw["q_scale"] = ops.quantize_e4m3_per_head(q)
+        k, kw["k_scale"] = ops.quantize_e4m3_per_head(k)
+        pk8, kw["pos_key_scale"] = ops.quantize_e4m3_per_head(pk.transpose(0, 1))
+        pq8, kw["pos_query_scale"] = ops.quantize_e4m3_per_head(pq.transpose(0, 1))
+        pk, pq = pk8.transpose(0, 1), pq8.transpose(0, 1)
+    out = torch.empty(q.shape, dtype=v.dtype, device=device)
+    return (q, k, v, pk, pq), kw, out, lens
+
+
+def cpu_baseline(H, D, L):
+    """The CPU oracle (numpy restatement of the eager path, fp32) on a bounded sample of the same
+    workload: one batch element, as many heads as fit in roughly 10-30 s."""
+    from oracle import disentangled_oracle as O
+    try:
+        from threadpoolctl import threadpool_info
+        threads = max([p.get("num_threads", 1) for p in threadpool_info()] + [1])
+    except Exception:
+        threads = os.cpu_count() or 1
+    rng = np.random.default_rng(0)
+    mk = lambda *s: (rng.standard_normal(s) * 0.02).astype(np.float32)
+    q, k, v = mk(1, 1, L, D), mk(1, 1, L, D), mk(1, 1, L, D)
+    pk, pq = mk(1, S2, D), mk(1, S2, D)
+    run = lambda: O.disentangled_attention(q, k, v, pk, pq, 256, 512, dtype=np.float32)
+    t0 = time.perf_counter()
+    run()
+    one = time.perf_counter() - t0
+    heads = int(max(1, min(H, 15.0 // max(one, 1e-3))))
+    t0 = time.perf_counter()
+    for _ in range(heads):
+        run()
+    dt = time.perf_counter() - t0
+    fl = flops([L], heads, D)
+    return {"value": round(fl / dt / 1e12, 5), "unit": "TFLOP/s", "cores": int(threads), "kind": "port",
+            "sample": "numpy fp32 oracle, %d of %d heads of one batch element at L=%d (%.1f s), %.0f tokens/s per layer"
+                      % (heads, H, L, dt, L / (dt / heads * H))}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="v3base_L4096_B8_bf16", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures ONE GPU only (the path is independent per (sequence, head, "
+                 "q-tile) and uses no collectives); run with --gpus 1")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
+    from flashdeberta_amd import ops
+
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    B, L, H, D, dt, kind = WORKLOADS[args.workload]
+    tensors, kw, out, lens = make_inputs(args.workload, device)
+    step = lambda: ops.disentangled_attention_fwd(*tensors, out=out, **kw)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()  # same stream the kernel is launched on (torch's current stream)
+    for _ in range(args.steps):
+        step()
+    ev1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    kern_ms = ev0.elapsed_time(ev1) / args.steps
+    fl = flops(lens, H, D)
+    tokens = sum(lens)
+    peak = PEAK_TFLOPS[dt]
+    if dt == "fp8":  # QK^T and the position products run in fp8, PV in bf16: blended bound
+        f8 = sum(H * (2 * l * l * D + 4 * l * S2 * D) for l in lens)
+        peak = fl / (f8 / PEAK_TFLOPS["fp8"] + (fl - f8) / PEAK_TFLOPS["bf16"])
+    achieved = fl / (kern_ms * 1e-3) / 1e12
+    rec = {
+        "metric": "disentangled_attn_fwd_tflops", "value": round(fl / (wall_ms * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dt, "data": "synthetic",
+        "tokens_per_s": round(tokens / (wall_ms * 1e-3), 1),
+        "content_only_tflops": round(sum(H * 4 * l * l * D for l in lens) / (wall_ms * 1e-3) / 1e12, 2),
+        "config": {"workload": args.workload, "batch": B, "seq_len": L if kind == "fixed" else "varlen(%d tokens)" % tokens,
+                   "heads": H, "head_dim": D, "position_buckets": 256, "pos_att_type": "c2p|p2c", "layout": kind},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": round(peak, 1), "unit": "TFLOP/s",
+                     "frac": round(achieved / peak, 4), "traffic": None,
+                     "kernel_ms": round(kern_ms, 4), "algorithmic_gflop_per_launch": round(fl / 1e9, 2)},
+    }
+    if not args.no_cpu:
+        rec["cpu_baseline"] = cpu_baseline(H, D, min(L, 4096))
+    print(json.dumps(rec))
+
+
+if __name__ == "__main__":
+    main()
