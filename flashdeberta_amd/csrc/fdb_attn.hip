@@ -7,14 +7,18 @@
 // the S accumulators as its B operand.
 //
 // Position terms (what the reference reads from two pre-multiplied [B,H,L,2S] tensors with a
-// per-element float log-bucket, src/flashdeberta/ops/flash_attention.py:236-268): for a tile the
-// relative positions r = i - j form a contiguous range, so the tile's content->position scores
-// are  C[r, i] = q_i . K_r[delta(r)]  and the position->content scores  P[r, j] = k_j . Q_r[delta(r)],
-// both plain MFMA products whose A rows are gathered through the integer table delta(r).  They
-// are parked in LDS indexed by r, and the element (i, j) picks C[i-j, i] + P[i-j, j]: an address
-// that is affine in (i, j), no per-element bucket arithmetic and no trip to HBM.
-// Tiles whose r range lies entirely in a saturated zone of delta (|i-j| large) need a single row
-// of K_r / Q_r: the bias is a_i + b_j and enters through the MFMA accumulator initial value.
+// per-element float log-bucket, src/flashdeberta/ops/flash_attention.py:236-268).  delta(r),
+// r = i - j, is an integer table that is constant for |r| >= R.  The key tiles of a query tile
+// therefore fall into three consecutive ranges:
+//   far-left  (every r >= R):  delta == delta(+R).  The content->position term is a per-row constant
+//              a_i = q_i . K_r[delta], folded into the exponent; the position->content term
+//              k_j . Q_r[delta] is folded into the MFMA by using q_i + Q_r[delta] as the query.
+//   near      the tile's relative positions form one contiguous range, so its bias values are
+//              C[r, i] = q_i . K_r[delta(r)] and P[r, j] = k_j . Q_r[delta(r)]: two more MFMA
+//              products whose A rows are gathered through the table.  They are parked in LDS
+//              indexed by r, and element (i, j) adds C[i-j, i] + P[i-j, j] -- addresses affine in
+//              (i, j), no per-element bucket arithmetic, no trip to HBM.
+//   far-right (every r <= -R): like far-left with delta(-R).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -26,8 +30,10 @@ typedef __attribute__((ext_vector_type(8))) float f32x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 typedef __attribute__((ext_vector_type(4))) _Float16 f16x4;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(8))) short s16x8;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
@@ -38,9 +44,12 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kWaves = 4;
-constexpr int kC2pRows = 96;   // 32 + 64 - 1 relative positions per wave tile, padded to 3 MFMA blocks
-constexpr int kP2cRows = 192;  // 128 + 64 - 1 per workgroup tile, padded to 6 MFMA blocks
-constexpr int kP2cStride = 65; // odd stride: the skewed read walks rows and columns together
+constexpr int kC2pRows = 96;     // 32 + 64 - 1 relative positions per wave tile, padded to 3 MFMA blocks
+constexpr int kC2pStride = 100;  // elements per query row of the wave's C[i][r] scratch
+constexpr int kP2cRows = 192;    // 128 + 64 - 1 per workgroup tile, padded to 6 MFMA blocks
+constexpr int kP2cStride = 196;  // elements per key row of the workgroup's P[j][r] scratch
+constexpr float kLazyTau = 8.f;  // the running reference point of a row is moved only when the tile
+                                 // maximum exceeds it by more than 2^8 (any reference point is valid)
 
 // ---- element traits --------------------------------------------------------------------------
 // frag: the 8 contraction elements one lane feeds to a K=16 step (lane = outer index l%32, the
@@ -48,12 +57,21 @@ constexpr int kP2cStride = 65; // odd stride: the skewed read walks rows and col
 struct Bf16Tr {
   static constexpr int SZ = 2;
   using frag = bf16x8;
+  using scratch_t = __bf16;
   static __device__ __forceinline__ frag zero() { return frag{0, 0, 0, 0, 0, 0, 0, 0}; }
   static __device__ __forceinline__ frag load(const void* p) { return *(const frag*)p; }
   static __device__ __forceinline__ f32x16 mma(frag a, frag b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
+  static __device__ __forceinline__ f32x8 to_f32(frag x) { return __builtin_convertvector(x, f32x8); }
   static __device__ __forceinline__ frag from_f32(f32x8 x) { return __builtin_convertvector(x, frag); }
+  // sum of the 8 elements (as rounded to the operand type) accumulated onto acc
+  static __device__ __forceinline__ float sum8(frag x, float acc) {
+    const bf16x2 one = {(__bf16)1.0f, (__bf16)1.0f};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_fdot2_f32_bf16(bf16x2{x[2 * e], x[2 * e + 1]}, one, acc, false);
+    return acc;
+  }
   static __device__ __forceinline__ void store4(char* p, float a, float b, float c, float d) {
     f32x4 x = {a, b, c, d};
     *(bf16x4*)p = __builtin_convertvector(x, bf16x4);
@@ -63,12 +81,20 @@ struct Bf16Tr {
 struct F16Tr {
   static constexpr int SZ = 2;
   using frag = f16x8;
+  using scratch_t = _Float16;
   static __device__ __forceinline__ frag zero() { return frag{0, 0, 0, 0, 0, 0, 0, 0}; }
   static __device__ __forceinline__ frag load(const void* p) { return *(const frag*)p; }
   static __device__ __forceinline__ f32x16 mma(frag a, frag b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
+  static __device__ __forceinline__ f32x8 to_f32(frag x) { return __builtin_convertvector(x, f32x8); }
   static __device__ __forceinline__ frag from_f32(f32x8 x) { return __builtin_convertvector(x, frag); }
+  static __device__ __forceinline__ float sum8(frag x, float acc) {
+    const f16x2 one = {(_Float16)1.0f, (_Float16)1.0f};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_fdot2(f16x2{x[2 * e], x[2 * e + 1]}, one, acc, false);
+    return acc;
+  }
   static __device__ __forceinline__ void store4(char* p, float a, float b, float c, float d) {
     f32x4 x = {a, b, c, d};
     *(f16x4*)p = __builtin_convertvector(x, f16x4);
@@ -78,6 +104,7 @@ struct F16Tr {
 struct F32Tr {
   static constexpr int SZ = 4;
   using frag = f32x8;
+  using scratch_t = float;
   static __device__ __forceinline__ frag zero() { return frag{0, 0, 0, 0, 0, 0, 0, 0}; }
   static __device__ __forceinline__ frag load(const void* p) { return *(const frag*)p; }
   // A K=16 step in fp32 is eight K=2 MFMAs; lane group g supplies k = 16*step + 8*g + e to the e-th.
@@ -86,7 +113,13 @@ struct F32Tr {
     for (int e = 0; e < 8; ++e) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], b[e], c, 0, 0, 0);
     return c;
   }
+  static __device__ __forceinline__ f32x8 to_f32(frag x) { return x; }
   static __device__ __forceinline__ frag from_f32(f32x8 x) { return x; }
+  static __device__ __forceinline__ float sum8(frag x, float acc) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc += x[e];
+    return acc;
+  }
   static __device__ __forceinline__ void store4(char* p, float a, float b, float c, float d) {
     *(f32x4*)p = f32x4{a, b, c, d};
   }
@@ -95,11 +128,14 @@ struct F32Tr {
 struct Fp8Tr {  // OCP e4m3, operands of the three score products only
   static constexpr int SZ = 1;
   using frag = long;
+  using scratch_t = __bf16;
   static __device__ __forceinline__ frag zero() { return 0; }
   static __device__ __forceinline__ frag load(const void* p) { return *(const long*)p; }
   static __device__ __forceinline__ f32x16 mma(frag a, frag b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a, b, c, 0, 0, 0);
   }
+  static __device__ __forceinline__ f32x8 to_f32(frag) { return f32x8{0, 0, 0, 0, 0, 0, 0, 0}; }  // unused
+  static __device__ __forceinline__ frag from_f32(f32x8) { return 0; }                             // unused
 };
 
 // V^T operand of a K=16 step: lane (d = l%32, g = l/32) needs V[j(g,e)][d] for
@@ -150,43 +186,126 @@ __device__ __forceinline__ float wave_half_sum(float x) { return x + __shfl_xor(
 
 template <class QT, class VT, int D>
 struct Cfg {
+  using ST = typename QT::scratch_t;
   static constexpr int KSTEPS = D / 16;
   static constexpr int DBLKS = D / 32;
   static constexpr int K_RS = D * QT::SZ + 16;  // LDS row stride (bytes) of the K tile
   static constexpr int V_RS = D * VT::SZ + 16;
   static constexpr int K_BYTES = FDB_BN * K_RS;
   static constexpr int V_BYTES = FDB_BN * V_RS;
-  static constexpr int C2P_BYTES = kWaves * kC2pRows * 32 * 4;
-  static constexpr int P2C_BYTES = kP2cRows * kP2cStride * 4;
-  static constexpr int FAR_BYTES = FDB_BN * 4;
-  static constexpr int LDS_BYTES = K_BYTES + V_BYTES + C2P_BYTES + P2C_BYTES + FAR_BYTES;
+  static constexpr int K_CHUNKS = (FDB_BN * D * QT::SZ / 16 + kThreads - 1) / kThreads;  // 16-byte chunks per thread
+  static constexpr int V_CHUNKS = (FDB_BN * D * VT::SZ / 16 + kThreads - 1) / kThreads;
+  static constexpr int C2P_BYTES = kWaves * 32 * kC2pStride * (int)sizeof(ST);
+  static constexpr int P2C_BYTES = FDB_BN * kP2cStride * (int)sizeof(ST);
+  static constexpr int lds_bytes(bool c2p, bool p2c) {
+    return K_BYTES + V_BYTES + (c2p ? C2P_BYTES : 0) + (p2c ? P2C_BYTES : 0);
+  }
 };
 
-// Copy a [64 x D] tile (rows j0.., zero beyond n_valid rows) from global to LDS in 16-byte chunks.
-template <int ROW_BYTES, int RS>
-__device__ __forceinline__ void stage_tile(char* lds, const char* gbase, int64_t row_stride_bytes, int j0,
-                                           int n_rows, int tid) {
+template <class ST>
+__device__ __forceinline__ void store4_scratch(ST* p, float a, float b, float c, float d);
+template <>
+__device__ __forceinline__ void store4_scratch<float>(float* p, float a, float b, float c, float d) {
+  *(f32x4*)p = f32x4{a, b, c, d};
+}
+template <>
+__device__ __forceinline__ void store4_scratch<__bf16>(__bf16* p, float a, float b, float c, float d) {
+  f32x4 x = {a, b, c, d};
+  *(bf16x4*)p = __builtin_convertvector(x, bf16x4);
+}
+template <>
+__device__ __forceinline__ void store4_scratch<_Float16>(_Float16* p, float a, float b, float c, float d) {
+  f32x4 x = {a, b, c, d};
+  *(f16x4*)p = __builtin_convertvector(x, f16x4);
+}
+
+// [64 x ROW_BYTES] tile: global -> registers (zero beyond n_rows), registers -> LDS.
+template <int ROW_BYTES, int NCH>
+__device__ __forceinline__ void tile_load(u32x4 (&reg)[NCH], const char* gbase, int64_t row_stride_bytes, int j0,
+                                          int n_rows, int tid) {
   constexpr int CPR = ROW_BYTES / 16;
   constexpr int TOTAL = FDB_BN * CPR;
 #pragma unroll
-  for (int c = tid; c < TOTAL; c += kThreads) {
+  for (int n = 0; n < NCH; ++n) {
+    const int c = tid + n * kThreads;
     const int row = c / CPR, cc = c % CPR;
-    u32x4 val = {0, 0, 0, 0};
-    if (j0 + row < n_rows) val = *(const u32x4*)(gbase + (int64_t)(j0 + row) * row_stride_bytes + cc * 16);
-    *(u32x4*)(lds + row * RS + cc * 16) = val;
+    reg[n] = u32x4{0, 0, 0, 0};
+    if ((TOTAL % kThreads == 0 || c < TOTAL) && j0 + row < n_rows)
+      reg[n] = *(const u32x4*)(gbase + (int64_t)(j0 + row) * row_stride_bytes + cc * 16);
+  }
+}
+template <int ROW_BYTES, int RS, int NCH>
+__device__ __forceinline__ void tile_store(char* lds, const u32x4 (&reg)[NCH], int tid) {
+  constexpr int CPR = ROW_BYTES / 16;
+  constexpr int TOTAL = FDB_BN * CPR;
+#pragma unroll
+  for (int n = 0; n < NCH; ++n) {
+    const int c = tid + n * kThreads;
+    const int row = c / CPR, cc = c % CPR;
+    if (TOTAL % kThreads == 0 || c < TOTAL) *(u32x4*)(lds + row * RS + cc * 16) = reg[n];
   }
 }
 
-template <class QT, class VT, int D, bool FP8>
-__global__ __launch_bounds__(kThreads, 1) void fdb_attn_kernel(const FdbKParams p) {
-  using C = Cfg<QT, VT, D>;
-  using qfrag = typename QT::frag;
+// One key tile after its scores are in sacc (raw products, position terms already added where the
+// tile needs them element-wise): mask, online soft-max in base 2, O^T += V^T P^T.
+//   x = sacc * x_scale + row_add   (row_add: the per-row constant of a far tile, already scaled)
+template <class VT, int D, bool MASK>
+__device__ __forceinline__ void softmax_pv(f32x16 (&sacc)[2], f32x16 (&o_acc)[D / 32], float& m_run, float& l_run,
+                                           float x_scale, float row_add, const char* Vs, int v_rs, int lane, int j0,
+                                           int i, int Lb, bool causal) {
   using vfrag = typename VT::frag;
+  const int g = lane >> 5;
+  if constexpr (MASK) {
+#pragma unroll
+    for (int jb = 0; jb < 2; ++jb)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int j = j0 + 32 * jb + 8 * (v >> 2) + 4 * g + (v & 3);
+        if (j >= Lb || (causal && j > i)) sacc[jb][v] = -INFINITY;
+      }
+  }
+  float mx = sacc[0][0];
+#pragma unroll
+  for (int jb = 0; jb < 2; ++jb)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) mx = fmaxf(mx, sacc[jb][v]);
+  mx = wave_half_max(mx) * x_scale + row_add;  // x_scale > 0
+  if (__any(mx > m_run + kLazyTau)) {
+    const float m_new = (mx > m_run + kLazyTau) ? mx : m_run;
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // m_run = -inf on the first tile: 0
+    l_run *= alpha;
+    m_run = m_new;
+#pragma unroll
+    for (int d = 0; d < D / 32; ++d)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) o_acc[d][v] *= alpha;
+  }
+  const float off = row_add - m_run;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    f32x8 pv;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) pv[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[c >> 1][8 * (c & 1) + e], x_scale, off));
+    const vfrag pf = VT::from_f32(pv);
+    l_run = VT::sum8(pf, l_run);  // the row sum is taken over the probabilities as the MFMA sees them
+#pragma unroll
+    for (int d = 0; d < D / 32; ++d) {
+      const vfrag vf = VtLoad<VT>::get(Vs, v_rs, c, d, lane);
+      o_acc[d] = VT::mma(vf, pf, o_acc[d]);
+    }
+  }
+}
+
+template <class QT, class VT, int D, bool FP8, bool C2P, bool P2C>
+__global__ __launch_bounds__(kThreads, 2) void fdb_attn_kernel(const FdbKParams p) {
+  using C = Cfg<QT, VT, D>;
+  using ST = typename C::ST;
+  using qfrag = typename QT::frag;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   char* Ks = smem;
   char* Vs = Ks + C::K_BYTES;
-  float* c2pS = (float*)(Vs + C::V_BYTES);
-  float* p2cS = c2pS + C::C2P_BYTES / 4;
+  ST* c2pS = (ST*)(Vs + C::V_BYTES);
+  ST* p2cS = (ST*)((char*)c2pS + (C2P ? C::C2P_BYTES : 0));
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, li = lane & 31, g = lane >> 5;
@@ -213,8 +332,9 @@ __global__ __launch_bounds__(kThreads, 1) void fdb_attn_kernel(const FdbKParams 
   const char* kb = p.k + (ko + (int64_t)tok0 * p.k_st + (int64_t)h * p.k_sh) * QT::SZ;
   const char* vb = p.v + (vo + (int64_t)tok0 * p.v_st + (int64_t)h * p.v_sh) * VT::SZ;
   char* ob = p.out + (oo + (int64_t)tok0 * p.o_st + (int64_t)h * p.o_sh) * VT::SZ;
-  const char* pkb = p.pk ? p.pk + (int64_t)h * p.pk_sh * QT::SZ : nullptr;
-  const char* pqb = p.pq ? p.pq + (int64_t)h * p.pq_sh * QT::SZ : nullptr;
+  const char* pkb = C2P ? p.pk + (int64_t)h * p.pk_sh * QT::SZ : nullptr;
+  const char* pqb = P2C ? p.pq + (int64_t)h * p.pq_sh * QT::SZ : nullptr;
+  const int64_t k_rsb = p.k_st * QT::SZ, v_rsb = p.v_st * VT::SZ;
 
   // fp8: raw products are in units of (q_scale*k_scale); bring the two position products to the
   // same unit so that one factor converts the sum.
@@ -222,8 +342,8 @@ __global__ __launch_bounds__(kThreads, 1) void fdb_attn_kernel(const FdbKParams 
   if constexpr (FP8) {
     const float qs = p.qs[h], ks = p.ks[h];
     x_scale *= qs * ks;
-    if (pkb) c2p_mul = p.pks[h] / ks;
-    if (pqb) p2c_mul = p.pqs[h] / qs;
+    if constexpr (C2P) c2p_mul = p.pks[h] / ks;
+    if constexpr (P2C) p2c_mul = p.pqs[h] / qs;
   }
 
   const int iw0 = m0 + wave * 32;  // first row of this wave
@@ -234,6 +354,48 @@ __global__ __launch_bounds__(kThreads, 1) void fdb_attn_kernel(const FdbKParams 
   for (int s = 0; s < C::KSTEPS; ++s)
     qf[s] = (i < Lb) ? QT::load(qb + ((int64_t)i * p.q_st + 16 * s + 8 * g) * QT::SZ) : QT::zero();
 
+  // ---- tile ranges ---------------------------------------------------------------------------
+  int j_end = Lb;
+  if (p.causal) j_end = min(Lb, m0 + FDB_BM);
+  const int n_tiles = (j_end + FDB_BN - 1) / FDB_BN;
+  constexpr bool kHasPos = C2P || P2C;
+  constexpr bool kFarOk = kHasPos && !FP8;  // fp8 cannot fold Q_r into an fp8 query: all tiles take the near path
+  int t_near0 = 0, t_near1 = n_tiles;       // near tiles are [t_near0, t_near1)
+  if constexpr (!kHasPos) {
+    t_near0 = t_near1 = n_tiles;            // no position term: every tile is a plain one
+  } else if constexpr (kFarOk) {
+    const int lim = m0 - (FDB_BN - 1) - p.R;  // far-left: j0 <= lim
+    t_near0 = lim >= 0 ? min(n_tiles, lim / FDB_BN + 1) : 0;
+    t_near1 = max(t_near0, min(n_tiles, (m0 + FDB_BM - 1 + p.R + FDB_BN - 1) / FDB_BN));  // far-right: j0 >= m0+127+R
+  }
+
+  // per-row constants and shifted queries of the two far zones
+  float a_far = 0.f;  // scaled to the exponent's unit
+  qfrag qfar[C::KSTEPS];
+  auto setup_far = [&](int side) {  // side 0: far-left (delta(+R)), 1: far-right (delta(-R))
+    const int delta = p.lut[side == 0 ? 2 * p.R : 0];
+    if constexpr (C2P) {
+      const char* row = pkb + (int64_t)delta * p.pk_sr * QT::SZ;
+      float acc = 0.f;
+#pragma unroll
+      for (int s = 0; s < C::KSTEPS; ++s) {
+        const f32x8 a = QT::to_f32(QT::load(row + (16 * s + 8 * g) * QT::SZ)), q8 = QT::to_f32(qf[s]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc = __builtin_fmaf(a[e], q8[e], acc);
+      }
+      a_far = wave_half_sum(acc) * x_scale;
+    }
+    if constexpr (P2C) {
+      const char* row = pqb + (int64_t)delta * p.pq_sr * QT::SZ;
+#pragma unroll
+      for (int s = 0; s < C::KSTEPS; ++s)
+        qfar[s] = QT::from_f32(QT::to_f32(qf[s]) + QT::to_f32(QT::load(row + (16 * s + 8 * g) * QT::SZ)));
+    } else {
+#pragma unroll
+      for (int s = 0; s < C::KSTEPS; ++s) qfar[s] = qf[s];
+    }
+  };
+
   f32x16 o_acc[C::DBLKS];
 #pragma unroll
   for (int d = 0; d < C::DBLKS; ++d)
@@ -241,17 +403,21 @@ __global__ __launch_bounds__(kThreads, 1) void fdb_attn_kernel(const FdbKParams 
     for (int v = 0; v < 16; ++v) o_acc[d][v] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;  // l_run: this lane's half of the row sum
 
-  int j_end = Lb;
-  if (p.causal) j_end = min(Lb, m0 + FDB_BM);
+  u32x4 kreg[C::K_CHUNKS], vreg[C::V_CHUNKS];
+  tile_load<D * QT::SZ>(kreg, kb, k_rsb, 0, Lb, tid);
+  tile_load<D * VT::SZ>(vreg, vb, v_rsb, 0, Lb, tid);
 
-  for (int j0 = 0; j0 < j_end; j0 += FDB_BN) {
+  auto stage = [&](int t) {
     __syncthreads();  // every wave is done with the previous tile and its bias scratch
-    stage_tile<D * QT::SZ, C::K_RS>(Ks, kb, p.k_st * QT::SZ, j0, Lb, tid);
-    stage_tile<D * VT::SZ, C::V_RS>(Vs, vb, p.v_st * VT::SZ, j0, Lb, tid);
+    tile_store<D * QT::SZ, C::K_RS>(Ks, kreg, tid);
+    tile_store<D * VT::SZ, C::V_RS>(Vs, vreg, tid);
     __syncthreads();
-
-    // ---- S^T = K Q^T -------------------------------------------------------------------------
-    f32x16 sacc[2];
+    if (t + 1 < n_tiles) {  // next tile's global loads fly during this tile's math
+      tile_load<D * QT::SZ>(kreg, kb, k_rsb, (t + 1) * FDB_BN, Lb, tid);
+      tile_load<D * VT::SZ>(vreg, vb, v_rsb, (t + 1) * FDB_BN, Lb, tid);
+    }
+  };
+  auto qk = [&](f32x16 (&sacc)[2], const qfrag (&qq)[C::KSTEPS]) {
 #pragma unroll
     for (int jb = 0; jb < 2; ++jb) {
 #pragma unroll
@@ -259,121 +425,105 @@ __global__ __launch_bounds__(kThreads, 1) void fdb_attn_kernel(const FdbKParams 
 #pragma unroll
       for (int s = 0; s < C::KSTEPS; ++s) {
         qfrag kf = QT::load(Ks + (jb * 32 + li) * C::K_RS + (16 * s + 8 * g) * QT::SZ);
-        sacc[jb] = QT::mma(kf, qf[s], sacc[jb]);
+        sacc[jb] = QT::mma(kf, qq[s], sacc[jb]);
       }
     }
+  };
+  auto finish = [&](f32x16 (&sacc)[2], int j0, float row_add) {
+    const bool need_mask = (j0 + FDB_BN > Lb) || (p.causal && j0 + FDB_BN - 1 > iw0);
+    if (need_mask)
+      softmax_pv<VT, D, true>(sacc, o_acc, m_run, l_run, x_scale, row_add, Vs, C::V_RS, lane, j0, i, Lb, p.causal != 0);
+    else
+      softmax_pv<VT, D, false>(sacc, o_acc, m_run, l_run, x_scale, row_add, Vs, C::V_RS, lane, j0, i, Lb, false);
+  };
+  auto far_range = [&](int t0, int t1, int side) {
+    if (t0 >= t1) return;
+    if constexpr (kFarOk) setup_far(side);
+    for (int t = t0; t < t1; ++t) {
+      stage(t);
+      f32x16 sacc[2];
+      if constexpr (kFarOk) qk(sacc, qfar); else qk(sacc, qf);
+      finish(sacc, t * FDB_BN, a_far);
+    }
+  };
 
-    // ---- position terms ----------------------------------------------------------------------
-    if (pkb) {
-      // C[r - r_lo, i] for the 95 relative positions this wave's 32 rows see in this key tile
-      const int r_lo = iw0 - (j0 + FDB_BN - 1);
+  // ---- far-left ------------------------------------------------------------------------------
+  far_range(0, t_near0, 0);
+
+  // ---- near ----------------------------------------------------------------------------------
+  if constexpr (kHasPos) {
+    for (int t = t_near0; t < t_near1; ++t) {
+      const int j0 = t * FDB_BN;
+      stage(t);
+      f32x16 sacc[2];
+      qk(sacc, qf);
+      if constexpr (C2P) {
+        // C[i][r - r_lo] for the 95 relative positions this wave's 32 rows see in this key tile
+        const int r_lo = iw0 - (j0 + FDB_BN - 1);
+        ST* dst0 = c2pS + (wave * 32 + li) * kC2pStride + 4 * g;
 #pragma unroll 1
-      for (int blk = 0; blk < 3; ++blk) {
-        int r = r_lo + 32 * blk + li;
-        r = max(-p.R, min(p.R, r));
-        const int delta = p.lut[r + p.R];
-        const char* row = pkb + (int64_t)delta * p.pk_sr * QT::SZ;
-        f32x16 acc;
+        for (int blk = 0; blk < 3; ++blk) {
+          int r = r_lo + 32 * blk + li;
+          r = max(-p.R, min(p.R, r));
+          const int delta = p.lut[r + p.R];
+          const char* row = pkb + (int64_t)delta * p.pk_sr * QT::SZ;
+          f32x16 acc;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+          for (int v = 0; v < 16; ++v) acc[v] = 0.f;
 #pragma unroll
-        for (int s = 0; s < C::KSTEPS; ++s) acc = QT::mma(QT::load(row + (16 * s + 8 * g) * QT::SZ), qf[s], acc);
-        float* dst = c2pS + wave * (kC2pRows * 32) + (32 * blk + 4 * g) * 32 + li;
+          for (int s = 0; s < C::KSTEPS; ++s) acc = QT::mma(QT::load(row + (16 * s + 8 * g) * QT::SZ), qf[s], acc);
+          if constexpr (FP8) acc *= c2p_mul;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) dst[(8 * (v >> 2) + (v & 3)) * 32] = FP8 ? acc[v] * c2p_mul : acc[v];
-      }
-    }
-    if (pqb) {
-      // P[r - r_lo, j] for the 191 relative positions of the whole 128 x 64 tile; 12 MFMA blocks
-      // (6 row blocks x 2 key blocks) shared by the 4 waves.
-      const int r_lo = m0 - (j0 + FDB_BN - 1);
-#pragma unroll 1
-      for (int n = 0; n < 3; ++n) {
-        const int task = wave * 3 + n, wblk = task >> 1, jblk = task & 1;
-        int r = r_lo + 32 * wblk + li;
-        r = max(-p.R, min(p.R, r));
-        const int delta = p.lut[r + p.R];
-        const char* row = pqb + (int64_t)delta * p.pq_sr * QT::SZ;
-        f32x16 acc;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc[v] = 0.f;
-#pragma unroll
-        for (int s = 0; s < C::KSTEPS; ++s) {
-          qfrag kf = QT::load(Ks + (jblk * 32 + li) * C::K_RS + (16 * s + 8 * g) * QT::SZ);
-          acc = QT::mma(QT::load(row + (16 * s + 8 * g) * QT::SZ), kf, acc);
+          for (int q4 = 0; q4 < 4; ++q4)  // rows r - r_lo = 32*blk + 8*q4 + 4*g + 0..3 of column i = li
+            store4_scratch<ST>(dst0 + 32 * blk + 8 * q4, acc[4 * q4], acc[4 * q4 + 1], acc[4 * q4 + 2], acc[4 * q4 + 3]);
         }
-        float* dst = p2cS + (32 * wblk + 4 * g) * kP2cStride + jblk * 32 + li;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) dst[(8 * (v >> 2) + (v & 3)) * kP2cStride] = FP8 ? acc[v] * p2c_mul : acc[v];
       }
-    }
-    if (pkb || pqb) {
+      if constexpr (P2C) {
+        // P[j][r - r_lo] for the 191 relative positions of the whole 128 x 64 tile; 12 MFMA blocks
+        // (6 row blocks x 2 key blocks) shared by the 4 waves.
+        const int r_lo = m0 - (j0 + FDB_BN - 1);
+#pragma unroll 1
+        for (int n = 0; n < 3; ++n) {
+          const int task = wave * 3 + n, wblk = task >> 1, jblk = task & 1;
+          int r = r_lo + 32 * wblk + li;
+          r = max(-p.R, min(p.R, r));
+          const int delta = p.lut[r + p.R];
+          const char* row = pqb + (int64_t)delta * p.pq_sr * QT::SZ;
+          f32x16 acc;
+#pragma unroll
+          for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+#pragma unroll
+          for (int s = 0; s < C::KSTEPS; ++s) {
+            qfrag kf = QT::load(Ks + (jblk * 32 + li) * C::K_RS + (16 * s + 8 * g) * QT::SZ);
+            acc = QT::mma(QT::load(row + (16 * s + 8 * g) * QT::SZ), kf, acc);
+          }
+          if constexpr (FP8) acc *= p2c_mul;
+          ST* dst0 = p2cS + (jblk * 32 + li) * kP2cStride + 32 * wblk + 4 * g;
+#pragma unroll
+          for (int q4 = 0; q4 < 4; ++q4)
+            store4_scratch<ST>(dst0 + 8 * q4, acc[4 * q4], acc[4 * q4 + 1], acc[4 * q4 + 2], acc[4 * q4 + 3]);
+        }
+      }
       __syncthreads();
       // element (j = j0 + jj, i): r - r_lo = li + 63 - jj (wave tile) / wave*32 + li + 63 - jj (workgroup tile)
-      const float* cbase = c2pS + wave * (kC2pRows * 32) + (li + 63 - 4 * g) * 32 + li;
-      const float* pbase = p2cS + (wave * 32 + li + 63 - 4 * g) * kP2cStride + 4 * g;
+      {
+        const ST* cbase = c2pS + (wave * 32 + li) * kC2pStride + (li + 63 - 4 * g);
+        const ST* pbase = p2cS + (4 * g) * kP2cStride + (wave * 32 + li + 63 - 4 * g);
 #pragma unroll
-      for (int jb = 0; jb < 2; ++jb)
+        for (int jb = 0; jb < 2; ++jb)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int cj = 32 * jb + 8 * (v >> 2) + (v & 3);  // jj = cj + 4*g
-          float add = 0.f;
-          if (pkb) add += cbase[-cj * 32];
-          if (pqb) add += pbase[-cj * kP2cStride + cj];
-          sacc[jb][v] += add;
-        }
-    }
-
-    // ---- mask, online soft-max (base 2) -------------------------------------------------------
-    const bool tail = (j0 + FDB_BN > Lb) || (p.causal && j0 + FDB_BN > iw0);
-    float mx = -INFINITY;
-#pragma unroll
-    for (int jb = 0; jb < 2; ++jb)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        float x = sacc[jb][v] * x_scale;
-        if (tail) {
-          const int j = j0 + 32 * jb + 8 * (v >> 2) + 4 * g + (v & 3);
-          if (j >= Lb || (p.causal && j > i)) x = -INFINITY;
-        }
-        sacc[jb][v] = x;
-        mx = fmaxf(mx, x);
+          for (int v = 0; v < 16; ++v) {
+            const int cj = 32 * jb + 8 * (v >> 2) + (v & 3);  // jj = cj + 4*g
+            if constexpr (C2P) sacc[jb][v] += (float)cbase[-cj];
+            if constexpr (P2C) sacc[jb][v] += (float)pbase[cj * kP2cStride - cj];
+          }
       }
-    mx = wave_half_max(mx);
-    const float m_new = fmaxf(m_run, mx);
-    // a row with no visible key so far keeps m_new = -inf; use 0 as the reference point then
-    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
-    float rs = 0.f;
-#pragma unroll
-    for (int jb = 0; jb < 2; ++jb)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const float e = __builtin_amdgcn_exp2f(sacc[jb][v] - m_use);
-        sacc[jb][v] = e;
-        rs += e;
-      }
-    l_run = l_run * alpha + rs;
-    m_run = m_new;
-#pragma unroll
-    for (int d = 0; d < C::DBLKS; ++d)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) o_acc[d][v] *= alpha;
-
-    // ---- O^T += V^T P^T -----------------------------------------------------------------------
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      f32x8 pv;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) pv[e] = sacc[c >> 1][8 * (c & 1) + e];
-      const vfrag pf = VT::from_f32(pv);
-#pragma unroll
-      for (int d = 0; d < C::DBLKS; ++d) {
-        const vfrag vf = VtLoad<VT>::get(Vs, C::V_RS, c, d, lane);
-        o_acc[d] = VT::mma(vf, pf, o_acc[d]);
-      }
+      finish(sacc, j0, 0.f);
     }
   }
+
+  // ---- far-right -----------------------------------------------------------------------------
+  far_range(t_near1, n_tiles, 1);
 
   // ---- epilogue ------------------------------------------------------------------------------
   const float l_tot = wave_half_sum(l_run);
@@ -395,15 +545,24 @@ __global__ __launch_bounds__(kThreads, 1) void fdb_attn_kernel(const FdbKParams 
   }
 }
 
-template <class QT, class VT, int D, bool FP8>
+template <class QT, class VT, int D, bool FP8, bool C2P, bool P2C>
 int launch_one(const FdbKParams& p, int grid_x, hipStream_t stream) {
   using C = Cfg<QT, VT, D>;
-  auto kern = fdb_attn_kernel<QT, VT, D, FP8>;
-  static_assert(C::LDS_BYTES <= 160 * 1024, "LDS budget");
-  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+  auto kern = fdb_attn_kernel<QT, VT, D, FP8, C2P, P2C>;
+  constexpr int lds = C::lds_bytes(C2P, P2C);
+  static_assert(lds <= 160 * 1024, "LDS budget");
+  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
   if (e != hipSuccess) return (int)e;
-  hipLaunchKernelGGL(kern, dim3(grid_x, p.H, 1), dim3(kThreads), C::LDS_BYTES, stream, p);
+  hipLaunchKernelGGL(kern, dim3(grid_x, p.H, 1), dim3(kThreads), lds, stream, p);
   return (int)hipGetLastError();
+}
+
+template <class QT, class VT, int D, bool FP8>
+int launch_pos(const FdbKParams& p, int grid_x, hipStream_t stream) {
+  if (p.pk && p.pq) return launch_one<QT, VT, D, FP8, true, true>(p, grid_x, stream);
+  if (p.pk) return launch_one<QT, VT, D, FP8, true, false>(p, grid_x, stream);
+  if (p.pq) return launch_one<QT, VT, D, FP8, false, true>(p, grid_x, stream);
+  return launch_one<QT, VT, D, FP8, false, false>(p, grid_x, stream);
 }
 
 }  // namespace
@@ -412,9 +571,9 @@ int fdb_launch_attn(const FdbKParams& p, int dtype, int head_dim, int grid_x, vo
   hipStream_t stream = (hipStream_t)stream_;
 #define FDB_DISPATCH_D(QT, VT, FP8)                                   \
   switch (head_dim) {                                                 \
-    case 32: return launch_one<QT, VT, 32, FP8>(p, grid_x, stream);   \
-    case 64: return launch_one<QT, VT, 64, FP8>(p, grid_x, stream);   \
-    case 128: return launch_one<QT, VT, 128, FP8>(p, grid_x, stream); \
+    case 32: return launch_pos<QT, VT, 32, FP8>(p, grid_x, stream);   \
+    case 64: return launch_pos<QT, VT, 64, FP8>(p, grid_x, stream);   \
+    case 128: return launch_pos<QT, VT, 128, FP8>(p, grid_x, stream); \
     default: return FDB_ERR_HEAD_DIM;                                 \
   }
   switch (dtype) {
@@ -422,8 +581,8 @@ int fdb_launch_attn(const FdbKParams& p, int dtype, int head_dim, int grid_x, vo
     case FDB_F16: FDB_DISPATCH_D(F16Tr, F16Tr, false)
     case FDB_F32:
       switch (head_dim) {
-        case 32: return launch_one<F32Tr, F32Tr, 32, false>(p, grid_x, stream);
-        case 64: return launch_one<F32Tr, F32Tr, 64, false>(p, grid_x, stream);
+        case 32: return launch_pos<F32Tr, F32Tr, 32, false>(p, grid_x, stream);
+        case 64: return launch_pos<F32Tr, F32Tr, 64, false>(p, grid_x, stream);
         default: return FDB_ERR_UNSUPPORTED;
       }
     case FDB_FP8_E4M3: FDB_DISPATCH_D(Fp8Tr, Bf16Tr, true)
