@@ -219,7 +219,8 @@ __device__ __forceinline__ void store4_scratch<_Float16>(_Float16* p, float a, f
   *(f16x4*)p = __builtin_convertvector(x, f16x4);
 }
 
-// [64 x ROW_BYTES] tile: global -> registers (zero beyond n_rows), registers -> LDS.
+// [64 x ROW_BYTES] tile: global -> registers -> LDS.  Rows past the end of the sequence re-read the
+// last valid row (finite data, no predication); their scores are masked to -inf before the soft-max.
 template <int ROW_BYTES, int NCH>
 __device__ __forceinline__ void tile_load(u32x4 (&reg)[NCH], const char* gbase, int64_t row_stride_bytes, int j0,
                                           int n_rows, int tid) {
@@ -228,10 +229,8 @@ __device__ __forceinline__ void tile_load(u32x4 (&reg)[NCH], const char* gbase, 
 #pragma unroll
   for (int n = 0; n < NCH; ++n) {
     const int c = tid + n * kThreads;
-    const int row = c / CPR, cc = c % CPR;
-    reg[n] = u32x4{0, 0, 0, 0};
-    if ((TOTAL % kThreads == 0 || c < TOTAL) && j0 + row < n_rows)
-      reg[n] = *(const u32x4*)(gbase + (int64_t)(j0 + row) * row_stride_bytes + cc * 16);
+    const int row = min(j0 + min(c / CPR, FDB_BN - 1), n_rows - 1), cc = c % CPR;
+    reg[n] = *(const u32x4*)(gbase + (int64_t)row * row_stride_bytes + cc * 16);
   }
 }
 template <int ROW_BYTES, int RS, int NCH>
@@ -296,8 +295,12 @@ __device__ __forceinline__ void softmax_pv(f32x16 (&sacc)[2], f32x16 (&o_acc)[D 
   }
 }
 
+// Two workgroups share a CU (and its 512 registers per lane) when the LDS footprint allows it.
+template <class QT, class VT, int D, bool C2P, bool P2C>
+constexpr int min_blocks() { return Cfg<QT, VT, D>::lds_bytes(C2P, P2C) <= 80 * 1024 ? 2 : 1; }
+
 template <class QT, class VT, int D, bool FP8, bool C2P, bool P2C>
-__global__ __launch_bounds__(kThreads, 2) void fdb_attn_kernel(const FdbKParams p) {
+__global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C>())) void fdb_attn_kernel(const FdbKParams p) {
   using C = Cfg<QT, VT, D>;
   using ST = typename C::ST;
   using qfrag = typename QT::frag;
@@ -452,50 +455,78 @@ __global__ __launch_bounds__(kThreads, 2) void fdb_attn_kernel(const FdbKParams 
 
   // ---- near ----------------------------------------------------------------------------------
   if constexpr (kHasPos) {
+    // Row offsets (bytes) into K_r / Q_r of the A rows this lane feeds to the position products
+    // of one tile; looked up through the table one tile ahead so that the row loads of a tile
+    // never wait for the table.
+    int64_t off_c[3], off_p[3];
+    auto lookup = [&](int t) {
+      const int j0 = t * FDB_BN;
+      if constexpr (C2P) {
+        const int r_lo = iw0 - (j0 + FDB_BN - 1);  // the 95 relative positions of this wave's 32 rows
+#pragma unroll
+        for (int blk = 0; blk < 3; ++blk) {
+          const int r = max(-p.R, min(p.R, r_lo + 32 * blk + li));
+          off_c[blk] = (int64_t)p.lut[r + p.R] * p.pk_sr * QT::SZ + 8 * g * QT::SZ;
+        }
+      }
+      if constexpr (P2C) {
+        const int r_lo = m0 - (j0 + FDB_BN - 1);  // the 191 relative positions of the 128 x 64 tile
+#pragma unroll
+        for (int n = 0; n < 3; ++n) {
+          const int wblk = (wave * 3 + n) >> 1;
+          const int r = max(-p.R, min(p.R, r_lo + 32 * wblk + li));
+          off_p[n] = (int64_t)p.lut[r + p.R] * p.pq_sr * QT::SZ + 8 * g * QT::SZ;
+        }
+      }
+    };
+    if (t_near0 < t_near1) lookup(t_near0);
     for (int t = t_near0; t < t_near1; ++t) {
       const int j0 = t * FDB_BN;
+      qfrag ac[C2P ? 3 : 1][C::KSTEPS], ap[P2C ? 3 : 1][C::KSTEPS];
+      if constexpr (C2P) {
+#pragma unroll
+        for (int blk = 0; blk < 3; ++blk)
+#pragma unroll
+          for (int s = 0; s < C::KSTEPS; ++s) ac[blk][s] = QT::load(pkb + off_c[blk] + 16 * s * QT::SZ);
+      }
+      if constexpr (P2C) {
+#pragma unroll
+        for (int n = 0; n < 3; ++n)
+#pragma unroll
+          for (int s = 0; s < C::KSTEPS; ++s) ap[n][s] = QT::load(pqb + off_p[n] + 16 * s * QT::SZ);
+      }
       stage(t);
+      if (t + 1 < t_near1) lookup(t + 1);
       f32x16 sacc[2];
       qk(sacc, qf);
       if constexpr (C2P) {
-        // C[i][r - r_lo] for the 95 relative positions this wave's 32 rows see in this key tile
-        const int r_lo = iw0 - (j0 + FDB_BN - 1);
+        // C[i][r - r_lo]: column i = li, rows 32*blk + 8*q4 + 4*g + 0..3
         ST* dst0 = c2pS + (wave * 32 + li) * kC2pStride + 4 * g;
-#pragma unroll 1
+#pragma unroll
         for (int blk = 0; blk < 3; ++blk) {
-          int r = r_lo + 32 * blk + li;
-          r = max(-p.R, min(p.R, r));
-          const int delta = p.lut[r + p.R];
-          const char* row = pkb + (int64_t)delta * p.pk_sr * QT::SZ;
           f32x16 acc;
 #pragma unroll
           for (int v = 0; v < 16; ++v) acc[v] = 0.f;
 #pragma unroll
-          for (int s = 0; s < C::KSTEPS; ++s) acc = QT::mma(QT::load(row + (16 * s + 8 * g) * QT::SZ), qf[s], acc);
+          for (int s = 0; s < C::KSTEPS; ++s) acc = QT::mma(ac[blk][s], qf[s], acc);
           if constexpr (FP8) acc *= c2p_mul;
 #pragma unroll
-          for (int q4 = 0; q4 < 4; ++q4)  // rows r - r_lo = 32*blk + 8*q4 + 4*g + 0..3 of column i = li
+          for (int q4 = 0; q4 < 4; ++q4)
             store4_scratch<ST>(dst0 + 32 * blk + 8 * q4, acc[4 * q4], acc[4 * q4 + 1], acc[4 * q4 + 2], acc[4 * q4 + 3]);
         }
       }
       if constexpr (P2C) {
-        // P[j][r - r_lo] for the 191 relative positions of the whole 128 x 64 tile; 12 MFMA blocks
-        // (6 row blocks x 2 key blocks) shared by the 4 waves.
-        const int r_lo = m0 - (j0 + FDB_BN - 1);
-#pragma unroll 1
+        // P[j][r - r_lo]: 12 MFMA blocks (6 row blocks x 2 key blocks) shared by the 4 waves
+#pragma unroll
         for (int n = 0; n < 3; ++n) {
           const int task = wave * 3 + n, wblk = task >> 1, jblk = task & 1;
-          int r = r_lo + 32 * wblk + li;
-          r = max(-p.R, min(p.R, r));
-          const int delta = p.lut[r + p.R];
-          const char* row = pqb + (int64_t)delta * p.pq_sr * QT::SZ;
           f32x16 acc;
 #pragma unroll
           for (int v = 0; v < 16; ++v) acc[v] = 0.f;
 #pragma unroll
           for (int s = 0; s < C::KSTEPS; ++s) {
             qfrag kf = QT::load(Ks + (jblk * 32 + li) * C::K_RS + (16 * s + 8 * g) * QT::SZ);
-            acc = QT::mma(QT::load(row + (16 * s + 8 * g) * QT::SZ), kf, acc);
+            acc = QT::mma(ap[n][s], kf, acc);
           }
           if constexpr (FP8) acc *= p2c_mul;
           ST* dst0 = p2cS + (jblk * 32 + li) * kP2cStride + 32 * wblk + 4 * g;
