@@ -22,6 +22,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "fdb_kernels.h"
 #include "../../include/fdb.h"
 
@@ -181,8 +183,26 @@ template <>
 struct VtLoad<F16Tr> : VtLoad16<F16Tr> {};
 
 // combine lane l with lane l^32 (the other half of the row's keys)
-__device__ __forceinline__ float wave_half_max(float x) { return fmaxf(x, __shfl_xor(x, 32)); }
-__device__ __forceinline__ float wave_half_sum(float x) { return x + __shfl_xor(x, 32); }
+// v_permlane32_swap exchanges lanes 32..63 of its first operand with lanes 0..31 of its second.
+// Fed two registers holding the same value, every lane ends up with its own value in one register
+// and its partner's (lane ^ 32) in the other.  Written as one asm block: the two operands must be
+// distinct registers, and the results must stay opaque to the optimiser.
+__device__ __forceinline__ void half_pair(float x, float& r0, float& r1) {
+  float a = x, b;
+  asm volatile("v_mov_b32 %1, %0\n\ts_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "=&v"(b));
+  r0 = a;
+  r1 = b;
+}
+__device__ __forceinline__ float wave_half_max(float x) {
+  float a, b;
+  half_pair(x, a, b);
+  return fmaxf(a, b);
+}
+__device__ __forceinline__ float wave_half_sum(float x) {
+  float a, b;
+  half_pair(x, a, b);
+  return a + b;
+}
 
 template <class QT, class VT, int D>
 struct Cfg {
@@ -375,7 +395,7 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C>())) void
   // per-row constants and shifted queries of the two far zones
   float a_far = 0.f;  // scaled to the exponent's unit
   qfrag qfar[C::KSTEPS];
-  auto setup_far = [&](int side) {  // side 0: far-left (delta(+R)), 1: far-right (delta(-R))
+  auto setup_far = [&](int side) __attribute__((always_inline)) {  // side 0: far-left (delta(+R)), 1: far-right (delta(-R))
     const int delta = p.lut[side == 0 ? 2 * p.R : 0];
     if constexpr (C2P) {
       const char* row = pkb + (int64_t)delta * p.pk_sr * QT::SZ;
@@ -410,7 +430,7 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C>())) void
   tile_load<D * QT::SZ>(kreg, kb, k_rsb, 0, Lb, tid);
   tile_load<D * VT::SZ>(vreg, vb, v_rsb, 0, Lb, tid);
 
-  auto stage = [&](int t) {
+  auto stage = [&](int t) __attribute__((always_inline)) {
     __syncthreads();  // every wave is done with the previous tile and its bias scratch
     tile_store<D * QT::SZ, C::K_RS>(Ks, kreg, tid);
     tile_store<D * VT::SZ, C::V_RS>(Vs, vreg, tid);
@@ -420,7 +440,7 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C>())) void
       tile_load<D * VT::SZ>(vreg, vb, v_rsb, (t + 1) * FDB_BN, Lb, tid);
     }
   };
-  auto qk = [&](f32x16 (&sacc)[2], const qfrag (&qq)[C::KSTEPS]) {
+  auto qk = [&](f32x16 (&sacc)[2], const qfrag (&qq)[C::KSTEPS]) __attribute__((always_inline)) {
 #pragma unroll
     for (int jb = 0; jb < 2; ++jb) {
 #pragma unroll
@@ -432,22 +452,25 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C>())) void
       }
     }
   };
-  auto finish = [&](f32x16 (&sacc)[2], int j0, float row_add) {
-    const bool need_mask = (j0 + FDB_BN > Lb) || (p.causal && j0 + FDB_BN - 1 > iw0);
-    if (need_mask)
-      softmax_pv<VT, D, true>(sacc, o_acc, m_run, l_run, x_scale, row_add, Vs, C::V_RS, lane, j0, i, Lb, p.causal != 0);
-    else
-      softmax_pv<VT, D, false>(sacc, o_acc, m_run, l_run, x_scale, row_add, Vs, C::V_RS, lane, j0, i, Lb, false);
-  };
-  auto far_range = [&](int t0, int t1, int side) {
-    if (t0 >= t1) return;
-    if constexpr (kFarOk) setup_far(side);
+  // Tiles that need no mask: entirely inside the sequence and, when causal, entirely below the
+  // diagonal of every row of the workgroup (causal runs keep it simple: all near tiles are masked).
+  const int n_full = p.causal ? min(Lb / FDB_BN, t_near0) : Lb / FDB_BN;
+  auto far_loop = [&](auto mask_tag, int t0, int t1) __attribute__((always_inline)) {
+    constexpr bool MASK = decltype(mask_tag)::value;
     for (int t = t0; t < t1; ++t) {
       stage(t);
       f32x16 sacc[2];
       if constexpr (kFarOk) qk(sacc, qfar); else qk(sacc, qf);
-      finish(sacc, t * FDB_BN, a_far);
+      softmax_pv<VT, D, MASK>(sacc, o_acc, m_run, l_run, x_scale, a_far, Vs, C::V_RS, lane, t * FDB_BN, i, Lb,
+                              MASK && p.causal != 0);
     }
+  };
+  auto far_range = [&](int t0, int t1, int side) __attribute__((always_inline)) {
+    if (t0 >= t1) return;
+    if constexpr (kFarOk) setup_far(side);
+    const int tm = max(t0, min(t1, n_full));
+    far_loop(std::false_type{}, t0, tm);
+    far_loop(std::true_type{}, tm, t1);
   };
 
   // ---- far-left ------------------------------------------------------------------------------
@@ -459,7 +482,7 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C>())) void
     // of one tile; looked up through the table one tile ahead so that the row loads of a tile
     // never wait for the table.
     int64_t off_c[3], off_p[3];
-    auto lookup = [&](int t) {
+    auto lookup = [&](int t) __attribute__((always_inline)) {
       const int j0 = t * FDB_BN;
       if constexpr (C2P) {
         const int r_lo = iw0 - (j0 + FDB_BN - 1);  // the 95 relative positions of this wave's 32 rows
@@ -480,7 +503,9 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C>())) void
       }
     };
     if (t_near0 < t_near1) lookup(t_near0);
-    for (int t = t_near0; t < t_near1; ++t) {
+    auto near_loop = [&](auto mask_tag, int t0, int t1) __attribute__((always_inline)) {
+    constexpr bool MASK = decltype(mask_tag)::value;
+    for (int t = t0; t < t1; ++t) {
       const int j0 = t * FDB_BN;
       qfrag ac[C2P ? 3 : 1][C::KSTEPS], ap[P2C ? 3 : 1][C::KSTEPS];
       if constexpr (C2P) {
@@ -549,8 +574,13 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C>())) void
             if constexpr (P2C) sacc[jb][v] += (float)pbase[cj * kP2cStride - cj];
           }
       }
-      finish(sacc, j0, 0.f);
+      softmax_pv<VT, D, MASK>(sacc, o_acc, m_run, l_run, x_scale, 0.f, Vs, C::V_RS, lane, j0, i, Lb,
+                              MASK && p.causal != 0);
     }
+    };
+    const int tm = max(t_near0, min(t_near1, n_full));
+    near_loop(std::false_type{}, t_near0, tm);
+    near_loop(std::true_type{}, tm, t_near1);
   }
 
   // ---- far-right -----------------------------------------------------------------------------
