@@ -167,13 +167,24 @@ int fdb_attn_fwd(const fdb_attn_args* a, void* stream) {
   p.B = a->batch; p.H = a->heads; p.L = a->max_seqlen;
   p.tiles_per_seq = (a->max_seqlen + FDB_BM - 1) / FDB_BM;
   p.R = a->lut_radius > 0 ? a->lut_radius : 1;
-  p.r_neg = -p.R; p.r_pos = p.R;
   p.causal = a->causal ? 1 : 0;
   p.scale_log2 = a->sm_scale * 1.4426950408889634f;
   int64_t grid_x = a->cu_seqlens ? fdb_worklist_max_tiles(a->total_tokens, a->batch)
                                  : (int64_t)a->batch * p.tiles_per_seq;
   if (grid_x < 1 || grid_x > INT32_MAX) return FDB_ERR_SHAPE;
-  return fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, stream);
+  // Split path: the far tiles in a far-only run of the fused kernel (lean, four workgroups per
+  // CU), the near tiles in the near kernel, which merges the two.  It needs the log-sum-exp buffer
+  // as the hand-over between the two launches.
+  if ((a->pos_key || a->pos_query) && a->lse && fdb_near_supported(a->dtype, a->head_dim)) {
+    const bool need_far = a->max_seqlen > p.R + FDB_BN - 1;  // otherwise no tile of any query tile is far
+    if (need_far) {
+      const int rc_far = fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, true, stream);
+      if (rc_far != 0) return rc_far;
+    }
+    p.far_done = need_far ? 1 : 0;
+    return fdb_launch_near(p, a->dtype, a->head_dim, (int)grid_x, stream);
+  }
+  return fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, false, stream);
 }
 
 int fdb_build_worklist(const int32_t* cu_seqlens, int32_t batch, int32_t total_tokens, int32_t* worklist,

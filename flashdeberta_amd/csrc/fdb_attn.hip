@@ -22,25 +22,11 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-#include <type_traits>
-
+#include "fdb_device.h"
 #include "fdb_kernels.h"
 #include "../../include/fdb.h"
 
-typedef __attribute__((ext_vector_type(16))) float f32x16;
-typedef __attribute__((ext_vector_type(8))) float f32x8;
-typedef __attribute__((ext_vector_type(4))) float f32x4;
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
-typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
-typedef __attribute__((ext_vector_type(4))) _Float16 f16x4;
-typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
-typedef __attribute__((ext_vector_type(4))) short s16x4;
-typedef __attribute__((ext_vector_type(8))) short s16x8;
-typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
-
-#define LDS_AS __attribute__((address_space(3)))
+using namespace fdb;
 
 namespace {
 
@@ -50,159 +36,7 @@ constexpr int kC2pRows = 96;     // 32 + 64 - 1 relative positions per wave tile
 constexpr int kC2pStride = 100;  // elements per query row of the wave's C[i][r] scratch
 constexpr int kP2cRows = 192;    // 128 + 64 - 1 per workgroup tile, padded to 6 MFMA blocks
 constexpr int kP2cStride = 196;  // elements per key row of the workgroup's P[j][r] scratch
-constexpr float kLazyTau = 8.f;  // the running reference point of a row is moved only when the tile
-                                 // maximum exceeds it by more than 2^8 (any reference point is valid)
 
-// ---- element traits --------------------------------------------------------------------------
-// frag: the 8 contraction elements one lane feeds to a K=16 step (lane = outer index l%32, the
-// elements are k = 16*step + 8*(l/32) + 0..7).
-struct Bf16Tr {
-  static constexpr int SZ = 2;
-  using frag = bf16x8;
-  using scratch_t = __bf16;
-  static __device__ __forceinline__ frag zero() { return frag{0, 0, 0, 0, 0, 0, 0, 0}; }
-  static __device__ __forceinline__ frag load(const void* p) { return *(const frag*)p; }
-  static __device__ __forceinline__ f32x16 mma(frag a, frag b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ f32x8 to_f32(frag x) { return __builtin_convertvector(x, f32x8); }
-  static __device__ __forceinline__ frag from_f32(f32x8 x) { return __builtin_convertvector(x, frag); }
-  // sum of the 8 elements (as rounded to the operand type) accumulated onto acc
-  static __device__ __forceinline__ float sum8(frag x, float acc) {
-    const bf16x2 one = {(__bf16)1.0f, (__bf16)1.0f};
-#pragma unroll
-    for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_fdot2_f32_bf16(bf16x2{x[2 * e], x[2 * e + 1]}, one, acc, false);
-    return acc;
-  }
-  static __device__ __forceinline__ void store4(char* p, float a, float b, float c, float d) {
-    f32x4 x = {a, b, c, d};
-    *(bf16x4*)p = __builtin_convertvector(x, bf16x4);
-  }
-};
-
-struct F16Tr {
-  static constexpr int SZ = 2;
-  using frag = f16x8;
-  using scratch_t = _Float16;
-  static __device__ __forceinline__ frag zero() { return frag{0, 0, 0, 0, 0, 0, 0, 0}; }
-  static __device__ __forceinline__ frag load(const void* p) { return *(const frag*)p; }
-  static __device__ __forceinline__ f32x16 mma(frag a, frag b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ f32x8 to_f32(frag x) { return __builtin_convertvector(x, f32x8); }
-  static __device__ __forceinline__ frag from_f32(f32x8 x) { return __builtin_convertvector(x, frag); }
-  static __device__ __forceinline__ float sum8(frag x, float acc) {
-    const f16x2 one = {(_Float16)1.0f, (_Float16)1.0f};
-#pragma unroll
-    for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_fdot2(f16x2{x[2 * e], x[2 * e + 1]}, one, acc, false);
-    return acc;
-  }
-  static __device__ __forceinline__ void store4(char* p, float a, float b, float c, float d) {
-    f32x4 x = {a, b, c, d};
-    *(f16x4*)p = __builtin_convertvector(x, f16x4);
-  }
-};
-
-struct F32Tr {
-  static constexpr int SZ = 4;
-  using frag = f32x8;
-  using scratch_t = float;
-  static __device__ __forceinline__ frag zero() { return frag{0, 0, 0, 0, 0, 0, 0, 0}; }
-  static __device__ __forceinline__ frag load(const void* p) { return *(const frag*)p; }
-  // A K=16 step in fp32 is eight K=2 MFMAs; lane group g supplies k = 16*step + 8*g + e to the e-th.
-  static __device__ __forceinline__ f32x16 mma(frag a, frag b, f32x16 c) {
-#pragma unroll
-    for (int e = 0; e < 8; ++e) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], b[e], c, 0, 0, 0);
-    return c;
-  }
-  static __device__ __forceinline__ f32x8 to_f32(frag x) { return x; }
-  static __device__ __forceinline__ frag from_f32(f32x8 x) { return x; }
-  static __device__ __forceinline__ float sum8(frag x, float acc) {
-#pragma unroll
-    for (int e = 0; e < 8; ++e) acc += x[e];
-    return acc;
-  }
-  static __device__ __forceinline__ void store4(char* p, float a, float b, float c, float d) {
-    *(f32x4*)p = f32x4{a, b, c, d};
-  }
-};
-
-struct Fp8Tr {  // OCP e4m3, operands of the three score products only
-  static constexpr int SZ = 1;
-  using frag = long;
-  using scratch_t = __bf16;
-  static __device__ __forceinline__ frag zero() { return 0; }
-  static __device__ __forceinline__ frag load(const void* p) { return *(const long*)p; }
-  static __device__ __forceinline__ f32x16 mma(frag a, frag b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a, b, c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ f32x8 to_f32(frag) { return f32x8{0, 0, 0, 0, 0, 0, 0, 0}; }  // unused
-  static __device__ __forceinline__ frag from_f32(f32x8) { return 0; }                             // unused
-};
-
-// V^T operand of a K=16 step: lane (d = l%32, g = l/32) needs V[j(g,e)][d] for
-// j(g,e) = 16*c + 8*(e/4) + 4*g + e%4 -- the key rows whose probabilities sit in this lane
-// group's accumulator registers.  V stays row-major in LDS.
-template <class VT>
-struct VtLoad;
-
-template <>
-struct VtLoad<F32Tr> {
-  static __device__ __forceinline__ f32x8 get(const char* vs, int rs, int c, int db, int lane) {
-    const int li = lane & 31, g = lane >> 5;
-    f32x8 r;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const int row = 16 * c + 8 * (e >> 2) + 4 * g + (e & 3);
-      r[e] = *(const float*)(vs + row * rs + (db * 32 + li) * 4);
-    }
-    return r;
-  }
-};
-
-// 16-bit: ds_read_tr16_b64.  Within each group of 16 lanes, source lane s supplies an 8-byte
-// address; destination lane i receives element (i%4) of source lanes 4*r + i/4, r = 0..3.
-// With source lane s pointing at V[row0 + s/4][col0 + 4*(s%4) ..+3], lane i gets column
-// col0 + i of rows row0 .. row0+3.
-template <class VT>
-struct VtLoad16 {
-  static __device__ __forceinline__ typename VT::frag get(const char* vs, int rs, int c, int db, int lane) {
-    const int s = lane & 15, grp = lane >> 4;
-    const int row = 16 * c + 4 * (grp >> 1) + (s >> 2);
-    const int col = db * 32 + 16 * (grp & 1) + 4 * (s & 3);
-    const char* a = vs + row * rs + col * 2;
-    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(a));
-    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(a + 8 * rs));
-    s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    return __builtin_bit_cast(typename VT::frag, both);
-  }
-};
-template <>
-struct VtLoad<Bf16Tr> : VtLoad16<Bf16Tr> {};
-template <>
-struct VtLoad<F16Tr> : VtLoad16<F16Tr> {};
-
-// combine lane l with lane l^32 (the other half of the row's keys)
-// v_permlane32_swap exchanges lanes 32..63 of its first operand with lanes 0..31 of its second.
-// Fed two registers holding the same value, every lane ends up with its own value in one register
-// and its partner's (lane ^ 32) in the other.  Written as one asm block: the two operands must be
-// distinct registers, and the results must stay opaque to the optimiser.
-__device__ __forceinline__ void half_pair(float x, float& r0, float& r1) {
-  float a = x, b;
-  asm volatile("v_mov_b32 %1, %0\n\ts_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "=&v"(b));
-  r0 = a;
-  r1 = b;
-}
-__device__ __forceinline__ float wave_half_max(float x) {
-  float a, b;
-  half_pair(x, a, b);
-  return fmaxf(a, b);
-}
-__device__ __forceinline__ float wave_half_sum(float x) {
-  float a, b;
-  half_pair(x, a, b);
-  return a + b;
-}
 
 template <class QT, class VT, int D>
 struct Cfg {
@@ -221,23 +55,6 @@ struct Cfg {
     return K_BYTES + V_BYTES + (c2p ? C2P_BYTES : 0) + (p2c ? P2C_BYTES : 0);
   }
 };
-
-template <class ST>
-__device__ __forceinline__ void store4_scratch(ST* p, float a, float b, float c, float d);
-template <>
-__device__ __forceinline__ void store4_scratch<float>(float* p, float a, float b, float c, float d) {
-  *(f32x4*)p = f32x4{a, b, c, d};
-}
-template <>
-__device__ __forceinline__ void store4_scratch<__bf16>(__bf16* p, float a, float b, float c, float d) {
-  f32x4 x = {a, b, c, d};
-  *(bf16x4*)p = __builtin_convertvector(x, bf16x4);
-}
-template <>
-__device__ __forceinline__ void store4_scratch<_Float16>(_Float16* p, float a, float b, float c, float d) {
-  f32x4 x = {a, b, c, d};
-  *(f16x4*)p = __builtin_convertvector(x, f16x4);
-}
 
 // [64 x ROW_BYTES] tile: global -> registers -> LDS.  Rows past the end of the sequence re-read the
 // last valid row (finite data, no predication); their scores are masked to -inf before the soft-max.
@@ -316,11 +133,16 @@ __device__ __forceinline__ void softmax_pv(f32x16 (&sacc)[2], f32x16 (&o_acc)[D 
 }
 
 // Two workgroups share a CU (and its 512 registers per lane) when the LDS footprint allows it.
-template <class QT, class VT, int D, bool C2P, bool P2C>
-constexpr int min_blocks() { return Cfg<QT, VT, D>::lds_bytes(C2P, P2C) <= 80 * 1024 ? 2 : 1; }
+template <class QT, class VT, int D, bool C2P, bool P2C, bool FAR_ONLY>
+constexpr int min_blocks() {
+  const int lds = FAR_ONLY ? Cfg<QT, VT, D>::lds_bytes(false, false) : Cfg<QT, VT, D>::lds_bytes(C2P, P2C);
+  return lds <= 40 * 1024 ? 4 : lds <= 80 * 1024 ? 2 : 1;
+}
 
-template <class QT, class VT, int D, bool FP8, bool C2P, bool P2C>
-__global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C>())) void fdb_attn_kernel(const FdbKParams p) {
+// FAR_ONLY: the near tiles are left to the near kernel; this one writes the far tiles' partial
+// result (rows normalised over the far keys, their log-sum-exp, zero / -inf where there is none).
+template <class QT, class VT, int D, bool FP8, bool C2P, bool P2C, bool FAR_ONLY>
+__global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, FAR_ONLY>())) void fdb_attn_kernel(const FdbKParams p) {
   using C = Cfg<QT, VT, D>;
   using ST = typename C::ST;
   using qfrag = typename QT::frag;
@@ -426,18 +248,28 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C>())) void
     for (int v = 0; v < 16; ++v) o_acc[d][v] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;  // l_run: this lane's half of the row sum
 
+  // the tile walked after tile t (far-only runs jump over the near range)
+  auto next_tile = [&](int t) __attribute__((always_inline)) {
+    return (FAR_ONLY && t + 1 >= t_near0 && t + 1 < t_near1) ? t_near1 : t + 1;
+  };
   u32x4 kreg[C::K_CHUNKS], vreg[C::V_CHUNKS];
-  tile_load<D * QT::SZ>(kreg, kb, k_rsb, 0, Lb, tid);
-  tile_load<D * VT::SZ>(vreg, vb, v_rsb, 0, Lb, tid);
+  {
+    const int first = next_tile(-1);
+    if (first < n_tiles) {
+      tile_load<D * QT::SZ>(kreg, kb, k_rsb, first * FDB_BN, Lb, tid);
+      tile_load<D * VT::SZ>(vreg, vb, v_rsb, first * FDB_BN, Lb, tid);
+    }
+  }
 
   auto stage = [&](int t) __attribute__((always_inline)) {
     __syncthreads();  // every wave is done with the previous tile and its bias scratch
     tile_store<D * QT::SZ, C::K_RS>(Ks, kreg, tid);
     tile_store<D * VT::SZ, C::V_RS>(Vs, vreg, tid);
     __syncthreads();
-    if (t + 1 < n_tiles) {  // next tile's global loads fly during this tile's math
-      tile_load<D * QT::SZ>(kreg, kb, k_rsb, (t + 1) * FDB_BN, Lb, tid);
-      tile_load<D * VT::SZ>(vreg, vb, v_rsb, (t + 1) * FDB_BN, Lb, tid);
+    const int nt = next_tile(t);
+    if (nt < n_tiles) {  // next tile's global loads fly during this tile's math
+      tile_load<D * QT::SZ>(kreg, kb, k_rsb, nt * FDB_BN, Lb, tid);
+      tile_load<D * VT::SZ>(vreg, vb, v_rsb, nt * FDB_BN, Lb, tid);
     }
   };
   auto qk = [&](f32x16 (&sacc)[2], const qfrag (&qq)[C::KSTEPS]) __attribute__((always_inline)) {
@@ -477,7 +309,7 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C>())) void
   far_range(0, t_near0, 0);
 
   // ---- near ----------------------------------------------------------------------------------
-  if constexpr (kHasPos) {
+  if constexpr (kHasPos && !FAR_ONLY) {
     // Row offsets (bytes) into K_r / Q_r of the A rows this lane feeds to the position products
     // of one tile; looked up through the table one tile ahead so that the row loads of a tile
     // never wait for the table.
@@ -606,11 +438,11 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C>())) void
   }
 }
 
-template <class QT, class VT, int D, bool FP8, bool C2P, bool P2C>
+template <class QT, class VT, int D, bool FP8, bool C2P, bool P2C, bool FAR_ONLY>
 int launch_one(const FdbKParams& p, int grid_x, hipStream_t stream) {
   using C = Cfg<QT, VT, D>;
-  auto kern = fdb_attn_kernel<QT, VT, D, FP8, C2P, P2C>;
-  constexpr int lds = C::lds_bytes(C2P, P2C);
+  auto kern = fdb_attn_kernel<QT, VT, D, FP8, C2P, P2C, FAR_ONLY>;
+  constexpr int lds = FAR_ONLY ? C::lds_bytes(false, false) : C::lds_bytes(C2P, P2C);
   static_assert(lds <= 160 * 1024, "LDS budget");
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
   if (e != hipSuccess) return (int)e;
@@ -619,22 +451,30 @@ int launch_one(const FdbKParams& p, int grid_x, hipStream_t stream) {
 }
 
 template <class QT, class VT, int D, bool FP8>
-int launch_pos(const FdbKParams& p, int grid_x, hipStream_t stream) {
-  if (p.pk && p.pq) return launch_one<QT, VT, D, FP8, true, true>(p, grid_x, stream);
-  if (p.pk) return launch_one<QT, VT, D, FP8, true, false>(p, grid_x, stream);
-  if (p.pq) return launch_one<QT, VT, D, FP8, false, true>(p, grid_x, stream);
-  return launch_one<QT, VT, D, FP8, false, false>(p, grid_x, stream);
+int launch_pos(const FdbKParams& p, int grid_x, bool far_only, hipStream_t stream) {
+  if constexpr (!FP8 && QT::SZ == 2 && D <= 64) {  // the combinations the near kernel covers
+    if (far_only) {
+      if (p.pk && p.pq) return launch_one<QT, VT, D, FP8, true, true, true>(p, grid_x, stream);
+      if (p.pk) return launch_one<QT, VT, D, FP8, true, false, true>(p, grid_x, stream);
+      return launch_one<QT, VT, D, FP8, false, true, true>(p, grid_x, stream);
+    }
+  }
+  if (far_only) return FDB_ERR_UNSUPPORTED;
+  if (p.pk && p.pq) return launch_one<QT, VT, D, FP8, true, true, false>(p, grid_x, stream);
+  if (p.pk) return launch_one<QT, VT, D, FP8, true, false, false>(p, grid_x, stream);
+  if (p.pq) return launch_one<QT, VT, D, FP8, false, true, false>(p, grid_x, stream);
+  return launch_one<QT, VT, D, FP8, false, false, false>(p, grid_x, stream);
 }
 
 }  // namespace
 
-int fdb_launch_attn(const FdbKParams& p, int dtype, int head_dim, int grid_x, void* stream_) {
+int fdb_launch_attn(const FdbKParams& p, int dtype, int head_dim, int grid_x, bool far_only, void* stream_) {
   hipStream_t stream = (hipStream_t)stream_;
 #define FDB_DISPATCH_D(QT, VT, FP8)                                   \
   switch (head_dim) {                                                 \
-    case 32: return launch_pos<QT, VT, 32, FP8>(p, grid_x, stream);   \
-    case 64: return launch_pos<QT, VT, 64, FP8>(p, grid_x, stream);   \
-    case 128: return launch_pos<QT, VT, 128, FP8>(p, grid_x, stream); \
+    case 32: return launch_pos<QT, VT, 32, FP8>(p, grid_x, far_only, stream);   \
+    case 64: return launch_pos<QT, VT, 64, FP8>(p, grid_x, far_only, stream);   \
+    case 128: return launch_pos<QT, VT, 128, FP8>(p, grid_x, far_only, stream); \
     default: return FDB_ERR_HEAD_DIM;                                 \
   }
   switch (dtype) {
@@ -642,8 +482,8 @@ int fdb_launch_attn(const FdbKParams& p, int dtype, int head_dim, int grid_x, vo
     case FDB_F16: FDB_DISPATCH_D(F16Tr, F16Tr, false)
     case FDB_F32:
       switch (head_dim) {
-        case 32: return launch_pos<F32Tr, F32Tr, 32, false>(p, grid_x, stream);
-        case 64: return launch_pos<F32Tr, F32Tr, 64, false>(p, grid_x, stream);
+        case 32: return launch_pos<F32Tr, F32Tr, 32, false>(p, grid_x, far_only, stream);
+        case 64: return launch_pos<F32Tr, F32Tr, 64, false>(p, grid_x, far_only, stream);
         default: return FDB_ERR_UNSUPPORTED;
       }
     case FDB_FP8_E4M3: FDB_DISPATCH_D(Fp8Tr, Bf16Tr, true)

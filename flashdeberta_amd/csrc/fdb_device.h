@@ -1,0 +1,228 @@
+// Device-side building blocks shared by the attention kernels: vector typedefs, element traits
+// (MFMA operand fragments per dtype), the V^T operand loader and the half-wave exchange.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <type_traits>
+
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(8))) float f32x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(4))) _Float16 f16x4;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(8))) short s16x8;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+
+#define LDS_AS __attribute__((address_space(3)))
+
+namespace fdb {
+
+constexpr float kLazyTau = 8.f;  // the running reference point of a row is moved only when the tile
+                                 // maximum exceeds it by more than 2^8 (any reference point is valid)
+
+// ---- element traits --------------------------------------------------------------------------
+// frag: the 8 contraction elements one lane feeds to a K=16 step (lane = outer index l%32, the
+// elements are k = 16*step + 8*(l/32) + 0..7).
+struct Bf16Tr {
+  static constexpr int SZ = 2;
+  using frag = bf16x8;
+  using scratch_t = __bf16;
+  static __device__ __forceinline__ frag zero() { return frag{0, 0, 0, 0, 0, 0, 0, 0}; }
+  static __device__ __forceinline__ frag load(const void* p) { return *(const frag*)p; }
+  static __device__ __forceinline__ f32x16 mma(frag a, frag b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x8 to_f32(frag x) { return __builtin_convertvector(x, f32x8); }
+  static __device__ __forceinline__ frag from_f32(f32x8 x) { return __builtin_convertvector(x, frag); }
+  // sum of the 8 elements (as rounded to the operand type) accumulated onto acc
+  static __device__ __forceinline__ float sum8(frag x, float acc) {
+    const bf16x2 one = {(__bf16)1.0f, (__bf16)1.0f};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_fdot2_f32_bf16(bf16x2{x[2 * e], x[2 * e + 1]}, one, acc, false);
+    return acc;
+  }
+  static __device__ __forceinline__ void store4(char* p, float a, float b, float c, float d) {
+    f32x4 x = {a, b, c, d};
+    *(bf16x4*)p = __builtin_convertvector(x, bf16x4);
+  }
+  static __device__ __forceinline__ f32x4 load4(const char* p) { return __builtin_convertvector(*(const bf16x4*)p, f32x4); }
+};
+
+struct F16Tr {
+  static constexpr int SZ = 2;
+  using frag = f16x8;
+  using scratch_t = _Float16;
+  static __device__ __forceinline__ frag zero() { return frag{0, 0, 0, 0, 0, 0, 0, 0}; }
+  static __device__ __forceinline__ frag load(const void* p) { return *(const frag*)p; }
+  static __device__ __forceinline__ f32x16 mma(frag a, frag b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x8 to_f32(frag x) { return __builtin_convertvector(x, f32x8); }
+  static __device__ __forceinline__ frag from_f32(f32x8 x) { return __builtin_convertvector(x, frag); }
+  static __device__ __forceinline__ float sum8(frag x, float acc) {
+    const f16x2 one = {(_Float16)1.0f, (_Float16)1.0f};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_fdot2(f16x2{x[2 * e], x[2 * e + 1]}, one, acc, false);
+    return acc;
+  }
+  static __device__ __forceinline__ void store4(char* p, float a, float b, float c, float d) {
+    f32x4 x = {a, b, c, d};
+    *(f16x4*)p = __builtin_convertvector(x, f16x4);
+  }
+  static __device__ __forceinline__ f32x4 load4(const char* p) { return __builtin_convertvector(*(const f16x4*)p, f32x4); }
+};
+
+struct F32Tr {
+  static constexpr int SZ = 4;
+  using frag = f32x8;
+  using scratch_t = float;
+  static __device__ __forceinline__ frag zero() { return frag{0, 0, 0, 0, 0, 0, 0, 0}; }
+  static __device__ __forceinline__ frag load(const void* p) { return *(const frag*)p; }
+  // A K=16 step in fp32 is eight K=2 MFMAs; lane group g supplies k = 16*step + 8*g + e to the e-th.
+  static __device__ __forceinline__ f32x16 mma(frag a, frag b, f32x16 c) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], b[e], c, 0, 0, 0);
+    return c;
+  }
+  static __device__ __forceinline__ f32x8 to_f32(frag x) { return x; }
+  static __device__ __forceinline__ frag from_f32(f32x8 x) { return x; }
+  static __device__ __forceinline__ float sum8(frag x, float acc) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc += x[e];
+    return acc;
+  }
+  static __device__ __forceinline__ void store4(char* p, float a, float b, float c, float d) {
+    *(f32x4*)p = f32x4{a, b, c, d};
+  }
+  static __device__ __forceinline__ f32x4 load4(const char* p) { return *(const f32x4*)p; }
+};
+
+struct Fp8Tr {  // OCP e4m3, operands of the three score products only
+  static constexpr int SZ = 1;
+  using frag = long;
+  using scratch_t = __bf16;
+  static __device__ __forceinline__ frag zero() { return 0; }
+  static __device__ __forceinline__ frag load(const void* p) { return *(const long*)p; }
+  static __device__ __forceinline__ f32x16 mma(frag a, frag b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x8 to_f32(frag) { return f32x8{0, 0, 0, 0, 0, 0, 0, 0}; }  // unused
+  static __device__ __forceinline__ frag from_f32(f32x8) { return 0; }                             // unused
+};
+
+// V^T operand of a K=16 step: lane (d = l%32, g = l/32) needs V[j(g,e)][d] for
+// j(g,e) = 16*c + 8*(e/4) + 4*g + e%4 -- the key rows whose probabilities sit in this lane
+// group's accumulator registers.  V stays row-major in LDS.
+template <class VT>
+struct VtLoad;
+
+template <>
+struct VtLoad<F32Tr> {
+  static __device__ __forceinline__ f32x8 get(const char* vs, int rs, int c, int db, int lane) {
+    const int li = lane & 31, g = lane >> 5;
+    f32x8 r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int row = 16 * c + 8 * (e >> 2) + 4 * g + (e & 3);
+      r[e] = *(const float*)(vs + row * rs + (db * 32 + li) * 4);
+    }
+    return r;
+  }
+};
+
+// 16-bit: ds_read_tr16_b64.  Within each group of 16 lanes, source lane s supplies an 8-byte
+// address; destination lane i receives element (i%4) of source lanes 4*r + i/4, r = 0..3.
+// With source lane s pointing at V[row0 + s/4][col0 + 4*(s%4) ..+3], lane i gets column
+// col0 + i of rows row0 .. row0+3.
+template <class VT>
+struct VtLoad16 {
+  static __device__ __forceinline__ typename VT::frag get(const char* vs, int rs, int c, int db, int lane) {
+    const int s = lane & 15, grp = lane >> 4;
+    const int row = 16 * c + 4 * (grp >> 1) + (s >> 2);
+    const int col = db * 32 + 16 * (grp & 1) + 4 * (s & 3);
+    const char* a = vs + row * rs + col * 2;
+    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(a));
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(a + 8 * rs));
+    s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(typename VT::frag, both);
+  }
+};
+template <>
+struct VtLoad<Bf16Tr> : VtLoad16<Bf16Tr> {};
+template <>
+struct VtLoad<F16Tr> : VtLoad16<F16Tr> {};
+
+// combine lane l with lane l^32 (the other half of the row's keys)
+// v_permlane32_swap exchanges lanes 32..63 of its first operand with lanes 0..31 of its second.
+// Fed two registers holding the same value, every lane ends up with its own value in one register
+// and its partner's (lane ^ 32) in the other.  Written as one asm block: the two operands must be
+// distinct registers, and the results must stay opaque to the optimiser.
+__device__ __forceinline__ void half_pair(float x, float& r0, float& r1) {
+  float a = x, b;
+  asm volatile("v_mov_b32 %1, %0\n\ts_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "=&v"(b));
+  r0 = a;
+  r1 = b;
+}
+__device__ __forceinline__ float wave_half_max(float x) {
+  float a, b;
+  half_pair(x, a, b);
+  return fmaxf(a, b);
+}
+__device__ __forceinline__ float wave_half_sum(float x) {
+  float a, b;
+  half_pair(x, a, b);
+  return a + b;
+}
+
+
+template <class ST>
+__device__ __forceinline__ void store4_scratch(ST* p, float a, float b, float c, float d);
+template <>
+__device__ __forceinline__ void store4_scratch<float>(float* p, float a, float b, float c, float d) {
+  *(f32x4*)p = f32x4{a, b, c, d};
+}
+template <>
+__device__ __forceinline__ void store4_scratch<__bf16>(__bf16* p, float a, float b, float c, float d) {
+  f32x4 x = {a, b, c, d};
+  *(bf16x4*)p = __builtin_convertvector(x, bf16x4);
+}
+template <>
+__device__ __forceinline__ void store4_scratch<_Float16>(_Float16* p, float a, float b, float c, float d) {
+  f32x4 x = {a, b, c, d};
+  *(f16x4*)p = __builtin_convertvector(x, f16x4);
+}
+
+// Four consecutive scratch elements from an address aligned only to the element size (gfx950
+// serves unaligned DS accesses), as fp32.
+template <class ST>
+__device__ __forceinline__ f32x4 load4_scratch_unaligned(const ST* p);
+template <>
+__device__ __forceinline__ f32x4 load4_scratch_unaligned<float>(const float* p) {
+  typedef f32x4 __attribute__((aligned(4))) f32x4_u;
+  return *(const f32x4_u*)p;
+}
+template <>
+__device__ __forceinline__ f32x4 load4_scratch_unaligned<__bf16>(const __bf16* p) {
+  typedef bf16x4 __attribute__((aligned(2))) bf16x4_u;
+  return __builtin_convertvector(*(const bf16x4_u*)p, f32x4);
+}
+template <>
+__device__ __forceinline__ f32x4 load4_scratch_unaligned<_Float16>(const _Float16* p) {
+  typedef f16x4 __attribute__((aligned(2))) f16x4_u;
+  return __builtin_convertvector(*(const f16x4_u*)p, f32x4);
+}
+
+// Orders this wave's earlier LDS accesses before its later ones (the LDS unit executes one wave's
+// operations in order; this only stops the compiler from moving them across).
+__device__ __forceinline__ void wave_lds_fence() {
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+}
+
+}  // namespace fdb

@@ -32,14 +32,20 @@ struct FdbKParams {
   int64_t pq_sh, pq_sr;
   int32_t B, H, L, tiles_per_seq;
   int32_t R;        // LUT radius
-  int32_t r_neg;    // delta(r) == delta(-R) for every r <= r_neg
-  int32_t r_pos;    // delta(r) == delta(+R) for every r >= r_pos
+  int32_t far_done; // near kernel only: the far tiles' partial result is already in out / lse
   int32_t causal;
   float scale_log2; // sm_scale * log2(e)
 };
 
 // Launchers return the hipError_t of the launch as int.
-int fdb_launch_attn(const FdbKParams& p, int dtype, int head_dim, int grid_x, void* stream);
+// fdb_launch_attn: one kernel walks every key tile.  far_only: it skips the near tiles and leaves
+// the far tiles' partial result (normalised rows in out, their log-sum-exp in lse, -inf where a row
+// has no far tile) for fdb_launch_near to merge.
+int fdb_launch_attn(const FdbKParams& p, int dtype, int head_dim, int grid_x, bool far_only, void* stream);
+// fdb_launch_near: the near tiles only (expanded relative-embedding rows staged in LDS rings),
+// merged with the far partial when p.far_done.  16-bit element types with head_dim <= 64.
+bool fdb_near_supported(int dtype, int head_dim);
+int fdb_launch_near(const FdbKParams& p, int dtype, int head_dim, int grid_x, void* stream);
 int fdb_launch_worklist(const int32_t* cu, int32_t batch, int32_t* wl, int32_t max_tiles, void* stream);
 int fdb_launch_quant(const void* x, int64_t x_st, int64_t x_sh, void* y, int64_t y_st, int64_t y_sh,
                      float* scale, uint32_t* absmax_ws, int32_t tokens, int32_t heads, int32_t head_dim,

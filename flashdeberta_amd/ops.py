@@ -139,7 +139,10 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
         out = torch.empty(q.shape, dtype=v.dtype, device=q.device)
     elif out.shape != q.shape or out.dtype != v.dtype or out.stride(-1) != 1:
         raise ValueError("out must have q's shape, v's dtype and a unit stride on D")
-    lse = torch.empty((T, H), dtype=torch.float32, device=q.device) if return_lse else None
+    # the log-sum-exp buffer is also the hand-over between the far-tile and near-tile launches, so it is
+    # always provided when a position term is present (T*H floats)
+    want_lse = return_lse or pos_key is not None or pos_query is not None
+    lse = torch.empty((T, H), dtype=torch.float32, device=q.device) if want_lse else None
     a.q, a.k, a.v, a.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
     a.pos_key, a.pos_query = (_ptr(pos_key) or ctypes.c_void_p()).value, (_ptr(pos_query) or ctypes.c_void_p()).value
     a.lse = lse.data_ptr() if lse is not None else None
