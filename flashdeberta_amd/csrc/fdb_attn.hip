@@ -136,6 +136,7 @@ __device__ __forceinline__ void softmax_pv(f32x16 (&sacc)[2], f32x16 (&o_acc)[D 
 template <class QT, class VT, int D, bool C2P, bool P2C, bool FAR_ONLY>
 constexpr int min_blocks() {
   const int lds = FAR_ONLY ? Cfg<QT, VT, D>::lds_bytes(false, false) : Cfg<QT, VT, D>::lds_bytes(C2P, P2C);
+  if (FAR_ONLY) return 3;  // the far zones need the shifted query and the per-row constants on top of the plain kernel
   return lds <= 40 * 1024 ? 4 : lds <= 80 * 1024 ? 2 : 1;
 }
 
