@@ -72,6 +72,18 @@ def make_inputs(name, device):
     return (q, k, v, pk, pq), kw, out, lens
 
 
+def measured_traffic(workload):
+    """HBM bytes per step as measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), scaled by the
+    copy-calibration kernel; recorded in profiles/hbm_traffic.json by hand from those runs.  None if
+    the workload has not been measured."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get(workload, {}).get("bytes_per_step")
+    except (OSError, ValueError):
+        return None
+
+
 def cpu_baseline(H, D, L):
     """The CPU oracle (numpy restatement of the eager path, fp32) on a bounded sample of the same
     workload: one batch element, as many heads as fit in roughly 10-30 s."""
@@ -107,6 +119,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="v3base_L4096_B8_bf16", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
+                    help="also run one device-to-device copy of this many MiB (a kernel of known HBM traffic "
+                         "against which rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures ONE GPU only (the path is independent per (sequence, head, "
@@ -120,6 +135,10 @@ def main():
     B, L, H, D, dt, kind = WORKLOADS[args.workload]
     tensors, kw, out, lens = make_inputs(args.workload, device)
     step = lambda: ops.disentangled_attention_fwd(*tensors, out=out, **kw)
+    if args.copy_calibration:
+        src = torch.empty(args.copy_calibration << 20, dtype=torch.uint8, device=device)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -148,7 +167,7 @@ def main():
         "config": {"workload": args.workload, "batch": B, "seq_len": L if kind == "fixed" else "varlen(%d tokens)" % tokens,
                    "heads": H, "head_dim": D, "position_buckets": 256, "pos_att_type": "c2p|p2c", "layout": kind},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": round(peak, 1), "unit": "TFLOP/s",
-                     "frac": round(achieved / peak, 4), "traffic": None,
+                     "frac": round(achieved / peak, 4), "traffic": measured_traffic(args.workload),
                      "kernel_ms": round(kern_ms, 4), "algorithmic_gflop_per_launch": round(fl / 1e9, 2)},
     }
     if not args.no_cpu:

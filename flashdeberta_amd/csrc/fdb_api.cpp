@@ -171,7 +171,8 @@ int fdb_attn_fwd(const fdb_attn_args* a, void* stream) {
   p.scale_log2 = a->sm_scale * 1.4426950408889634f;
   int64_t grid_x = a->cu_seqlens ? fdb_worklist_max_tiles(a->total_tokens, a->batch)
                                  : (int64_t)a->batch * p.tiles_per_seq;
-  if (grid_x < 1 || grid_x > INT32_MAX) return FDB_ERR_SHAPE;
+  if (grid_x < 1 || grid_x * a->heads > INT32_MAX) return FDB_ERR_SHAPE;
+  p.grid_x = (int32_t)grid_x;
   // Split path: the far tiles in a far-only run of the fused kernel (lean, four workgroups per
   // CU), the near tiles in the near kernel, which merges the two.  It needs the log-sum-exp buffer
   // as the hand-over between the two launches.

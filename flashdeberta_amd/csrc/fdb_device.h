@@ -218,6 +218,23 @@ __device__ __forceinline__ f32x4 load4_scratch_unaligned<_Float16>(const _Float1
   return __builtin_convertvector(*(const f16x4_u*)p, f32x4);
 }
 
+// Linear workgroup id -> (query-tile index within the launch, head).  The hardware deals
+// workgroups to the 8 XCDs round-robin by linear id, and each XCD has its own L2.  In the fixed
+// layout, when the number of (sequence, head) groups is a multiple of 8, groups are dealt to XCDs
+// whole: all query tiles of a group then stream the same K and V through one L2.
+__device__ __forceinline__ void block_map(int n, int nx, int heads, int tiles_per_seq, bool fixed, int& xq, int& h) {
+  const int groups = fixed ? (nx / tiles_per_seq) * heads : 1;
+  if (fixed && (groups & 7) == 0) {
+    const int xcd = n & 7, slot = n >> 3;
+    const int grp = xcd + 8 * (slot / tiles_per_seq);
+    xq = (grp / heads) * tiles_per_seq + slot % tiles_per_seq;
+    h = grp % heads;
+  } else {
+    xq = n % nx;
+    h = n / nx;
+  }
+}
+
 // Orders this wave's earlier LDS accesses before its later ones (the LDS unit executes one wave's
 // operations in order; this only stops the compiler from moving them across).
 __device__ __forceinline__ void wave_lds_fence() {

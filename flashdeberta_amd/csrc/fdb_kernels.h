@@ -31,6 +31,7 @@ struct FdbKParams {
   int64_t pk_sh, pk_sr;
   int64_t pq_sh, pq_sr;
   int32_t B, H, L, tiles_per_seq;
+  int32_t grid_x;   // query tiles in the launch (the grid is grid_x * H workgroups)
   int32_t R;        // LUT radius
   int32_t far_done; // near kernel only: the far tiles' partial result is already in out / lse
   int32_t causal;

@@ -111,21 +111,22 @@ __global__ __launch_bounds__(kNThreads, 1) void fdb_near_kernel(const FdbKParams
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, li = lane & 31, g = lane >> 5;
   const int wr = wave & 3, wk = wave >> 2;
-  const int h = blockIdx.y;
+  int xq, h;
+  block_map((int)blockIdx.x, p.grid_x, p.H, p.tiles_per_seq, p.cu == nullptr, xq, h);
   ST* scr = (ST*)scr_raw + wave * (32 * kScrStride);
 
   int b, m0, tok0, Lb;
   int64_t qo, ko, vo, oo;
   if (p.cu) {
-    if ((int)blockIdx.x >= p.wl[0]) return;
-    b = p.wl[2 + 2 * blockIdx.x];
-    m0 = p.wl[3 + 2 * blockIdx.x];
+    if (xq >= p.wl[0]) return;
+    b = p.wl[2 + 2 * xq];
+    m0 = p.wl[3 + 2 * xq];
     tok0 = p.cu[b];
     Lb = p.cu[b + 1] - tok0;
     qo = ko = vo = oo = 0;
   } else {
-    b = blockIdx.x / p.tiles_per_seq;
-    m0 = (blockIdx.x % p.tiles_per_seq) * FDB_BM;
+    b = xq / p.tiles_per_seq;
+    m0 = (xq % p.tiles_per_seq) * FDB_BM;
     tok0 = p.seq_start ? min(max(p.seq_start[b], 0), p.L) : 0;
     Lb = p.seq_len ? min(max(p.seq_len[b], 0), p.L - tok0) : p.L;
     if (m0 >= Lb) return;
@@ -391,7 +392,7 @@ int launch_near_one(const FdbKParams& p, int grid_x, hipStream_t stream) {
   static_assert(lds <= 160 * 1024, "LDS budget");
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
   if (e != hipSuccess) return (int)e;
-  hipLaunchKernelGGL(kern, dim3(grid_x, p.H, 1), dim3(kNThreads), lds, stream, p);
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid_x * p.H, 1, 1), dim3(kNThreads), lds, stream, p);
   return (int)hipGetLastError();
 }
 
