@@ -80,7 +80,7 @@ def _pos_arg(x, H, D, span, name):
 def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seqlens=None, max_seqlen=None,
                                sm_scale=None, position_buckets=0, max_relative_positions=0, causal=False,
                                return_lse=False, seq_start=None, seq_len=None, q_scale=None, k_scale=None, pos_key_scale=None,
-                               pos_query_scale=None, out=None):
+                               pos_query_scale=None, out=None, single_kernel=False):
     """Fused forward.  Layouts (strides are free except a unit stride on D):
          fixed length : q, k, v  [B, L, H, D]   -> out [B, L, H, D] (contiguous: a free view of [B, L, H*D])
          packed varlen: q, k, v  [T, H, D] + cu_seqlens int32 [B+1] (+ max_seqlen upper bound) -> out [T, H, D]
@@ -90,6 +90,8 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
        tokens [seq_start, seq_start+seq_len); only those rows of `out` are written, so pass a zeroed `out`
        (or ignore the padded rows).  Either may be None (0 / L).
        fp8: q/k/pos_* are torch.float8_e4m3fn with float32 per-head scales; v is bfloat16.
+       single_kernel=True withholds the log-sum-exp buffer, which makes the library walk all key tiles in
+       one kernel instead of the far-tile / near-tile pair of launches (same result; for comparison).
     """
     if not q.is_cuda:
         raise RuntimeError("disentangled_attention_fwd runs on the GPU only; got device %s" % q.device)
@@ -141,7 +143,7 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
         raise ValueError("out must have q's shape, v's dtype and a unit stride on D")
     # the log-sum-exp buffer is also the hand-over between the far-tile and near-tile launches, so it is
     # always provided when a position term is present (T*H floats)
-    want_lse = return_lse or pos_key is not None or pos_query is not None
+    want_lse = return_lse or ((pos_key is not None or pos_query is not None) and not single_kernel)
     lse = torch.empty((T, H), dtype=torch.float32, device=q.device) if want_lse else None
     a.q, a.k, a.v, a.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
     a.pos_key, a.pos_query = (_ptr(pos_key) or ctypes.c_void_p()).value, (_ptr(pos_query) or ctypes.c_void_p()).value

@@ -113,6 +113,22 @@ def test_strided_inputs_and_reference_call_shape():
     _check(out, ref, TOL[torch.bfloat16])
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,L,pb,mr", [(2, 1500, 256, 512), (1, 700, 32, 64), (2, 300, 256, 512)])
+def test_one_kernel_and_two_kernel_paths_agree(dtype, B, L, pb, mr):
+    """With a log-sum-exp buffer the library runs the far tiles and the near tiles as two launches;
+    without one a single kernel walks every tile.  Both must match the oracle and each other."""
+    q, k, v, pk, pq = _inputs(B, L, 3, 64, pb, mr, dtype, 77, 1.0)
+    args = [_dev(x) for x in (q, k, v, pk, pq)]
+    kw = dict(position_buckets=pb, max_relative_positions=mr)
+    two = ops.disentangled_attention_fwd(*args, **kw)
+    one = ops.disentangled_attention_fwd(*args, single_kernel=True, **kw)
+    ref = _oracle_blhd(q, k, v, pk, pq, pb, mr)
+    _check(two, ref, TOL[dtype], "two launches")
+    _check(one, ref, TOL[dtype], "one launch")
+    assert (two.float() - one.float()).abs().max().item() <= TOL[dtype]
+
+
 # ---- delta indices are bit-exact inside the kernel ----------------------------------------------
 @pytest.mark.parametrize("pb,mr,L", [(256, 512, 1200), (32, 64, 300), (0, 40, 130)])
 @pytest.mark.parametrize("term", ["c2p", "p2c"])
