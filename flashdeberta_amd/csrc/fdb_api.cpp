@@ -2,6 +2,7 @@
 // table, and dispatch to the device launchers.  No device memory is allocated here.
 #include <math.h>
 #include <stdint.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <hip/hip_runtime_api.h>
@@ -179,13 +180,15 @@ int fdb_attn_fwd(const fdb_attn_args* a, void* stream) {
   if ((a->pos_key || a->pos_query) && a->lse && fdb_near_supported(a->dtype, a->head_dim)) {
     const bool need_far = a->max_seqlen > p.R + FDB_BN - 1;  // otherwise no tile of any query tile is far
     if (need_far) {
-      const int rc_far = fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, true, stream);
+      const int rc_far = fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, FDB_MODE_FAR_ONLY, stream);
       if (rc_far != 0) return rc_far;
     }
     p.far_done = need_far ? 1 : 0;
+    static const int near_impl = getenv("FDB_NEAR_IMPL") ? atoi(getenv("FDB_NEAR_IMPL")) : 1;
+    if (near_impl == 1) return fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, FDB_MODE_NEAR_RING, stream);
     return fdb_launch_near(p, a->dtype, a->head_dim, (int)grid_x, stream);
   }
-  return fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, false, stream);
+  return fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, FDB_MODE_FUSED, stream);
 }
 
 int fdb_build_worklist(const int32_t* cu_seqlens, int32_t batch, int32_t total_tokens, int32_t* worklist,

@@ -36,6 +36,16 @@ constexpr int kC2pRows = 96;     // 32 + 64 - 1 relative positions per wave tile
 constexpr int kC2pStride = 100;  // elements per query row of the wave's C[i][r] scratch
 constexpr int kP2cRows = 192;    // 128 + 64 - 1 per workgroup tile, padded to 6 MFMA blocks
 constexpr int kP2cStride = 196;  // elements per key row of the workgroup's P[j][r] scratch
+constexpr int kRing = 256;       // rows of a ring: the 191 relative positions of a tile + the 64 of the batch in flight
+
+// Kernel modes.  kFused: one kernel walks every tile (the rows of the position products are
+// gathered from global memory).  kFarOnly: the near tiles are left to a second launch; this one
+// writes the far tiles' partial result (rows normalised over the far keys, their log-sum-exp,
+// zero / -inf where there is none).  kNearRing: that second launch -- near tiles only, the rows
+// E_K[r] = K_r[delta(r)], E_Q[r] = Q_r[delta(r)] of the relative positions in reach staged once per
+// workgroup in two LDS rings that slide 64 positions per key tile, and the far partial merged in
+// the epilogue.
+constexpr int kFused = 0, kFarOnly = 1, kNearRing = 2;
 
 
 template <class QT, class VT, int D>
@@ -51,8 +61,13 @@ struct Cfg {
   static constexpr int V_CHUNKS = (FDB_BN * D * VT::SZ / 16 + kThreads - 1) / kThreads;
   static constexpr int C2P_BYTES = kWaves * 32 * kC2pStride * (int)sizeof(ST);
   static constexpr int P2C_BYTES = FDB_BN * kP2cStride * (int)sizeof(ST);
+  static constexpr int RING_BYTES = kRing * K_RS;  // one ring of expanded relative-embedding rows
   static constexpr int lds_bytes(bool c2p, bool p2c) {
     return K_BYTES + V_BYTES + (c2p ? C2P_BYTES : 0) + (p2c ? P2C_BYTES : 0);
+  }
+  static constexpr int lds_bytes_mode(int mode, bool c2p, bool p2c) {
+    return mode == 1 ? lds_bytes(false, false)
+                     : lds_bytes(c2p, p2c) + (mode == 2 ? (c2p ? RING_BYTES : 0) + (p2c ? RING_BYTES : 0) : 0);
   }
 };
 
@@ -133,25 +148,28 @@ __device__ __forceinline__ void softmax_pv(f32x16 (&sacc)[2], f32x16 (&o_acc)[D 
 }
 
 // Two workgroups share a CU (and its 512 registers per lane) when the LDS footprint allows it.
-template <class QT, class VT, int D, bool C2P, bool P2C, bool FAR_ONLY>
+template <class QT, class VT, int D, bool C2P, bool P2C, int MODE>
 constexpr int min_blocks() {
-  const int lds = FAR_ONLY ? Cfg<QT, VT, D>::lds_bytes(false, false) : Cfg<QT, VT, D>::lds_bytes(C2P, P2C);
-  if (FAR_ONLY) return 3;  // the far zones need the shifted query and the per-row constants on top of the plain kernel
+  const int lds = Cfg<QT, VT, D>::lds_bytes_mode(MODE, C2P, P2C);
+  if (MODE == kFarOnly) return 3;  // the far zones need the shifted query and the per-row constants on top of the plain kernel
+  if (MODE == kNearRing) return 2;  // one workgroup fits a CU; the bound keeps every value in the 256 registers VALU code can read
   return lds <= 40 * 1024 ? 4 : lds <= 80 * 1024 ? 2 : 1;
 }
 
-// FAR_ONLY: the near tiles are left to the near kernel; this one writes the far tiles' partial
-// result (rows normalised over the far keys, their log-sum-exp, zero / -inf where there is none).
-template <class QT, class VT, int D, bool FP8, bool C2P, bool P2C, bool FAR_ONLY>
-__global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, FAR_ONLY>())) void fdb_attn_kernel(const FdbKParams p) {
+template <class QT, class VT, int D, bool FP8, bool C2P, bool P2C, int MODE>
+__global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())) void fdb_attn_kernel(const FdbKParams p) {
   using C = Cfg<QT, VT, D>;
   using ST = typename C::ST;
   using qfrag = typename QT::frag;
+  constexpr bool FAR_ONLY = MODE == kFarOnly, RING = MODE == kNearRing;
+  static_assert(!RING || (!FP8 && QT::SZ == 2 && (C2P || P2C)), "the ring mode is for the position terms of the 16-bit types");
   extern __shared__ __attribute__((aligned(16))) char smem[];
   char* Ks = smem;
   char* Vs = Ks + C::K_BYTES;
   ST* c2pS = (ST*)(Vs + C::V_BYTES);
   ST* p2cS = (ST*)((char*)c2pS + (C2P ? C::C2P_BYTES : 0));
+  char* EK = (char*)p2cS + (P2C ? C::P2C_BYTES : 0);
+  char* EQ = EK + (C2P ? C::RING_BYTES : 0);
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, li = lane & 31, g = lane >> 5;
@@ -250,14 +268,15 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, FAR_ONLY
     for (int v = 0; v < 16; ++v) o_acc[d][v] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;  // l_run: this lane's half of the row sum
 
-  // the tile walked after tile t (far-only runs jump over the near range)
+  // the tile walked after tile t (far-only runs jump over the near range, ring runs walk nothing else)
+  const int t_end = RING ? t_near1 : n_tiles;
   auto next_tile = [&](int t) __attribute__((always_inline)) {
     return (FAR_ONLY && t + 1 >= t_near0 && t + 1 < t_near1) ? t_near1 : t + 1;
   };
   u32x4 kreg[C::K_CHUNKS], vreg[C::V_CHUNKS];
   {
-    const int first = next_tile(-1);
-    if (first < n_tiles) {
+    const int first = RING ? t_near0 : next_tile(-1);
+    if (first < t_end) {
       tile_load<D * QT::SZ>(kreg, kb, k_rsb, first * FDB_BN, Lb, tid);
       tile_load<D * VT::SZ>(vreg, vb, v_rsb, first * FDB_BN, Lb, tid);
     }
@@ -269,7 +288,7 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, FAR_ONLY
     tile_store<D * VT::SZ, C::V_RS>(Vs, vreg, tid);
     __syncthreads();
     const int nt = next_tile(t);
-    if (nt < n_tiles) {  // next tile's global loads fly during this tile's math
+    if (nt < t_end) {  // next tile's global loads fly during this tile's math
       tile_load<D * QT::SZ>(kreg, kb, k_rsb, nt * FDB_BN, Lb, tid);
       tile_load<D * VT::SZ>(vreg, vb, v_rsb, nt * FDB_BN, Lb, tid);
     }
@@ -308,10 +327,196 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, FAR_ONLY
   };
 
   // ---- far-left ------------------------------------------------------------------------------
-  far_range(0, t_near0, 0);
+  if constexpr (!RING) far_range(0, t_near0, 0);
 
   // ---- near ----------------------------------------------------------------------------------
-  if constexpr (kHasPos && !FAR_ONLY) {
+  if constexpr (RING) {
+    // Relative positions of the workgroup tile k = t - t_near0: r in [r_hi0 - 64k - 190, r_hi0 - 64k];
+    // u = r_hi0 - r counts downwards from the first tile's largest r, ring slot = u & 255,
+    // batch = u / 64 (tile k reads batches k .. k+2).  A batch is staged like a K tile: the same
+    // 16-byte chunks per thread, its table values one stage ahead of its rows.
+    constexpr int RCH = C::K_CHUNKS, CPR = D * QT::SZ / 16, KS = C::KSTEPS;
+    const int r_hi0 = m0 + FDB_BM - 1 - t_near0 * FDB_BN;
+    u32x4 ekreg[RCH], eqreg[RCH];
+    int dnext[RCH];
+    auto batch_delta = [&](int batch, int (&dl)[RCH]) __attribute__((always_inline)) {
+#pragma unroll
+      for (int n = 0; n < RCH; ++n) {
+        const int r = r_hi0 - (batch * 64 + min((tid + n * kThreads) / CPR, FDB_BN - 1));
+        dl[n] = p.lut[max(-p.R, min(p.R, r)) + p.R];
+      }
+    };
+    auto batch_load = [&](const int (&dl)[RCH]) __attribute__((always_inline)) {
+#pragma unroll
+      for (int n = 0; n < RCH; ++n) {
+        const int cc = (tid + n * kThreads) % CPR;
+        if constexpr (C2P) ekreg[n] = *(const u32x4*)(pkb + (int64_t)dl[n] * p.pk_sr * QT::SZ + cc * 16);
+        if constexpr (P2C) eqreg[n] = *(const u32x4*)(pqb + (int64_t)dl[n] * p.pq_sr * QT::SZ + cc * 16);
+      }
+    };
+    auto batch_store = [&](int batch) __attribute__((always_inline)) {
+      const int seg = (batch & 3) * 64 * C::K_RS;
+      if constexpr (C2P) tile_store<D * QT::SZ, C::K_RS>(EK + seg, ekreg, tid);
+      if constexpr (P2C) tile_store<D * QT::SZ, C::K_RS>(EQ + seg, eqreg, tid);
+    };
+    // tile t = t_near0 + k: K, V and batch k+2 to LDS ...
+    auto ring_stage = [&](int t) __attribute__((always_inline)) {
+      __syncthreads();
+      tile_store<D * QT::SZ, C::K_RS>(Ks, kreg, tid);
+      tile_store<D * VT::SZ, C::V_RS>(Vs, vreg, tid);
+      batch_store(t - t_near0 + 2);
+      __syncthreads();
+    };
+    // ... and tile t+1's K, V and batch k+3 into the registers, in four pieces that are issued
+    // between the MFMAs of the tile
+    auto ring_prefetch = [&](int t, int piece) __attribute__((always_inline)) {
+      if (t + 1 < t_near1) {
+        if (piece == 0) batch_load(dnext);  // its table values were loaded a tile ago: no wait on the loads issued below
+        if (piece == 1) tile_load<D * QT::SZ>(kreg, kb, k_rsb, (t + 1) * FDB_BN, Lb, tid);
+        if (piece == 2) tile_load<D * VT::SZ>(vreg, vb, v_rsb, (t + 1) * FDB_BN, Lb, tid);
+        if (piece == 3 && t + 2 < t_near1) batch_delta(t - t_near0 + 4, dnext);
+      }
+    };
+    if (t_near0 < t_near1) {
+#pragma unroll 1
+      for (int bt = 0; bt < 2; ++bt) {
+        batch_delta(bt, dnext);
+        batch_load(dnext);
+        batch_store(bt);
+      }
+      batch_delta(2, dnext);
+      batch_load(dnext);
+      batch_delta(3, dnext);
+    }
+    // The query loads are consumed here: left pending into the loop, their first use would make
+    // the compiler wait for every outstanding vector-memory load at the top of each tile.
+#pragma unroll
+    for (int s = 0; s < KS; ++s) asm volatile("" ::"v"(qf[s]));
+
+    // per-lane scratch addresses (elements)
+    const int colb = 8 * g * QT::SZ;
+    ST* c_wr = c2pS + (wave * 32 + li) * kC2pStride + 4 * g;                         // C[i = li][32*blk + 8*q4 + 4*g ..+3]
+    // C[i][li + 63 - jj] for jj = 8*n + 4*g + 3 .. + 0 is the window of four elements that starts
+    // at li + 60 - 4*g - 8*n = 4*(chunk) + (li & 3).  Only 8-byte-aligned LDS reads run at speed (a
+    // misaligned one is served lane by lane), so the two aligned chunks around the window are read
+    // and the window is cut out of them with per-lane selects and a funnel shift.
+    const ST* c_rd = c2pS + (wave * 32 + li) * kC2pStride + 4 * ((li >> 2) + 15 - g);  // chunk of window n = 0; window n is 8*n elements lower
+    const bool c_odd_chunk = (li & 2) != 0;   // the window starts in the second dword of the chunk
+    const uint32_t c_shift = 16 * (li & 1);   // ... and in the high half of that dword
+    const ST* p_rd = p2cS + (4 * g) * kP2cStride + (wave * 32 + li + 63 - 4 * g);    // P[jj][wave*32 + li + 63 - jj]
+
+    // One near tile.  The wave is alone on its SIMD, so the instruction stream itself has to overlap
+    // the units: the position products come first, one MFMA per step, and each step also issues the
+    // LDS read of an operand two blocks ahead and a quarter of the previous block's write-out to the
+    // scratch.  Blocks: P (rows E_Q block `wave` against key halves 0 and 1, rows E_Q block
+    // 4 + wave/2 against key half wave%2), C (rows E_K blocks wave + 0..2 against the queries), then
+    // the content product, under which the last write-out hides.
+    auto ring_tile = [&](auto mask_tag, int t) __attribute__((always_inline)) {
+      constexpr bool MASK = decltype(mask_tag)::value;
+      constexpr int nP = P2C ? 3 : 0, nC = C2P ? 3 : 0, NB = nP + nC, nLP = P2C ? 2 : 0, NL = nLP + nC;
+      constexpr int QPS = 4 / KS;  // write-out quarters per step
+      const int j0 = t * FDB_BN;
+      ring_stage(t);
+      const int ubase = 190 + 64 * (t - t_near0) - li;
+      // A rows of operand load l: E_Q block `wave` (l = 0), 4 + wave/2 (l = 1) when P2C; then E_K blocks wave + 0..2
+      auto a_row = [&](int l) __attribute__((always_inline)) -> const char* {
+        if (l < nLP) return EQ + ((ubase - 32 * (l == 0 ? wave : 4 + (wave >> 1))) & (kRing - 1)) * C::K_RS + colb;
+        return EK + ((ubase - 32 * (wave + l - nLP)) & (kRing - 1)) * C::K_RS + colb;
+      };
+      auto blk_load = [](int b) { return P2C ? (b < 2 ? 0 : b - 1) : b; };
+      qfrag kf[2][KS], kx[KS], af[2][KS];
+#pragma unroll
+      for (int jb = 0; jb < 2; ++jb)
+#pragma unroll
+        for (int s = 0; s < KS; ++s) kf[jb][s] = QT::load(Ks + (32 * jb + li) * C::K_RS + colb + 16 * s * QT::SZ);
+#pragma unroll
+      for (int l = 0; l < 2; ++l)
+#pragma unroll
+        for (int s = 0; s < KS; ++s) af[l][s] = QT::load(a_row(l) + 16 * s * QT::SZ);
+      if constexpr (P2C) {
+#pragma unroll
+        for (int s = 0; s < KS; ++s) kx[s] = QT::load(Ks + (32 * (wave & 1) + li) * C::K_RS + colb + 16 * s * QT::SZ);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      f32x16 acc[2], sacc[2], zero;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) zero[v] = 0.f;
+      auto writeout = [&](int b, int q4) __attribute__((always_inline)) {
+        ST* dst;
+        if (b < nP) {
+          const int wblk = b < 2 ? wave : 4 + (wave >> 1), jblk = b < 2 ? b : (wave & 1);
+          dst = p2cS + (jblk * 32 + li) * kP2cStride + 32 * wblk + 4 * g + 8 * q4;
+        } else {
+          dst = c_wr + 32 * (b - nP) + 8 * q4;
+        }
+        store4_scratch<ST>(dst, acc[b & 1][4 * q4], acc[b & 1][4 * q4 + 1], acc[b & 1][4 * q4 + 2], acc[b & 1][4 * q4 + 3]);
+      };
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+          const int l = blk_load(b);
+          const qfrag bop = b < nP ? (b == 0 ? kf[0][s] : b == 1 ? kf[1][s] : kx[s]) : qf[s];
+          acc[b & 1] = QT::mma(af[l & 1][s], bop, s == 0 ? zero : acc[b & 1]);
+          if ((b + 1 == NB || blk_load(b + 1) != l) && l + 2 < NL) af[l & 1][s] = QT::load(a_row(l + 2) + 16 * s * QT::SZ);
+          if (b > 0) {
+#pragma unroll
+            for (int e = 0; e < QPS; ++e) writeout(b - 1, QPS * s + e);
+          }
+          if (b == 1) {
+#pragma unroll
+            for (int e = 0; e < QPS; ++e) ring_prefetch(t, QPS * s + e);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        if (P2C && C2P && b == nP) __syncthreads();  // the three P blocks of every wave are in the scratch
+      }
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) writeout(NB - 1, q4);
+      if (P2C && !C2P) __syncthreads();
+      wave_lds_fence();  // this wave's C write-outs precede its reads below (the LDS unit keeps a wave's operations in order)
+      // element (j = j0 + jj, i): jj = 32*jb + 8*q + 4*g + e adds C[i][li + 63 - jj] + P[jj][wave*32 + li + 63 - jj].
+      // The scratch reads keep the LDS unit busy for longer than they take to issue: the MFMAs of
+      // the content product are spread between them.
+      u32x4 cw[C2P ? 8 : 1];
+      uint32_t px[P2C ? 32 : 1];
+#pragma unroll
+      for (int n = 0; n < 8; ++n) {
+        if constexpr (C2P) {
+          const u32x2 lo = *(const u32x2*)(c_rd - 8 * n), hi = *(const u32x2*)(c_rd - 8 * n + 4);
+          cw[n] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+        }
+        if constexpr (P2C) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) px[4 * n + e] = *(const uint16_t*)(p_rd + (8 * n + e) * (kP2cStride - 1));
+        }
+        if (n < 2 * KS) sacc[n / KS] = QT::mma(kf[n / KS][n % KS], qf[n % KS], n % KS == 0 ? zero : sacc[n / KS]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int jb = 0; jb < 2; ++jb)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          if constexpr (C2P) {
+            const u32x4 d = cw[4 * jb + q];
+            const uint32_t wa = c_odd_chunk ? d[1] : d[0], wb = c_odd_chunk ? d[2] : d[1], wc = c_odd_chunk ? d[3] : d[2];
+            const uint32_t w[2] = {__builtin_amdgcn_alignbit(wb, wa, c_shift), __builtin_amdgcn_alignbit(wc, wb, c_shift)};  // window elements 0,1 | 2,3 for e = 3,2 | 1,0
+            sacc[jb][4 * q + 0] = QT::add_hi(sacc[jb][4 * q + 0], w[1]);
+            sacc[jb][4 * q + 1] = QT::add_lo(sacc[jb][4 * q + 1], w[1]);
+            sacc[jb][4 * q + 2] = QT::add_hi(sacc[jb][4 * q + 2], w[0]);
+            sacc[jb][4 * q + 3] = QT::add_lo(sacc[jb][4 * q + 3], w[0]);
+          }
+          if constexpr (P2C) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sacc[jb][4 * q + e] = QT::add_lo(sacc[jb][4 * q + e], px[16 * jb + 4 * q + e]);
+          }
+        }
+      softmax_pv<VT, D, MASK>(sacc, o_acc, m_run, l_run, x_scale, 0.f, Vs, C::V_RS, lane, j0, i, Lb, MASK && p.causal != 0);
+    };
+    const int tm = max(t_near0, min(t_near1, n_full));
+    for (int t = t_near0; t < tm; ++t) ring_tile(std::false_type{}, t);
+    for (int t = tm; t < t_near1; ++t) ring_tile(std::true_type{}, t);
+  } else if constexpr (kHasPos && !FAR_ONLY) {
     // Row offsets (bytes) into K_r / Q_r of the A rows this lane feeds to the position products
     // of one tile; looked up through the table one tile ahead so that the row loads of a tile
     // never wait for the table.
@@ -418,10 +623,44 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, FAR_ONLY
   }
 
   // ---- far-right -----------------------------------------------------------------------------
-  far_range(t_near1, n_tiles, 1);
+  if constexpr (!RING) far_range(t_near1, n_tiles, 1);
 
   // ---- epilogue ------------------------------------------------------------------------------
   const float l_tot = wave_half_sum(l_run);
+  if constexpr (RING) {
+    // merge with the far tiles' partial result (rows normalised over the far keys in out, their
+    // log-sum-exp in lse), normalise, store
+    if (i < Lb) {
+      char* orow = ob + (int64_t)i * p.o_st * VT::SZ;
+      const int64_t tok = p.cu ? (int64_t)tok0 + i : (int64_t)b * p.L + tok0 + i;
+      float w_far = 0.f, w_near = 1.f, m_out = m_run;
+      if (p.far_done) {
+        const float lf = p.lse[tok * p.H + h] * 1.4426950408889634f;  // base 2 (-inf: no far tile)
+        const float ln_ = m_run + __builtin_amdgcn_logf(l_tot);
+        m_out = fmaxf(lf, ln_);
+        w_far = __builtin_amdgcn_exp2f(lf - m_out);
+        w_near = __builtin_amdgcn_exp2f(m_run - m_out);
+      }
+      const float denom = w_far + w_near * l_tot;
+      const float inv = denom > 0.f ? 1.f / denom : 0.f;
+      const float sn = w_near * inv, sf = w_far * inv;
+#pragma unroll
+      for (int d = 0; d < C::DBLKS; ++d)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          char* dst = orow + (32 * d + 8 * q4 + 4 * g) * VT::SZ;
+          float f0 = 0.f, f1 = 0.f, f2 = 0.f, f3 = 0.f;
+          if (p.far_done) {
+            const f32x4 far4 = VT::load4(dst);
+            f0 = far4[0] * sf; f1 = far4[1] * sf; f2 = far4[2] * sf; f3 = far4[3] * sf;
+          }
+          VT::store4(dst, o_acc[d][4 * q4] * sn + f0, o_acc[d][4 * q4 + 1] * sn + f1, o_acc[d][4 * q4 + 2] * sn + f2,
+                     o_acc[d][4 * q4 + 3] * sn + f3);
+        }
+      if (p.lse && g == 0) p.lse[tok * p.H + h] = (m_out + __builtin_amdgcn_logf(denom)) * 0.6931471805599453f;
+    }
+    return;
+  }
   const float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
   if (i < Lb) {
     char* orow = ob + (int64_t)i * p.o_st * VT::SZ;
@@ -440,11 +679,11 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, FAR_ONLY
   }
 }
 
-template <class QT, class VT, int D, bool FP8, bool C2P, bool P2C, bool FAR_ONLY>
+template <class QT, class VT, int D, bool FP8, bool C2P, bool P2C, int MODE>
 int launch_one(const FdbKParams& p, int grid_x, hipStream_t stream) {
   using C = Cfg<QT, VT, D>;
-  auto kern = fdb_attn_kernel<QT, VT, D, FP8, C2P, P2C, FAR_ONLY>;
-  constexpr int lds = FAR_ONLY ? C::lds_bytes(false, false) : C::lds_bytes(C2P, P2C);
+  auto kern = fdb_attn_kernel<QT, VT, D, FP8, C2P, P2C, MODE>;
+  constexpr int lds = C::lds_bytes_mode(MODE, C2P, P2C);
   static_assert(lds <= 160 * 1024, "LDS budget");
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
   if (e != hipSuccess) return (int)e;
@@ -453,30 +692,35 @@ int launch_one(const FdbKParams& p, int grid_x, hipStream_t stream) {
 }
 
 template <class QT, class VT, int D, bool FP8>
-int launch_pos(const FdbKParams& p, int grid_x, bool far_only, hipStream_t stream) {
-  if constexpr (!FP8 && QT::SZ == 2 && D <= 64) {  // the combinations the near kernel covers
-    if (far_only) {
-      if (p.pk && p.pq) return launch_one<QT, VT, D, FP8, true, true, true>(p, grid_x, stream);
-      if (p.pk) return launch_one<QT, VT, D, FP8, true, false, true>(p, grid_x, stream);
-      return launch_one<QT, VT, D, FP8, false, true, true>(p, grid_x, stream);
+int launch_pos(const FdbKParams& p, int grid_x, int mode, hipStream_t stream) {
+  if constexpr (!FP8 && QT::SZ == 2 && D <= 64) {  // the combinations the two-launch path covers
+    if (mode == kFarOnly) {
+      if (p.pk && p.pq) return launch_one<QT, VT, D, FP8, true, true, kFarOnly>(p, grid_x, stream);
+      if (p.pk) return launch_one<QT, VT, D, FP8, true, false, kFarOnly>(p, grid_x, stream);
+      if (p.pq) return launch_one<QT, VT, D, FP8, false, true, kFarOnly>(p, grid_x, stream);
+    }
+    if (mode == kNearRing) {
+      if (p.pk && p.pq) return launch_one<QT, VT, D, FP8, true, true, kNearRing>(p, grid_x, stream);
+      if (p.pk) return launch_one<QT, VT, D, FP8, true, false, kNearRing>(p, grid_x, stream);
+      if (p.pq) return launch_one<QT, VT, D, FP8, false, true, kNearRing>(p, grid_x, stream);
     }
   }
-  if (far_only) return FDB_ERR_UNSUPPORTED;
-  if (p.pk && p.pq) return launch_one<QT, VT, D, FP8, true, true, false>(p, grid_x, stream);
-  if (p.pk) return launch_one<QT, VT, D, FP8, true, false, false>(p, grid_x, stream);
-  if (p.pq) return launch_one<QT, VT, D, FP8, false, true, false>(p, grid_x, stream);
-  return launch_one<QT, VT, D, FP8, false, false, false>(p, grid_x, stream);
+  if (mode != kFused) return FDB_ERR_UNSUPPORTED;
+  if (p.pk && p.pq) return launch_one<QT, VT, D, FP8, true, true, kFused>(p, grid_x, stream);
+  if (p.pk) return launch_one<QT, VT, D, FP8, true, false, kFused>(p, grid_x, stream);
+  if (p.pq) return launch_one<QT, VT, D, FP8, false, true, kFused>(p, grid_x, stream);
+  return launch_one<QT, VT, D, FP8, false, false, kFused>(p, grid_x, stream);
 }
 
 }  // namespace
 
-int fdb_launch_attn(const FdbKParams& p, int dtype, int head_dim, int grid_x, bool far_only, void* stream_) {
+int fdb_launch_attn(const FdbKParams& p, int dtype, int head_dim, int grid_x, int mode, void* stream_) {
   hipStream_t stream = (hipStream_t)stream_;
 #define FDB_DISPATCH_D(QT, VT, FP8)                                   \
   switch (head_dim) {                                                 \
-    case 32: return launch_pos<QT, VT, 32, FP8>(p, grid_x, far_only, stream);   \
-    case 64: return launch_pos<QT, VT, 64, FP8>(p, grid_x, far_only, stream);   \
-    case 128: return launch_pos<QT, VT, 128, FP8>(p, grid_x, far_only, stream); \
+    case 32: return launch_pos<QT, VT, 32, FP8>(p, grid_x, mode, stream);   \
+    case 64: return launch_pos<QT, VT, 64, FP8>(p, grid_x, mode, stream);   \
+    case 128: return launch_pos<QT, VT, 128, FP8>(p, grid_x, mode, stream); \
     default: return FDB_ERR_HEAD_DIM;                                 \
   }
   switch (dtype) {
@@ -484,8 +728,8 @@ int fdb_launch_attn(const FdbKParams& p, int dtype, int head_dim, int grid_x, bo
     case FDB_F16: FDB_DISPATCH_D(F16Tr, F16Tr, false)
     case FDB_F32:
       switch (head_dim) {
-        case 32: return launch_pos<F32Tr, F32Tr, 32, false>(p, grid_x, far_only, stream);
-        case 64: return launch_pos<F32Tr, F32Tr, 64, false>(p, grid_x, far_only, stream);
+        case 32: return launch_pos<F32Tr, F32Tr, 32, false>(p, grid_x, mode, stream);
+        case 64: return launch_pos<F32Tr, F32Tr, 64, false>(p, grid_x, mode, stream);
         default: return FDB_ERR_UNSUPPORTED;
       }
     case FDB_FP8_E4M3: FDB_DISPATCH_D(Fp8Tr, Bf16Tr, true)

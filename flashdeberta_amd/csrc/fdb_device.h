@@ -18,6 +18,7 @@ typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(8))) short s16x8;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
 #define LDS_AS __attribute__((address_space(3)))
 
@@ -51,6 +52,15 @@ struct Bf16Tr {
     f32x4 x = {a, b, c, d};
     *(bf16x4*)p = __builtin_convertvector(x, bf16x4);
   }
+  // acc + the low / high element of a packed pair, one instruction each.  The selectors carry -0
+  // in the unused half: (1, +0) would be encoded as the inline constant 1.0, which the dot
+  // instruction reads as the fp32 pattern, i.e. as (+0, 1).
+  static __device__ __forceinline__ float add_lo(float acc, uint32_t pair) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pair), bf16x2{(__bf16)1.0f, (__bf16)-0.0f}, acc, false);
+  }
+  static __device__ __forceinline__ float add_hi(float acc, uint32_t pair) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pair), bf16x2{(__bf16)-0.0f, (__bf16)1.0f}, acc, false);
+  }
   static __device__ __forceinline__ f32x4 load4(const char* p) { return __builtin_convertvector(*(const bf16x4*)p, f32x4); }
 };
 
@@ -74,6 +84,12 @@ struct F16Tr {
   static __device__ __forceinline__ void store4(char* p, float a, float b, float c, float d) {
     f32x4 x = {a, b, c, d};
     *(f16x4*)p = __builtin_convertvector(x, f16x4);
+  }
+  static __device__ __forceinline__ float add_lo(float acc, uint32_t pair) {
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, pair), f16x2{(_Float16)1.0f, (_Float16)-0.0f}, acc, false);
+  }
+  static __device__ __forceinline__ float add_hi(float acc, uint32_t pair) {
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, pair), f16x2{(_Float16)-0.0f, (_Float16)1.0f}, acc, false);
   }
   static __device__ __forceinline__ f32x4 load4(const char* p) { return __builtin_convertvector(*(const f16x4*)p, f32x4); }
 };
@@ -101,6 +117,8 @@ struct F32Tr {
     *(f32x4*)p = f32x4{a, b, c, d};
   }
   static __device__ __forceinline__ f32x4 load4(const char* p) { return *(const f32x4*)p; }
+  static __device__ __forceinline__ float add_lo(float acc, uint32_t) { return acc; }  // 16-bit scratch only
+  static __device__ __forceinline__ float add_hi(float acc, uint32_t) { return acc; }
 };
 
 struct Fp8Tr {  // OCP e4m3, operands of the three score products only
@@ -114,6 +132,8 @@ struct Fp8Tr {  // OCP e4m3, operands of the three score products only
   }
   static __device__ __forceinline__ f32x8 to_f32(frag) { return f32x8{0, 0, 0, 0, 0, 0, 0, 0}; }  // unused
   static __device__ __forceinline__ frag from_f32(f32x8) { return 0; }                             // unused
+  static __device__ __forceinline__ float add_lo(float acc, uint32_t) { return acc; }               // unused
+  static __device__ __forceinline__ float add_hi(float acc, uint32_t) { return acc; }
 };
 
 // V^T operand of a K=16 step: lane (d = l%32, g = l/32) needs V[j(g,e)][d] for

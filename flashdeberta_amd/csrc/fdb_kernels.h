@@ -39,10 +39,16 @@ struct FdbKParams {
 };
 
 // Launchers return the hipError_t of the launch as int.
-// fdb_launch_attn: one kernel walks every key tile.  far_only: it skips the near tiles and leaves
-// the far tiles' partial result (normalised rows in out, their log-sum-exp in lse, -inf where a row
-// has no far tile) for fdb_launch_near to merge.
-int fdb_launch_attn(const FdbKParams& p, int dtype, int head_dim, int grid_x, bool far_only, void* stream);
+// fdb_launch_attn, by mode:
+//   FDB_MODE_FUSED      one kernel walks every key tile;
+//   FDB_MODE_FAR_ONLY   it skips the near tiles and leaves the far tiles' partial result (normalised
+//                       rows in out, their log-sum-exp in lse, -inf where a row has no far tile);
+//   FDB_MODE_NEAR_RING  the near tiles only, four waves of 32 rows x 64 keys with the expanded
+//                       relative-embedding rows in LDS rings, merged with the far partial when
+//                       p.far_done.
+// The last two exist for the 16-bit element types with head_dim <= 64 (fdb_near_supported).
+enum { FDB_MODE_FUSED = 0, FDB_MODE_FAR_ONLY = 1, FDB_MODE_NEAR_RING = 2 };
+int fdb_launch_attn(const FdbKParams& p, int dtype, int head_dim, int grid_x, int mode, void* stream);
 // fdb_launch_near: the near tiles only (expanded relative-embedding rows staged in LDS rings),
 // merged with the far partial when p.far_done.  16-bit element types with head_dim <= 64.
 bool fdb_near_supported(int dtype, int head_dim);

@@ -233,7 +233,13 @@ __global__ __launch_bounds__(kNThreads, 1) void fdb_near_kernel(const FdbKParams
   // A row (block bk, lane li): r = r_lo + 32*bk + li  ->  u = r_hi0 - r = ubase - 32*bk + 64*k
   const int ubase = 158 - 32 * (wr - wk) - li;
   // scratch reads: element (jj = 8q + 4g + t, i = li) of the sub-tile reads index r - r_lo = li + 31 - jj
-  const ST* c_rd = scr + li * kScrStride + (li + 31 - 4 * g);         // C[i = li][.], minus cj = 8q + t
+  // C[i = li][li + 31 - jj] for jj = 8q + 4g + 3 .. + 0 is the window of four elements that starts at
+  // li + 28 - 4g - 8q = 4 * chunk + (li & 3).  Only 8-byte-aligned LDS reads run at speed (a
+  // misaligned one is served lane by lane): the two aligned chunks around the window are read and
+  // the window is cut out with per-lane selects and a funnel shift.
+  const ST* c_rd = scr + li * kScrStride + 4 * ((li >> 2) + 7 - g);   // chunk of window q = 0; window q is 8q elements lower
+  const bool c_odd_chunk = (li & 2) != 0;
+  const uint32_t c_shift = 16 * (li & 1);
   const ST* p_rd = scr + (4 * g) * kScrStride + (li + 31 - 4 * g);    // P[jj][.],     plus cj * (stride - 1)
   ST* scr_wr = scr + li * kScrStride + 4 * g;                         // row = this lane's MFMA column
 
@@ -289,8 +295,8 @@ __global__ __launch_bounds__(kNThreads, 1) void fdb_near_kernel(const FdbKParams
     // ---- through the wave's scratch: write C, read its skewed diagonal, write P over it, read ------
     // The LDS unit runs one wave's operations in order, so the reads of C are served before the
     // writes of P that follow them; only the compiler needs the fences.
-    f32x4 cval[4];
-    float pval[16];
+    u32x4 cw[4];
+    uint32_t px[16];
     if constexpr (C2P) {
 #pragma unroll
       for (int bk = 0; bk < 2; ++bk)
@@ -300,7 +306,10 @@ __global__ __launch_bounds__(kNThreads, 1) void fdb_near_kernel(const FdbKParams
                              cacc[bk][4 * q4 + 3]);
       wave_lds_fence();
 #pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) cval[q4] = load4_scratch_unaligned<ST>(c_rd - (8 * q4 + 3));  // indices X-8q-3 .. X-8q
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const u32x2 lo = *(const u32x2*)(c_rd - 8 * q4), hi = *(const u32x2*)(c_rd - 8 * q4 + 4);
+        cw[q4] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+      }
       wave_lds_fence();
     }
     if constexpr (P2C) {
@@ -312,13 +321,24 @@ __global__ __launch_bounds__(kNThreads, 1) void fdb_near_kernel(const FdbKParams
                              pacc[bk][4 * q4 + 3]);
       wave_lds_fence();
 #pragma unroll
-      for (int v = 0; v < 16; ++v) pval[v] = (float)p_rd[(8 * (v >> 2) + (v & 3)) * (kScrStride - 1)];
+      for (int v = 0; v < 16; ++v) px[v] = *(const uint16_t*)(p_rd + (8 * (v >> 2) + (v & 3)) * (kScrStride - 1));
       wave_lds_fence();
     }
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      if constexpr (C2P) sacc[v] += cval[v >> 2][3 - (v & 3)];
-      if constexpr (P2C) sacc[v] += pval[v];
+    for (int q4 = 0; q4 < 4; ++q4) {
+      if constexpr (C2P) {
+        const u32x4 d = cw[q4];
+        const uint32_t wa = c_odd_chunk ? d[1] : d[0], wb = c_odd_chunk ? d[2] : d[1], wc = c_odd_chunk ? d[3] : d[2];
+        const uint32_t w0 = __builtin_amdgcn_alignbit(wb, wa, c_shift), w1 = __builtin_amdgcn_alignbit(wc, wb, c_shift);
+        sacc[4 * q4 + 0] = QT::add_hi(sacc[4 * q4 + 0], w1);  // window elements 3, 2, 1, 0 for jj offsets 0, 1, 2, 3
+        sacc[4 * q4 + 1] = QT::add_lo(sacc[4 * q4 + 1], w1);
+        sacc[4 * q4 + 2] = QT::add_hi(sacc[4 * q4 + 2], w0);
+        sacc[4 * q4 + 3] = QT::add_lo(sacc[4 * q4 + 3], w0);
+      }
+      if constexpr (P2C) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sacc[4 * q4 + e] = QT::add_lo(sacc[4 * q4 + e], px[4 * q4 + e]);
+      }
     }
     near_softmax_pv<VT, D, MASK>(sacc, o_acc, m_run, l_run, x_scale, Vs + buf * C::V_BYTES + 32 * wk * C::V_RS, C::V_RS,
                                  lane, jw0, i, Lb, MASK && p.causal != 0);
