@@ -135,6 +135,9 @@ int fdb_attn_check(const fdb_attn_args* a) {
                                 a->pos_query ? a->pq_stride_h : 0, a->pos_query ? a->pq_stride_r : 0};
   for (int64_t s : qk_strides)
     if ((s * qsz) % 16 != 0) return FDB_ERR_ALIGN;
+  // the kernels walk K and V with 32-bit row strides (in bytes)
+  if (a->k_stride_t < 0 || a->v_stride_t < 0 || a->k_stride_t * qsz > INT32_MAX || a->v_stride_t * vsz > INT32_MAX)
+    return FDB_ERR_SHAPE;
   const int64_t v_strides[] = {a->v_stride_b, a->v_stride_t, a->v_stride_h, a->o_stride_b, a->o_stride_t, a->o_stride_h};
   for (int64_t s : v_strides)
     if ((s * vsz) % 16 != 0) return FDB_ERR_ALIGN;

@@ -62,10 +62,15 @@ struct Cfg {
   static constexpr int C2P_BYTES = kWaves * 32 * kC2pStride * (int)sizeof(ST);
   static constexpr int P2C_BYTES = FDB_BN * kP2cStride * (int)sizeof(ST);
   static constexpr int RING_BYTES = kRing * K_RS;  // one ring of expanded relative-embedding rows
+  // Tiles of 128-byte rows with no position products in the kernel go global -> LDS directly,
+  // three K/V buffers deep (see the kernel).
+  static constexpr bool DMA_OK = QT::SZ == 2 && VT::SZ == 2 && D == 64;
+  static constexpr int DMA_TILE = FDB_BN * 128, DMA_BUF = 2 * DMA_TILE, DMA_BYTES = 3 * DMA_BUF;
   static constexpr int lds_bytes(bool c2p, bool p2c) {
     return K_BYTES + V_BYTES + (c2p ? C2P_BYTES : 0) + (p2c ? P2C_BYTES : 0);
   }
   static constexpr int lds_bytes_mode(int mode, bool c2p, bool p2c) {
+    if (DMA_OK && (mode == 1 || (mode == 0 && !c2p && !p2c))) return DMA_BYTES;
     return mode == 1 ? lds_bytes(false, false)
                      : lds_bytes(c2p, p2c) + (mode == 2 ? (c2p ? RING_BYTES : 0) + (p2c ? RING_BYTES : 0) : 0);
   }
@@ -74,7 +79,7 @@ struct Cfg {
 // [64 x ROW_BYTES] tile: global -> registers -> LDS.  Rows past the end of the sequence re-read the
 // last valid row (finite data, no predication); their scores are masked to -inf before the soft-max.
 template <int ROW_BYTES, int NCH>
-__device__ __forceinline__ void tile_load(u32x4 (&reg)[NCH], const char* gbase, int64_t row_stride_bytes, int j0,
+__device__ __forceinline__ void tile_load(u32x4 (&reg)[NCH], const char* gbase, uint32_t row_stride_bytes, int j0,
                                           int n_rows, int tid) {
   constexpr int CPR = ROW_BYTES / 16;
   constexpr int TOTAL = FDB_BN * CPR;
@@ -82,7 +87,7 @@ __device__ __forceinline__ void tile_load(u32x4 (&reg)[NCH], const char* gbase, 
   for (int n = 0; n < NCH; ++n) {
     const int c = tid + n * kThreads;
     const int row = min(j0 + min(c / CPR, FDB_BN - 1), n_rows - 1), cc = c % CPR;
-    reg[n] = *(const u32x4*)(gbase + (int64_t)row * row_stride_bytes + cc * 16);
+    reg[n] = *(const u32x4*)(gbase + (uint64_t)(uint32_t)row * row_stride_bytes + cc * 16);  // one 32 x 32 -> 64-bit multiply-add
   }
 }
 template <int ROW_BYTES, int RS, int NCH>
@@ -100,9 +105,9 @@ __device__ __forceinline__ void tile_store(char* lds, const u32x4 (&reg)[NCH], i
 // One key tile after its scores are in sacc (raw products, position terms already added where the
 // tile needs them element-wise): mask, online soft-max in base 2, O^T += V^T P^T.
 //   x = sacc * x_scale + row_add   (row_add: the per-row constant of a far tile, already scaled)
-template <class VT, int D, bool MASK>
+template <class VT, int D, bool MASK, class VL>
 __device__ __forceinline__ void softmax_pv(f32x16 (&sacc)[2], f32x16 (&o_acc)[D / 32], float& m_run, float& l_run,
-                                           float x_scale, float row_add, const char* Vs, int v_rs, int lane, int j0,
+                                           float x_scale, float row_add, const VL& vload, int lane, int j0,
                                            int i, int Lb, bool causal) {
   using vfrag = typename VT::frag;
   const int g = lane >> 5;
@@ -141,7 +146,67 @@ __device__ __forceinline__ void softmax_pv(f32x16 (&sacc)[2], f32x16 (&o_acc)[D 
     l_run = VT::sum8(pf, l_run);  // the row sum is taken over the probabilities as the MFMA sees them
 #pragma unroll
     for (int d = 0; d < D / 32; ++d) {
-      const vfrag vf = VtLoad<VT>::get(Vs, v_rs, c, d, lane);
+      const vfrag vf = vload(c, d);
+      o_acc[d] = VT::mma(vf, pf, o_acc[d]);
+    }
+  }
+}
+
+// The same for tiles whose scores leave the MFMA ready for the exponential: the query operand
+// carries the soft-max scale and the accumulator started from negm = row_add - (reference point of
+// the row), so sacc = x - reference.  The reference point moves only when the tile maximum exceeds
+// it by more than the lazy threshold (or on the row's first tile, whose reference is 0); the tile
+// at hand and negm are then shifted to the new one.
+template <class VT, int D, bool MASK, class VL>
+__device__ __forceinline__ void softmax_pv_pre(f32x16 (&sacc)[2], f32x16 (&o_acc)[D / 32], float& m_run, float& l_run,
+                                               float row_add, f32x16& negm, const VL& vload, int lane, int j0,
+                                               int i, int Lb, bool causal) {
+  using vfrag = typename VT::frag;
+  const int g = lane >> 5;
+  if constexpr (MASK) {
+#pragma unroll
+    for (int jb = 0; jb < 2; ++jb)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int j = j0 + 32 * jb + 8 * (v >> 2) + 4 * g + (v & 3);
+        if (j >= Lb || (causal && j > i)) sacc[jb][v] = -INFINITY;
+      }
+  }
+  float mx = sacc[0][0];
+#pragma unroll
+  for (int jb = 0; jb < 2; ++jb)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) mx = fmaxf(mx, sacc[jb][v]);
+  mx = wave_half_max(mx);
+  const bool first = m_run == -INFINITY;
+  if (__any(mx > kLazyTau || first)) {
+    const bool mv = mx > kLazyTau || first;
+    const float shift = mv ? mx : 0.f;
+    const float alpha = first ? 0.f : __builtin_amdgcn_exp2f(-shift);
+    m_run = (first ? 0.f : m_run) + shift;
+    l_run *= alpha;
+#pragma unroll
+    for (int d = 0; d < D / 32; ++d)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) o_acc[d][v] *= alpha;
+#pragma unroll
+    for (int jb = 0; jb < 2; ++jb)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) sacc[jb][v] -= shift;
+    const float nm = row_add - m_run;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) negm[v] = nm;
+  }
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    f32x8 pv;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) pv[e] = __builtin_amdgcn_exp2f(sacc[c >> 1][8 * (c & 1) + e]);
+    const vfrag pf = VT::from_f32(pv);
+    l_run = VT::sum8(pf, l_run);
+#pragma unroll
+    for (int d = 0; d < D / 32; ++d) {
+      const vfrag vf = vload(c, d);
       o_acc[d] = VT::mma(vf, pf, o_acc[d]);
     }
   }
@@ -153,7 +218,7 @@ constexpr int min_blocks() {
   const int lds = Cfg<QT, VT, D>::lds_bytes_mode(MODE, C2P, P2C);
   if (MODE == kFarOnly) return 3;  // the far zones need the shifted query and the per-row constants on top of the plain kernel
   if (MODE == kNearRing) return 2;  // one workgroup fits a CU; the bound keeps every value in the 256 registers VALU code can read
-  return lds <= 40 * 1024 ? 4 : lds <= 80 * 1024 ? 2 : 1;
+  return lds <= 40 * 1024 ? 3 : lds <= 80 * 1024 ? 2 : 1;  // three: 170 registers, the plain loop's working set without spills
 }
 
 template <class QT, class VT, int D, bool FP8, bool C2P, bool P2C, int MODE>
@@ -199,7 +264,7 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
   char* ob = p.out + (oo + (int64_t)tok0 * p.o_st + (int64_t)h * p.o_sh) * VT::SZ;
   const char* pkb = C2P ? p.pk + (int64_t)h * p.pk_sh * QT::SZ : nullptr;
   const char* pqb = P2C ? p.pq + (int64_t)h * p.pq_sh * QT::SZ : nullptr;
-  const int64_t k_rsb = p.k_st * QT::SZ, v_rsb = p.v_st * VT::SZ;
+  const uint32_t k_rsb = (uint32_t)(p.k_st * QT::SZ), v_rsb = (uint32_t)(p.v_st * VT::SZ);  // the host checks that they fit
 
   // fp8: raw products are in units of (q_scale*k_scale); bring the two position products to the
   // same unit so that one factor converts the sum.
@@ -234,11 +299,22 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
     t_near1 = max(t_near0, min(n_tiles, (m0 + FDB_BM - 1 + p.R + FDB_BN - 1) / FDB_BN));  // far-right: j0 >= m0+127+R
   }
 
-  // per-row constants and shifted queries of the two far zones
+  // per-row constants and shifted queries of the two far zones.  Except in fp8 the far / plain
+  // tiles use queries that carry the soft-max scale (PRE), and their accumulators start from negm.
+  f32x16 o_acc[C::DBLKS];
+#pragma unroll
+  for (int d = 0; d < C::DBLKS; ++d)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) o_acc[d][v] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;  // l_run: this lane's half of the row sum
+  constexpr bool PRE = !FP8;
   float a_far = 0.f;  // scaled to the exponent's unit
   qfrag qfar[C::KSTEPS];
+  f32x16 negm;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) negm[v] = 0.f;
   auto setup_far = [&](int side) __attribute__((always_inline)) {  // side 0: far-left (delta(+R)), 1: far-right (delta(-R))
-    const int delta = p.lut[side == 0 ? 2 * p.R : 0];
+    const int delta = kHasPos ? p.lut[side == 0 ? 2 * p.R : 0] : 0;
     if constexpr (C2P) {
       const char* row = pkb + (int64_t)delta * p.pk_sr * QT::SZ;
       float acc = 0.f;
@@ -254,54 +330,122 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
       const char* row = pqb + (int64_t)delta * p.pq_sr * QT::SZ;
 #pragma unroll
       for (int s = 0; s < C::KSTEPS; ++s)
-        qfar[s] = QT::from_f32(QT::to_f32(qf[s]) + QT::to_f32(QT::load(row + (16 * s + 8 * g) * QT::SZ)));
+        qfar[s] = QT::from_f32((QT::to_f32(qf[s]) + QT::to_f32(QT::load(row + (16 * s + 8 * g) * QT::SZ))) * x_scale);
     } else {
 #pragma unroll
-      for (int s = 0; s < C::KSTEPS; ++s) qfar[s] = qf[s];
+      for (int s = 0; s < C::KSTEPS; ++s) qfar[s] = QT::from_f32(QT::to_f32(qf[s]) * x_scale);
     }
+    const float nm = a_far - (m_run == -INFINITY ? 0.f : m_run);
+#pragma unroll
+    for (int v = 0; v < 16; ++v) negm[v] = nm;
   };
 
-  f32x16 o_acc[C::DBLKS];
-#pragma unroll
-  for (int d = 0; d < C::DBLKS; ++d)
-#pragma unroll
-    for (int v = 0; v < 16; ++v) o_acc[d][v] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;  // l_run: this lane's half of the row sum
 
   // the tile walked after tile t (far-only runs jump over the near range, ring runs walk nothing else)
   const int t_end = RING ? t_near1 : n_tiles;
   auto next_tile = [&](int t) __attribute__((always_inline)) {
     return (FAR_ONLY && t + 1 >= t_near0 && t + 1 < t_near1) ? t_near1 : t + 1;
   };
+  // Two ways of staging the K and V tiles.
+  //
+  // Through registers (any row size): global -> registers one tile ahead, registers -> padded LDS
+  // rows between two barriers.
+  //
+  // Direct (128-byte rows, kernels without position products): global_load_lds writes the tile
+  // into one of three LDS buffers two tiles ahead; one barrier per tile, no staging registers, and
+  // the loads have two tile periods to land.  A load instruction fills 1 KB = 8 rows, lane l the
+  // 16-byte slot l; rows are not padded, so slot (row, s) holds chunk s ^ f(row) of the row,
+  // f(row) = 4*bit1(row) | bits3:2(row): sixteen consecutive rows put one chunk in sixteen
+  // different bank groups (the K fragments), and four consecutive rows put chunks 0..3 in disjoint
+  // ones (the transposing V reads).
+  constexpr bool DMA = C::DMA_OK && !RING && !FP8 && (FAR_ONLY || !kHasPos);
   u32x4 kreg[C::K_CHUNKS], vreg[C::V_CHUNKS];
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(LDS_AS char*)smem;
+  int dma_cur = 0;                 // byte offset of the buffer that holds the tile at hand
+  uint32_t kcur[4], vcur[4];       // this lane's read offsets into it
+  uint32_t klane = 0, vlane = 0;
+  if constexpr (DMA) {
+    const int fl = 4 * ((li >> 1) & 1) | ((li >> 2) & 3);  // f(row) of the K fragment rows 32*jb + li
+    klane = li * 128 + ((g ^ fl) * 16);                    // chunk 2*s + g: slot (2*s) ^ g ^ f
+    // V^T operand (c, d-block db, half h): row 16c + 8h + 4*(grp/2) + s16/4, 8-byte unit 8db + 4*(grp%2) + s16%4
+    const int s16 = lane & 15, grp = lane >> 4;
+    const int slotl = (2 * (grp & 1) + ((s16 & 3) >> 1)) ^ (4 * ((s16 >> 3) & 1)) ^ (grp >> 1);  // chunk ^ f, less (4db) ^ (2h)
+    vlane = (4 * (grp >> 1) + (s16 >> 2)) * 128 + slotl * 16 + (s16 & 1) * 8;
+  }
+  auto dma_issue = [&](int tile, int bufoff) __attribute__((always_inline)) {
+#pragma unroll
+    for (int q2 = 0; q2 < 2; ++q2) {  // this wave's two 8-row groups of K and of V
+      const int row = 16 * wave + 8 * q2 + (lane >> 3);
+      const uint32_t c = (lane & 7) ^ (4 * ((lane >> 4) & 1)) ^ (lane >> 5) ^ (2 * q2);  // slot ^ f(row)
+      const uint32_t rg = (uint32_t)min(tile * FDB_BN + row, Lb - 1);  // rows past the end re-read the last one
+      const uint32_t dst = lds0 + bufoff + (2 * wave + q2) * 1024;
+      dma16(kb + (uint64_t)rg * k_rsb + c * 16, dst);
+      dma16(vb + (uint64_t)rg * v_rsb + c * 16, dst + C::DMA_TILE);
+    }
+  };
   {
     const int first = RING ? t_near0 : next_tile(-1);
     if (first < t_end) {
-      tile_load<D * QT::SZ>(kreg, kb, k_rsb, first * FDB_BN, Lb, tid);
-      tile_load<D * VT::SZ>(vreg, vb, v_rsb, first * FDB_BN, Lb, tid);
+      if constexpr (DMA) {
+        dma_issue(first, 0);
+        const int second = next_tile(first);
+        if (second < t_end) dma_issue(second, C::DMA_BUF);
+        dma_cur = 2 * C::DMA_BUF;  // stage() steps to buffer 0
+      } else {
+        tile_load<D * QT::SZ>(kreg, kb, k_rsb, first * FDB_BN, Lb, tid);
+        tile_load<D * VT::SZ>(vreg, vb, v_rsb, first * FDB_BN, Lb, tid);
+      }
     }
   }
 
   auto stage = [&](int t) __attribute__((always_inline)) {
-    __syncthreads();  // every wave is done with the previous tile and its bias scratch
-    tile_store<D * QT::SZ, C::K_RS>(Ks, kreg, tid);
-    tile_store<D * VT::SZ, C::V_RS>(Vs, vreg, tid);
-    __syncthreads();
-    const int nt = next_tile(t);
-    if (nt < t_end) {  // next tile's global loads fly during this tile's math
-      tile_load<D * QT::SZ>(kreg, kb, k_rsb, nt * FDB_BN, Lb, tid);
-      tile_load<D * VT::SZ>(vreg, vb, v_rsb, nt * FDB_BN, Lb, tid);
+    if constexpr (DMA) {
+      const int nt = next_tile(t);
+      if (nt < t_end) wait_vmcnt<4>(); else wait_vmcnt<0>();  // this wave's part of tile t has landed (tile nt's may still fly)
+      __syncthreads();  // ... and everyone's; every wave is done with the tile before
+      dma_cur = dma_cur == 2 * C::DMA_BUF ? 0 : dma_cur + C::DMA_BUF;
+      if (nt < t_end) {
+        const int nn = next_tile(nt);
+        if (nn < t_end) dma_issue(nn, dma_cur >= C::DMA_BUF ? dma_cur - C::DMA_BUF : 2 * C::DMA_BUF);  // the buffer the tile before used
+      }
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        kcur[x] = (klane ^ (32 * x)) + dma_cur;
+        vcur[x] = (vlane ^ (64 * (x >> 1) ^ 32 * (x & 1))) + dma_cur + C::DMA_TILE;
+      }
+    } else {
+      __syncthreads();  // every wave is done with the previous tile and its bias scratch
+      tile_store<D * QT::SZ, C::K_RS>(Ks, kreg, tid);
+      tile_store<D * VT::SZ, C::V_RS>(Vs, vreg, tid);
+      __syncthreads();
+      const int nt = next_tile(t);
+      if (nt < t_end) {  // next tile's global loads fly during this tile's math
+        tile_load<D * QT::SZ>(kreg, kb, k_rsb, nt * FDB_BN, Lb, tid);
+        tile_load<D * VT::SZ>(vreg, vb, v_rsb, nt * FDB_BN, Lb, tid);
+      }
     }
   };
-  auto qk = [&](f32x16 (&sacc)[2], const qfrag (&qq)[C::KSTEPS]) __attribute__((always_inline)) {
+  auto vload = [&](int c, int d) __attribute__((always_inline)) {
+    if constexpr (DMA) {
+      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(smem + vcur[2 * d] + 2048 * c));
+      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(smem + vcur[2 * d + 1] + 2048 * c + 1024));
+      return __builtin_bit_cast(typename VT::frag, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    } else {
+      return VtLoad<VT>::get(Vs, C::V_RS, c, d, lane);
+    }
+  };
+  f32x16 zero16;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) zero16[v] = 0.f;
+  auto qk = [&](f32x16 (&sacc)[2], const qfrag (&qq)[C::KSTEPS], const f32x16& init) __attribute__((always_inline)) {
 #pragma unroll
     for (int jb = 0; jb < 2; ++jb) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) sacc[jb][v] = 0.f;
-#pragma unroll
       for (int s = 0; s < C::KSTEPS; ++s) {
-        qfrag kf = QT::load(Ks + (jb * 32 + li) * C::K_RS + (16 * s + 8 * g) * QT::SZ);
-        sacc[jb] = QT::mma(kf, qq[s], sacc[jb]);
+        qfrag kf;
+        if constexpr (DMA) kf = QT::load(smem + kcur[s] + jb * 4096);
+        else kf = QT::load(Ks + (jb * 32 + li) * C::K_RS + (16 * s + 8 * g) * QT::SZ);
+        sacc[jb] = QT::mma(kf, qq[s], s == 0 ? init : sacc[jb]);
       }
     }
   };
@@ -313,14 +457,20 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
     for (int t = t0; t < t1; ++t) {
       stage(t);
       f32x16 sacc[2];
-      if constexpr (kFarOk) qk(sacc, qfar); else qk(sacc, qf);
-      softmax_pv<VT, D, MASK>(sacc, o_acc, m_run, l_run, x_scale, a_far, Vs, C::V_RS, lane, t * FDB_BN, i, Lb,
-                              MASK && p.causal != 0);
+      if constexpr (PRE) {
+        qk(sacc, qfar, negm);
+        softmax_pv_pre<VT, D, MASK>(sacc, o_acc, m_run, l_run, a_far, negm, vload, lane, t * FDB_BN, i, Lb,
+                                    MASK && p.causal != 0);
+      } else {
+        qk(sacc, qf, zero16);
+        softmax_pv<VT, D, MASK>(sacc, o_acc, m_run, l_run, x_scale, a_far, vload, lane, t * FDB_BN, i, Lb,
+                                MASK && p.causal != 0);
+      }
     }
   };
   auto far_range = [&](int t0, int t1, int side) __attribute__((always_inline)) {
     if (t0 >= t1) return;
-    if constexpr (kFarOk) setup_far(side);
+    if constexpr (PRE) setup_far(side);
     const int tm = max(t0, min(t1, n_full));
     far_loop(std::false_type{}, t0, tm);
     far_loop(std::true_type{}, tm, t1);
@@ -511,7 +661,7 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
             for (int e = 0; e < 4; ++e) sacc[jb][4 * q + e] = QT::add_lo(sacc[jb][4 * q + e], px[16 * jb + 4 * q + e]);
           }
         }
-      softmax_pv<VT, D, MASK>(sacc, o_acc, m_run, l_run, x_scale, 0.f, Vs, C::V_RS, lane, j0, i, Lb, MASK && p.causal != 0);
+      softmax_pv<VT, D, MASK>(sacc, o_acc, m_run, l_run, x_scale, 0.f, vload, lane, j0, i, Lb, MASK && p.causal != 0);
     };
     const int tm = max(t_near0, min(t_near1, n_full));
     for (int t = t_near0; t < tm; ++t) ring_tile(std::false_type{}, t);
@@ -562,7 +712,7 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
       stage(t);
       if (t + 1 < t_near1) lookup(t + 1);
       f32x16 sacc[2];
-      qk(sacc, qf);
+      qk(sacc, qf, zero16);
       if constexpr (C2P) {
         // C[i][r - r_lo]: column i = li, rows 32*blk + 8*q4 + 4*g + 0..3
         ST* dst0 = c2pS + (wave * 32 + li) * kC2pStride + 4 * g;
@@ -613,7 +763,7 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
             if constexpr (P2C) sacc[jb][v] += (float)pbase[cj * kP2cStride - cj];
           }
       }
-      softmax_pv<VT, D, MASK>(sacc, o_acc, m_run, l_run, x_scale, 0.f, Vs, C::V_RS, lane, j0, i, Lb,
+      softmax_pv<VT, D, MASK>(sacc, o_acc, m_run, l_run, x_scale, 0.f, vload, lane, j0, i, Lb,
                               MASK && p.causal != 0);
     }
     };

@@ -255,6 +255,23 @@ __device__ __forceinline__ void block_map(int n, int nx, int heads, int tiles_pe
   }
 }
 
+// 16 bytes per lane from global memory straight into LDS: lane l's data lands at lds_base + 16*l
+// (lds_base: byte offset in the workgroup's LDS, the same in every lane).  Issued through asm so
+// that the compiler keeps no account of it: the kernel waits for these loads itself, with
+// wait_vmcnt, and only for the tile it is about to read.  Loads complete in issue order, so the
+// compiler's own vmcnt waits, which do not count them, can only wait longer than needed.  M0 is
+// written without being declared (it is a reserved register): nothing else in these kernels uses it.
+__device__ __forceinline__ void dma16(const void* g, uint32_t lds_base) {
+  const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(base) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  static_assert(N == 0 || N == 4, "counts used by the kernels");
+  if constexpr (N == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if constexpr (N == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+}
+
 // Orders this wave's earlier LDS accesses before its later ones (the LDS unit executes one wave's
 // operations in order; this only stops the compiler from moving them across).
 __device__ __forceinline__ void wave_lds_fence() {
