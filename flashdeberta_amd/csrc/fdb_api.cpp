@@ -2,7 +2,6 @@
 // table, and dispatch to the device launchers.  No device memory is allocated here.
 #include <math.h>
 #include <stdint.h>
-#include <stdlib.h>
 #include <string.h>
 
 #include <hip/hip_runtime_api.h>
@@ -177,9 +176,9 @@ int fdb_attn_fwd(const fdb_attn_args* a, void* stream) {
                                  : (int64_t)a->batch * p.tiles_per_seq;
   if (grid_x < 1 || grid_x * a->heads > INT32_MAX) return FDB_ERR_SHAPE;
   p.grid_x = (int32_t)grid_x;
-  // Split path: the far tiles in a far-only run of the fused kernel (lean, four workgroups per
-  // CU), the near tiles in the near kernel, which merges the two.  It needs the log-sum-exp buffer
-  // as the hand-over between the two launches.
+  // Split path: the far tiles in a far-only run of the kernel (three workgroups per CU), the near
+  // tiles in a second run (ring mode, one workgroup per CU), which merges the two.  It needs the
+  // log-sum-exp buffer as the hand-over between the two launches.
   if ((a->pos_key || a->pos_query) && a->lse && fdb_near_supported(a->dtype, a->head_dim)) {
     const bool need_far = a->max_seqlen > p.R + FDB_BN - 1;  // otherwise no tile of any query tile is far
     if (need_far) {
@@ -187,9 +186,7 @@ int fdb_attn_fwd(const fdb_attn_args* a, void* stream) {
       if (rc_far != 0) return rc_far;
     }
     p.far_done = need_far ? 1 : 0;
-    static const int near_impl = getenv("FDB_NEAR_IMPL") ? atoi(getenv("FDB_NEAR_IMPL")) : 1;
-    if (near_impl == 1) return fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, FDB_MODE_NEAR_RING, stream);
-    return fdb_launch_near(p, a->dtype, a->head_dim, (int)grid_x, stream);
+    return fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, FDB_MODE_NEAR_RING, stream);
   }
   return fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, FDB_MODE_FUSED, stream);
 }

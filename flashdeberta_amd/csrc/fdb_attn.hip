@@ -237,7 +237,8 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
   char* EQ = EK + (C2P ? C::RING_BYTES : 0);
 
   const int tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63, li = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // in scalar registers: what depends on it alone stays scalar
+  const int lane = tid & 63, li = lane & 31, g = lane >> 5;
   int xq, h;
   block_map((int)blockIdx.x, p.grid_x, p.H, p.tiles_per_seq, p.cu == nullptr, xq, h);
 
@@ -863,6 +864,10 @@ int launch_pos(const FdbKParams& p, int grid_x, int mode, hipStream_t stream) {
 }
 
 }  // namespace
+
+bool fdb_near_supported(int dtype, int head_dim) {
+  return (dtype == FDB_BF16 || dtype == FDB_F16) && (head_dim == 32 || head_dim == 64);
+}
 
 int fdb_launch_attn(const FdbKParams& p, int dtype, int head_dim, int grid_x, int mode, void* stream_) {
   hipStream_t stream = (hipStream_t)stream_;

@@ -33,7 +33,7 @@ struct FdbKParams {
   int32_t B, H, L, tiles_per_seq;
   int32_t grid_x;   // query tiles in the launch (the grid is grid_x * H workgroups)
   int32_t R;        // LUT radius
-  int32_t far_done; // near kernel only: the far tiles' partial result is already in out / lse
+  int32_t far_done; // ring mode only: the far tiles' partial result is already in out / lse
   int32_t causal;
   float scale_log2; // sm_scale * log2(e)
 };
@@ -49,10 +49,7 @@ struct FdbKParams {
 // The last two exist for the 16-bit element types with head_dim <= 64 (fdb_near_supported).
 enum { FDB_MODE_FUSED = 0, FDB_MODE_FAR_ONLY = 1, FDB_MODE_NEAR_RING = 2 };
 int fdb_launch_attn(const FdbKParams& p, int dtype, int head_dim, int grid_x, int mode, void* stream);
-// fdb_launch_near: the near tiles only (expanded relative-embedding rows staged in LDS rings),
-// merged with the far partial when p.far_done.  16-bit element types with head_dim <= 64.
 bool fdb_near_supported(int dtype, int head_dim);
-int fdb_launch_near(const FdbKParams& p, int dtype, int head_dim, int grid_x, void* stream);
 int fdb_launch_worklist(const int32_t* cu, int32_t batch, int32_t* wl, int32_t max_tiles, void* stream);
 int fdb_launch_quant(const void* x, int64_t x_st, int64_t x_sh, void* y, int64_t y_st, int64_t y_sh,
                      float* scale, uint32_t* absmax_ws, int32_t tokens, int32_t heads, int32_t head_dim,
