@@ -752,7 +752,36 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
       }
       __syncthreads();
       // element (j = j0 + jj, i): r - r_lo = li + 63 - jj (wave tile) / wave*32 + li + 63 - jj (workgroup tile)
-      {
+      if constexpr (sizeof(ST) == 2) {
+        // 16-bit scratch.  C[i][li + 63 - jj] for jj = 8*n + 4*g + 3 .. + 0 is the window of four elements
+        // that starts at 4*chunk + (li & 3): a misaligned 8-byte LDS read is served lane by lane, so the
+        // two aligned chunks around the window are read and the window is cut out of them; every
+        // element is then added with one dot instruction.
+        const ST* c_rd = c2pS + (wave * 32 + li) * kC2pStride + 4 * ((li >> 2) + 15 - g);
+        const ST* p_rd = p2cS + (4 * g) * kP2cStride + (wave * 32 + li + 63 - 4 * g);
+        const bool c_odd_chunk = (li & 2) != 0;
+        const uint32_t c_shift = 16 * (li & 1);
+#pragma unroll
+        for (int n = 0; n < 8; ++n) {
+          const int jb = n >> 2, q = n & 3;
+          if constexpr (C2P) {
+            const u32x2 lo = *(const u32x2*)(c_rd - 8 * n), hi = *(const u32x2*)(c_rd - 8 * n + 4);
+            const uint32_t wa = c_odd_chunk ? lo[1] : lo[0], wb = c_odd_chunk ? hi[0] : lo[1], wc = c_odd_chunk ? hi[1] : hi[0];
+            const uint32_t w0 = __builtin_amdgcn_alignbit(wb, wa, c_shift), w1 = __builtin_amdgcn_alignbit(wc, wb, c_shift);
+            sacc[jb][4 * q + 0] = scratch_add_hi<ST>(sacc[jb][4 * q + 0], w1);
+            sacc[jb][4 * q + 1] = scratch_add_lo<ST>(sacc[jb][4 * q + 1], w1);
+            sacc[jb][4 * q + 2] = scratch_add_hi<ST>(sacc[jb][4 * q + 2], w0);
+            sacc[jb][4 * q + 3] = scratch_add_lo<ST>(sacc[jb][4 * q + 3], w0);
+          }
+          if constexpr (P2C) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const uint32_t x = *(const uint16_t*)(p_rd + (8 * n + e) * (kP2cStride - 1));
+              sacc[jb][4 * q + e] = scratch_add_lo<ST>(sacc[jb][4 * q + e], x);
+            }
+          }
+        }
+      } else {
         const ST* cbase = c2pS + (wave * 32 + li) * kC2pStride + (li + 63 - 4 * g);
         const ST* pbase = p2cS + (4 * g) * kP2cStride + (wave * 32 + li + 63 - 4 * g);
 #pragma unroll

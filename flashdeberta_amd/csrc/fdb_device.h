@@ -238,6 +238,24 @@ __device__ __forceinline__ f32x4 load4_scratch_unaligned<_Float16>(const _Float1
   return __builtin_convertvector(*(const f16x4_u*)p, f32x4);
 }
 
+// acc + the low / high element of a packed pair of 16-bit scratch values
+template <class ST>
+__device__ __forceinline__ float scratch_add_lo(float acc, uint32_t pair);
+template <class ST>
+__device__ __forceinline__ float scratch_add_hi(float acc, uint32_t pair);
+template <>
+__device__ __forceinline__ float scratch_add_lo<__bf16>(float acc, uint32_t pair) { return Bf16Tr::add_lo(acc, pair); }
+template <>
+__device__ __forceinline__ float scratch_add_hi<__bf16>(float acc, uint32_t pair) { return Bf16Tr::add_hi(acc, pair); }
+template <>
+__device__ __forceinline__ float scratch_add_lo<_Float16>(float acc, uint32_t pair) { return F16Tr::add_lo(acc, pair); }
+template <>
+__device__ __forceinline__ float scratch_add_hi<_Float16>(float acc, uint32_t pair) { return F16Tr::add_hi(acc, pair); }
+template <>
+__device__ __forceinline__ float scratch_add_lo<float>(float acc, uint32_t) { return acc; }  // fp32 scratch is read element-wise
+template <>
+__device__ __forceinline__ float scratch_add_hi<float>(float acc, uint32_t) { return acc; }
+
 // Linear workgroup id -> (query-tile index within the launch, head).  The hardware deals
 // workgroups to the 8 XCDs round-robin by linear id, and each XCD has its own L2.  In the fixed
 // layout, when the number of (sequence, head) groups is a multiple of 8, groups are dealt to XCDs
