@@ -177,8 +177,8 @@ int fdb_attn_fwd(const fdb_attn_args* a, void* stream) {
   if (grid_x < 1 || grid_x * a->heads > INT32_MAX) return FDB_ERR_SHAPE;
   p.grid_x = (int32_t)grid_x;
   // Split path: the far tiles in a far-only run of the kernel (three workgroups per CU), the near
-  // tiles in a second run (ring mode, one workgroup per CU), which merges the two.  It needs the
-  // log-sum-exp buffer as the hand-over between the two launches.
+  // tiles in a second launch, which merges the two.  It needs the log-sum-exp buffer as the
+  // hand-over between the two launches.
   if ((a->pos_key || a->pos_query) && a->lse && fdb_near_supported(a->dtype, a->head_dim)) {
     const bool need_far = a->max_seqlen > p.R + FDB_BN - 1;  // otherwise no tile of any query tile is far
     if (need_far) {
@@ -186,6 +186,8 @@ int fdb_attn_fwd(const fdb_attn_args* a, void* stream) {
       if (rc_far != 0) return rc_far;
     }
     p.far_done = need_far ? 1 : 0;
+    // head_dim 64: the near kernel (32-key steps, two workgroups per CU); head_dim 32: the fused kernel's ring mode
+    if (fdb_near32_supported(a->dtype, a->head_dim)) return fdb_launch_near32(p, a->dtype, (int)grid_x, stream);
     return fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, FDB_MODE_NEAR_RING, stream);
   }
   return fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, FDB_MODE_FUSED, stream);

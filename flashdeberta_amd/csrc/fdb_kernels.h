@@ -50,6 +50,10 @@ struct FdbKParams {
 enum { FDB_MODE_FUSED = 0, FDB_MODE_FAR_ONLY = 1, FDB_MODE_NEAR_RING = 2 };
 int fdb_launch_attn(const FdbKParams& p, int dtype, int head_dim, int grid_x, int mode, void* stream);
 bool fdb_near_supported(int dtype, int head_dim);
+// fdb_launch_near32: the near tiles in 32-key steps, 66 KB of LDS so that two workgroups share a CU
+// (16-bit element types, head_dim 64); merges the far partial like the ring mode.
+bool fdb_near32_supported(int dtype, int head_dim);
+int fdb_launch_near32(const FdbKParams& p, int dtype, int grid_x, void* stream);
 int fdb_launch_worklist(const int32_t* cu, int32_t batch, int32_t* wl, int32_t max_tiles, void* stream);
 int fdb_launch_quant(const void* x, int64_t x_st, int64_t x_sh, void* y, int64_t y_st, int64_t y_sh,
                      float* scale, uint32_t* absmax_ws, int32_t tokens, int32_t heads, int32_t head_dim,

@@ -1,0 +1,444 @@
+// Near tiles of the disentangled-attention forward for gfx950, head_dim 64, 16-bit types: the key
+// tiles of a query tile in which the bucketed relative position delta(i - j) is not constant
+// (|i - j| < R + tile size).  Second launch of the two-launch path: the far tiles' partial result
+// (rows normalised over the far keys in out, their log-sum-exp in lse) is merged in the epilogue.
+//
+// The position products need the rows E_K[r] = K_r[delta(r)] and E_Q[r] = Q_r[delta(r)] for the
+// contiguous range of relative positions r of a tile.  They are staged in LDS rings with coalesced
+// loads, so the MFMA A operands are plain LDS reads.
+//
+// What shapes this kernel is LDS: a wave alone on its SIMD issues a dependent instruction only
+// every eight to nine cycles, and nothing else hides that but a second wave.  Two workgroups share
+// a CU when each stays under 80 KB, which the rings allow only with 32-key steps:
+//   workgroup = 4 waves x 32 query rows, one step = 32 keys;
+//   a step sees 159 relative positions (5 batches of 32), and since the rows of the next step are
+//   stored after every wave has finished reading the ring in the current one, the rings hold
+//   exactly 5 batches = 160 rows of 128 bytes, unpadded and XOR-swizzled;
+//   a wave's 32 x 32 sub-tile sees 63 relative positions, so both position products are 2 MFMA row
+//   blocks, private to the wave: C[i][r] = q_i . E_K[r] and P[j][r] = k_j . E_Q[r] go, one after
+//   the other, through one per-wave LDS scratch from which element (i, j) reads index r = i - j.
+// LDS: K 4.5 KB + V 4.5 KB + rings 40 KB + scratch 17 KB = 66 KB.
+//
+// Staging rides inside the step, between its two barriers B1 (top: K, the ring rows and V's buffer
+// are ready / free) and B2 (every wave has its operands of the step out of LDS):
+//   after B1: V(s) registers -> LDS (read by the soft-max at the end of the step), V(s+1) global -> registers;
+//   after B2: K(s+1) and batch k+5 registers -> LDS, then K(s+2), the rows of batch k+6 and the table
+//             values of batch k+7 global -> registers.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "fdb_device.h"
+#include "fdb_kernels.h"
+#include "../../include/fdb.h"
+
+using namespace fdb;
+
+namespace {
+
+constexpr int kNThreads = 256;
+constexpr int kStep = 32;        // keys per step
+constexpr int kRingRows = 160;   // 5 batches of 32 relative positions
+constexpr int kScrStride = 68;   // elements per row of a wave's [32][64] bias scratch
+constexpr int kRowBytes = 128;   // head_dim 64, 16-bit
+constexpr int kKvStride = kRowBytes + 16;
+
+struct NCfg {
+  static constexpr int K_BYTES = kStep * kKvStride;
+  static constexpr int V_BYTES = kStep * kKvStride;
+  static constexpr int RING_BYTES = kRingRows * kRowBytes;
+  static constexpr int SCR_BYTES = 4 * 32 * kScrStride * 2;
+  static constexpr int lds_bytes(bool c2p, bool p2c) {
+    return K_BYTES + V_BYTES + (c2p ? RING_BYTES : 0) + (p2c ? RING_BYTES : 0) + SCR_BYTES;
+  }
+};
+
+// f(row) of the ring swizzle: slot (row, s) holds chunk s ^ f(row), f = 4*bit1(row) | bits3:2(row);
+// sixteen consecutive rows put one chunk in sixteen different bank groups.
+__device__ __forceinline__ int ring_f(int row) { return 4 * ((row >> 1) & 1) | ((row >> 2) & 3); }
+
+template <class QT, class VT, bool C2P, bool P2C>
+__global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams p) {
+  constexpr int D = 64, KS = 4, DBLKS = 2;
+  using ST = typename QT::scratch_t;
+  using qfrag = typename QT::frag;
+  using vfrag = typename VT::frag;
+  static_assert(QT::SZ == 2 && VT::SZ == 2, "16-bit element types only");
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  char* Ks = smem;                      // [32][144]
+  char* Vs = Ks + NCfg::K_BYTES;        // [32][144]
+  char* EK = Vs + NCfg::V_BYTES;        // [160][128] rows K_r[delta(r)], slot = (r_hi0 - r) mod 160
+  char* EQ = EK + (C2P ? NCfg::RING_BYTES : 0);
+  char* scr_raw = EQ + (P2C ? NCfg::RING_BYTES : 0);
+
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63, li = lane & 31, g = lane >> 5;
+  int xq, h;
+  block_map((int)blockIdx.x, p.grid_x, p.H, p.tiles_per_seq, p.cu == nullptr, xq, h);
+  ST* scr = (ST*)scr_raw + wave * (32 * kScrStride);
+
+  int b, m0, tok0, Lb;
+  int64_t qo, ko, vo, oo;
+  if (p.cu) {
+    if (xq >= p.wl[0]) return;
+    b = p.wl[2 + 2 * xq];
+    m0 = p.wl[3 + 2 * xq];
+    tok0 = p.cu[b];
+    Lb = p.cu[b + 1] - tok0;
+    qo = ko = vo = oo = 0;
+  } else {
+    b = xq / p.tiles_per_seq;
+    m0 = (xq % p.tiles_per_seq) * FDB_BM;
+    tok0 = p.seq_start ? min(max(p.seq_start[b], 0), p.L) : 0;
+    Lb = p.seq_len ? min(max(p.seq_len[b], 0), p.L - tok0) : p.L;
+    if (m0 >= Lb) return;
+    qo = b * p.q_sb; ko = b * p.k_sb; vo = b * p.v_sb; oo = b * p.o_sb;
+  }
+  const char* qb = p.q + (qo + (int64_t)tok0 * p.q_st + (int64_t)h * p.q_sh) * 2;
+  const char* kb = p.k + (ko + (int64_t)tok0 * p.k_st + (int64_t)h * p.k_sh) * 2;
+  const char* vb = p.v + (vo + (int64_t)tok0 * p.v_st + (int64_t)h * p.v_sh) * 2;
+  char* ob = p.out + (oo + (int64_t)tok0 * p.o_st + (int64_t)h * p.o_sh) * 2;
+  const char* pkb = C2P ? p.pk + (int64_t)h * p.pk_sh * 2 : nullptr;
+  const char* pqb = P2C ? p.pq + (int64_t)h * p.pq_sh * 2 : nullptr;
+  const uint32_t k_rsb = (uint32_t)(p.k_st * 2), v_rsb = (uint32_t)(p.v_st * 2);  // the host checks that they fit
+  const float x_scale = p.scale_log2;
+
+  const int iw0 = m0 + wave * 32;
+  const int i = iw0 + li;
+
+  qfrag qf[KS];
+#pragma unroll
+  for (int s = 0; s < KS; ++s)
+    qf[s] = (i < Lb) ? QT::load(qb + ((int64_t)i * p.q_st + 16 * s + 8 * g) * 2) : QT::zero();
+  // Consume the query loads here: left pending into the loop, their first use would make the
+  // compiler wait for every outstanding vector-memory load at the top of each step.
+#pragma unroll
+  for (int s = 0; s < KS; ++s) asm volatile("" ::"v"(qf[s]));
+
+  // ---- the near range: the 64-key tiles the far-only run skips, walked 32 keys at a time -----------
+  int j_end = Lb;
+  if (p.causal) j_end = min(Lb, m0 + FDB_BM);
+  const int n_tiles = (j_end + FDB_BN - 1) / FDB_BN;
+  const int lim = m0 - (FDB_BN - 1) - p.R;
+  const int t0 = lim >= 0 ? min(n_tiles, lim / FDB_BN + 1) : 0;
+  const int t1 = max(t0, min(n_tiles, (m0 + FDB_BM - 1 + p.R + FDB_BN - 1) / FDB_BN));
+  const int s0 = 2 * t0;                                                   // first 32-key step
+  const int s1 = max(s0, min(2 * t1, (j_end + kStep - 1) / kStep));        // one past the last
+  const int n_steps = s1 - s0;
+  const int n_full = p.causal ? 0 : max(0, min(n_steps, Lb / kStep - s0));  // steps k < n_full need no mask
+
+  // relative positions of the workgroup at step k = s - s0: r in [r_hi0 - 32k - 158, r_hi0 - 32k];
+  // u = r_hi0 - r counts downwards from the first step's largest r; ring slot = u mod 160; batch = u / 32.
+  const int r_hi0 = m0 + FDB_BM - 1 - s0 * kStep;
+
+  // ---- staging: one 16-byte chunk per thread of K, of V and of one batch of each ring ----------------
+  const int srow = tid >> 3, scc = tid & 7;
+  const int ring_wr = srow * kRowBytes + ((scc ^ ring_f(srow)) * 16);  // within a batch's segment
+  u32x4 kreg = {0, 0, 0, 0}, vreg = {0, 0, 0, 0}, ekreg = {0, 0, 0, 0}, eqreg = {0, 0, 0, 0};
+  int dnext = 0;
+  auto k_load = [&](int s) __attribute__((always_inline)) {
+    const int row = min(s * kStep + srow, Lb - 1);  // rows past the end re-read the last one; their scores are masked
+    kreg = *(const u32x4*)(kb + (uint64_t)(uint32_t)row * k_rsb + scc * 16);
+  };
+  auto v_load = [&](int s) __attribute__((always_inline)) {
+    const int row = min(s * kStep + srow, Lb - 1);
+    vreg = *(const u32x4*)(vb + (uint64_t)(uint32_t)row * v_rsb + scc * 16);
+  };
+  auto batch_delta = [&](int batch) __attribute__((always_inline)) {  // table row of this thread's ring row
+    const int r = r_hi0 - (batch * 32 + srow);
+    return (int)p.lut[max(-p.R, min(p.R, r)) + p.R];
+  };
+  auto batch_load = [&](int delta) __attribute__((always_inline)) {
+    if constexpr (C2P) ekreg = *(const u32x4*)(pkb + (int64_t)delta * p.pk_sr * 2 + scc * 16);
+    if constexpr (P2C) eqreg = *(const u32x4*)(pqb + (int64_t)delta * p.pq_sr * 2 + scc * 16);
+  };
+  auto batch_store = [&](int batch) __attribute__((always_inline)) {
+    const int seg = (batch % 5) * (32 * kRowBytes);
+    if constexpr (C2P) *(u32x4*)(EK + seg + ring_wr) = ekreg;
+    if constexpr (P2C) *(u32x4*)(EQ + seg + ring_wr) = eqreg;
+  };
+
+  f32x16 o_acc[DBLKS];
+#pragma unroll
+  for (int d = 0; d < DBLKS; ++d)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) o_acc[d][v] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  // ---- prologue: step 0's K and ring batches 0..4 to LDS; V(0), K(1), batch 5 in the registers --------
+  if (n_steps > 0) {
+    k_load(s0);
+    *(u32x4*)(Ks + srow * kKvStride + scc * 16) = kreg;
+#pragma unroll 1
+    for (int bt = 0; bt < 5; ++bt) {
+      batch_load(batch_delta(bt));
+      batch_store(bt);
+    }
+    v_load(s0);
+    if (n_steps > 1) {
+      k_load(s0 + 1);
+      batch_load(batch_delta(5));
+      dnext = batch_delta(6);
+    }
+  }
+
+  // ---- per-lane constants ------------------------------------------------------------------------------
+  // A row (block bk, lane li) of the wave's sub-tile at step k: r = iw0 - 32s - 31 + 32bk + li, i.e.
+  // u = 158 + 32k - 32*(wave + bk) - li; its slot keeps the low five bits of 158 - li for ever.
+  const int fr = ring_f(158 - li);
+  uint32_t rlx[KS];  // chunk 2s + g of the row sits in slot (2s) ^ g ^ f
+#pragma unroll
+  for (int s = 0; s < KS; ++s) rlx[s] = ((g ^ fr) * 16) ^ (32 * s);
+  int slot0 = (158 - li + 32 * ((5 - wave) % 5)) % kRingRows;  // block 0 at step 0 (u = 158 - li - 32*wave, mod 160)
+  const char* Kt = Ks + li * kKvStride + 8 * g * 2;
+  // scratch: C[i = li][r - r_lo], P[jj = li][r - r_lo]; element (jj = 8q + 4g + e, i = li) reads index li + 31 - jj.
+  // C's window of four elements starts at li + 28 - 4g - 8q = 4*chunk + (li & 3): two aligned chunks are
+  // read and the window is cut out (a misaligned 8-byte LDS read is served lane by lane).
+  const ST* c_rd = scr + li * kScrStride + 4 * ((li >> 2) + 7 - g);
+  const bool c_odd_chunk = (li & 2) != 0;
+  const uint32_t c_shift = 16 * (li & 1);
+  const ST* p_rd = scr + (4 * g) * kScrStride + (li + 31 - 4 * g);  // P[jj][.], plus cj * (stride - 1)
+  ST* scr_wr = scr + li * kScrStride + 4 * g;                       // row = this lane's MFMA column
+
+  // Block 1 of a step holds the rows that were block 0 of the step before: the A operands stay in
+  // registers for two steps, in two buffers that swap roles (the loop is unrolled over the parity),
+  // and a step reads only its new block 0 from the rings.
+  qfrag ac[2][C2P ? KS : 1], aq[2][P2C ? KS : 1];
+  auto ring_read = [&](int buf, int slot) __attribute__((always_inline)) {
+#pragma unroll
+    for (int x = 0; x < KS; ++x) {
+      if constexpr (C2P) ac[buf][x] = QT::load(EK + slot * kRowBytes + rlx[x]);
+      if constexpr (P2C) aq[buf][x] = QT::load(EQ + slot * kRowBytes + rlx[x]);
+    }
+  };
+  if (n_steps > 0) {
+    __syncthreads();  // the prologue's ring rows
+    ring_read(1, slot0 >= 32 ? slot0 - 32 : slot0 + (kRingRows - 32));  // block 1 of step 0
+  }
+
+  auto step = [&](auto mask_tag, auto par_tag, int k) __attribute__((always_inline)) {
+    constexpr bool MASK = decltype(mask_tag)::value;
+    constexpr int PAR = decltype(par_tag)::value;  // buffer of this step's block 0
+    const int s = s0 + k;
+    const int j0 = s * kStep;
+    __syncthreads();  // B1
+    // ---- operands of the step out of LDS ------------------------------------------------------------------
+    qfrag kf[KS];
+#pragma unroll
+    for (int x = 0; x < KS; ++x) kf[x] = QT::load(Kt + 16 * x * 2);
+    ring_read(PAR, slot0);
+    // V of this step to LDS, V of the next one on its way
+    *(u32x4*)(Vs + srow * kKvStride + scc * 16) = vreg;
+    if (k + 1 < n_steps) v_load(s + 1);
+    // ---- the five products, the position ones through the wave's scratch ------------------------------------
+    // C, then the content product (independent work while C drains), C to the scratch; only then P, in the
+    // registers C has left (the fence below keeps the two from being live together); after B2 and the
+    // staging, C's skewed diagonal is read, P is written over it and read.  The LDS unit runs one wave's
+    // operations in order, so the reads of C are served before the writes of P that follow them; only the
+    // compiler needs the fences.
+    f32x16 sacc, zero;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) zero[v] = 0.f;
+    u32x4 cw[4];
+    uint32_t px[16];
+    if constexpr (C2P) {
+      f32x16 cacc[2];
+#pragma unroll
+      for (int bk = 0; bk < 2; ++bk)
+#pragma unroll
+        for (int x = 0; x < KS; ++x) cacc[bk] = QT::mma(ac[PAR ^ bk][x], qf[x], x == 0 ? zero : cacc[bk]);
+#pragma unroll
+      for (int x = 0; x < KS; ++x) sacc = QT::mma(kf[x], qf[x], x == 0 ? zero : sacc);
+#pragma unroll
+      for (int bk = 0; bk < 2; ++bk)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4)  // C[i = li][32*bk + 8*q4 + 4*g + 0..3]
+          store4_scratch<ST>(scr_wr + 32 * bk + 8 * q4, cacc[bk][4 * q4], cacc[bk][4 * q4 + 1], cacc[bk][4 * q4 + 2],
+                             cacc[bk][4 * q4 + 3]);
+      __builtin_amdgcn_sched_barrier(0);
+    } else {
+#pragma unroll
+      for (int x = 0; x < KS; ++x) sacc = QT::mma(kf[x], qf[x], x == 0 ? zero : sacc);
+    }
+    f32x16 pacc[2];
+    if constexpr (P2C) {
+#pragma unroll
+      for (int bk = 0; bk < 2; ++bk)
+#pragma unroll
+        for (int x = 0; x < KS; ++x) pacc[bk] = QT::mma(aq[PAR ^ bk][x], kf[x], x == 0 ? zero : pacc[bk]);
+    }
+    // ---- B2: nobody reads K or the ring of this step from LDS any more --------------------------------------
+    __syncthreads();
+    if (k + 1 < n_steps) {
+      *(u32x4*)(Ks + srow * kKvStride + scc * 16) = kreg;
+      batch_store(k + 5);
+      if (k + 2 < n_steps) {
+        batch_load(dnext);  // its table value was loaded a step ago: no wait on the loads issued below
+        k_load(s + 2);
+        if (k + 3 < n_steps) dnext = batch_delta(k + 7);
+      }
+    }
+    if constexpr (C2P) {
+      wave_lds_fence();
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const u32x2 lo = *(const u32x2*)(c_rd - 8 * q4), hi = *(const u32x2*)(c_rd - 8 * q4 + 4);
+        cw[q4] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+      }
+      wave_lds_fence();
+    }
+    if constexpr (P2C) {
+#pragma unroll
+      for (int bk = 0; bk < 2; ++bk)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4)  // P[jj = li][32*bk + 8*q4 + 4*g + 0..3]
+          store4_scratch<ST>(scr_wr + 32 * bk + 8 * q4, pacc[bk][4 * q4], pacc[bk][4 * q4 + 1], pacc[bk][4 * q4 + 2],
+                             pacc[bk][4 * q4 + 3]);
+      wave_lds_fence();
+#pragma unroll
+      for (int v = 0; v < 16; ++v) px[v] = *(const uint16_t*)(p_rd + (8 * (v >> 2) + (v & 3)) * (kScrStride - 1));
+      wave_lds_fence();
+    }
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      if constexpr (C2P) {
+        const u32x4 d = cw[q4];
+        const uint32_t wa = c_odd_chunk ? d[1] : d[0], wb = c_odd_chunk ? d[2] : d[1], wc = c_odd_chunk ? d[3] : d[2];
+        const uint32_t w0 = __builtin_amdgcn_alignbit(wb, wa, c_shift), w1 = __builtin_amdgcn_alignbit(wc, wb, c_shift);
+        sacc[4 * q4 + 0] = QT::add_hi(sacc[4 * q4 + 0], w1);  // window elements 3, 2, 1, 0 for jj offsets 0, 1, 2, 3
+        sacc[4 * q4 + 1] = QT::add_lo(sacc[4 * q4 + 1], w1);
+        sacc[4 * q4 + 2] = QT::add_hi(sacc[4 * q4 + 2], w0);
+        sacc[4 * q4 + 3] = QT::add_lo(sacc[4 * q4 + 3], w0);
+      }
+      if constexpr (P2C) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sacc[4 * q4 + e] = QT::add_lo(sacc[4 * q4 + e], px[4 * q4 + e]);
+      }
+    }
+    // ---- mask, online soft-max in base 2, O^T += V^T P^T ---------------------------------------------------
+    if constexpr (MASK) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int j = j0 + 8 * (v >> 2) + 4 * g + (v & 3);
+        if (j >= Lb || (p.causal && j > i)) sacc[v] = -INFINITY;
+      }
+    }
+    float mx = sacc[0];
+#pragma unroll
+    for (int v = 1; v < 16; ++v) mx = fmaxf(mx, sacc[v]);
+    mx = wave_half_max(mx) * x_scale;  // x_scale > 0
+    if (__any(mx > m_run + kLazyTau)) {
+      const float m_new = (mx > m_run + kLazyTau) ? mx : m_run;
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // m_run = -inf before the first visible key: 0
+      l_run *= alpha;
+      m_run = m_new;
+#pragma unroll
+      for (int d = 0; d < DBLKS; ++d)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o_acc[d][v] *= alpha;
+    }
+    const float off = (MASK && m_run == -INFINITY) ? 0.f : -m_run;  // a row that has seen no visible key yet
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      f32x8 pv;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) pv[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[8 * c + e], x_scale, off));
+      const vfrag pf = VT::from_f32(pv);
+      l_run = VT::sum8(pf, l_run);
+#pragma unroll
+      for (int d = 0; d < DBLKS; ++d) {
+        const vfrag vf = VtLoad<VT>::get(Vs, kKvStride, c, d, lane);
+        o_acc[d] = VT::mma(vf, pf, o_acc[d]);
+      }
+    }
+    slot0 = slot0 + 32 >= kRingRows ? slot0 + 32 - kRingRows : slot0 + 32;
+  };
+  {
+    using T0 = std::integral_constant<int, 0>;
+    using T1 = std::integral_constant<int, 1>;
+    int k = 0;
+#pragma unroll 1
+    for (; k + 1 < n_full; k += 2) {
+      step(std::false_type{}, T0{}, k);
+      step(std::false_type{}, T1{}, k + 1);
+    }
+    if (k < n_full) {
+      step(std::false_type{}, T0{}, k);
+      ++k;
+    }
+    if ((k & 1) && k < n_steps) {
+      step(std::true_type{}, T1{}, k);
+      ++k;
+    }
+#pragma unroll 1
+    for (; k + 1 < n_steps; k += 2) {
+      step(std::true_type{}, T0{}, k);
+      step(std::true_type{}, T1{}, k + 1);
+    }
+    if (k < n_steps) step(std::true_type{}, T0{}, k);
+  }
+
+  // ---- epilogue: merge with the far tiles' partial result, normalise, store ------------------------------
+  const float l_tot = wave_half_sum(l_run);
+  if (i < Lb) {
+    char* orow = ob + (int64_t)i * p.o_st * 2;
+    const int64_t tok = p.cu ? (int64_t)tok0 + i : (int64_t)b * p.L + tok0 + i;
+    float w_far = 0.f, w_near = 1.f, m_out = m_run;
+    if (p.far_done) {
+      const float lf = p.lse[tok * p.H + h] * 1.4426950408889634f;  // far log-sum-exp, base 2 (-inf: no far tile)
+      const float ln_ = m_run + __builtin_amdgcn_logf(l_tot);
+      m_out = fmaxf(lf, ln_);
+      w_far = __builtin_amdgcn_exp2f(lf - m_out);
+      w_near = __builtin_amdgcn_exp2f(m_run - m_out);
+    }
+    const float denom = w_far + w_near * l_tot;
+    const float inv = denom > 0.f ? 1.f / denom : 0.f;
+    const float sn = w_near * inv, sf = w_far * inv;
+#pragma unroll
+    for (int d = 0; d < DBLKS; ++d)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        char* dst = orow + (32 * d + 8 * q4 + 4 * g) * 2;
+        float f0 = 0.f, f1 = 0.f, f2 = 0.f, f3 = 0.f;
+        if (p.far_done) {
+          const f32x4 far4 = VT::load4(dst);
+          f0 = far4[0] * sf; f1 = far4[1] * sf; f2 = far4[2] * sf; f3 = far4[3] * sf;
+        }
+        VT::store4(dst, o_acc[d][4 * q4] * sn + f0, o_acc[d][4 * q4 + 1] * sn + f1, o_acc[d][4 * q4 + 2] * sn + f2,
+                   o_acc[d][4 * q4 + 3] * sn + f3);
+      }
+    if (p.lse && g == 0) p.lse[tok * p.H + h] = (m_out + __builtin_amdgcn_logf(denom)) * 0.6931471805599453f;
+  }
+}
+
+template <class QT, bool C2P, bool P2C>
+int launch_near_one(const FdbKParams& p, int grid_x, hipStream_t stream) {
+  auto kern = fdb_near_kernel<QT, QT, C2P, P2C>;
+  constexpr int lds = NCfg::lds_bytes(C2P, P2C);
+  static_assert(lds <= 80 * 1024, "two workgroups per CU");
+  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+  if (e != hipSuccess) return (int)e;
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid_x * p.H, 1, 1), dim3(kNThreads), lds, stream, p);
+  return (int)hipGetLastError();
+}
+
+template <class QT>
+int launch_near_pos(const FdbKParams& p, int grid_x, hipStream_t stream) {
+  if (p.pk && p.pq) return launch_near_one<QT, true, true>(p, grid_x, stream);
+  if (p.pk) return launch_near_one<QT, true, false>(p, grid_x, stream);
+  if (p.pq) return launch_near_one<QT, false, true>(p, grid_x, stream);
+  return FDB_ERR_UNSUPPORTED;
+}
+
+}  // namespace
+
+bool fdb_near32_supported(int dtype, int head_dim) {
+  return (dtype == FDB_BF16 || dtype == FDB_F16) && head_dim == 64;
+}
+
+int fdb_launch_near32(const FdbKParams& p, int dtype, int grid_x, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (dtype == FDB_BF16) return launch_near_pos<Bf16Tr>(p, grid_x, stream);
+  if (dtype == FDB_F16) return launch_near_pos<F16Tr>(p, grid_x, stream);
+  return FDB_ERR_UNSUPPORTED;
+}
