@@ -17,7 +17,7 @@
 //   a wave's 32 x 32 sub-tile sees 63 relative positions, so both position products are 2 MFMA row
 //   blocks, private to the wave: C[i][r] = q_i . E_K[r] and P[j][r] = k_j . E_Q[r] go, one after
 //   the other, through one per-wave LDS scratch from which element (i, j) reads index r = i - j.
-// LDS: K 4.5 KB + V 4.5 KB + rings 40 KB + scratch 17 KB = 66 KB.
+// LDS: K 4 KB + V 4 KB + rings 40 KB + scratch 17 KB = 65 KB.
 //
 // Staging rides inside the step, between its two barriers B1 (top: K, the ring rows and V's buffer
 // are ready / free) and B2 (every wave has its operands of the step out of LDS):
@@ -40,11 +40,10 @@ constexpr int kStep = 32;        // keys per step
 constexpr int kRingRows = 160;   // 5 batches of 32 relative positions
 constexpr int kScrStride = 68;   // elements per row of a wave's [32][64] bias scratch
 constexpr int kRowBytes = 128;   // head_dim 64, 16-bit
-constexpr int kKvStride = kRowBytes + 16;
 
 struct NCfg {
-  static constexpr int K_BYTES = kStep * kKvStride;
-  static constexpr int V_BYTES = kStep * kKvStride;
+  static constexpr int K_BYTES = kStep * kRowBytes;  // K and V rows are swizzled like the ring rows
+  static constexpr int V_BYTES = kStep * kRowBytes;
   static constexpr int RING_BYTES = kRingRows * kRowBytes;
   static constexpr int SCR_BYTES = 4 * 32 * kScrStride * 2;
   static constexpr int lds_bytes(bool c2p, bool p2c) {
@@ -64,8 +63,8 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
   using vfrag = typename VT::frag;
   static_assert(QT::SZ == 2 && VT::SZ == 2, "16-bit element types only");
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  char* Ks = smem;                      // [32][144]
-  char* Vs = Ks + NCfg::K_BYTES;        // [32][144]
+  char* Ks = smem;                      // [32][128]
+  char* Vs = Ks + NCfg::K_BYTES;        // [32][128]
   char* EK = Vs + NCfg::V_BYTES;        // [160][128] rows K_r[delta(r)], slot = (r_hi0 - r) mod 160
   char* EQ = EK + (C2P ? NCfg::RING_BYTES : 0);
   char* scr_raw = EQ + (P2C ? NCfg::RING_BYTES : 0);
@@ -168,7 +167,7 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
   // ---- prologue: step 0's K and ring batches 0..4 to LDS; V(0), K(1), batch 5 in the registers --------
   if (n_steps > 0) {
     k_load(s0);
-    *(u32x4*)(Ks + srow * kKvStride + scc * 16) = kreg;
+    *(u32x4*)(Ks + ring_wr) = kreg;
 #pragma unroll 1
     for (int bt = 0; bt < 5; ++bt) {
       batch_load(batch_delta(bt));
@@ -190,7 +189,18 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
 #pragma unroll
   for (int s = 0; s < KS; ++s) rlx[s] = ((g ^ fr) * 16) ^ (32 * s);
   int slot0 = (158 - li + 32 * ((5 - wave) % 5)) % kRingRows;  // block 0 at step 0 (u = 158 - li - 32*wave, mod 160)
-  const char* Kt = Ks + li * kKvStride + 8 * g * 2;
+  uint32_t klx[KS], vlx[4];  // K fragment rows li; V^T operand (c, d-block db, half h): row 16c + 8h + 4*(grp/2) + s16/4,
+                             // 8-byte unit 8db + 4*(grp%2) + s16%4, i.e. chunk ^ f = lane part ^ (4db) ^ (2h)
+  {
+    const int s16 = lane & 15, grp = lane >> 4;
+    const int slotl = (2 * (grp & 1) + ((s16 & 3) >> 1)) ^ (4 * ((s16 >> 3) & 1)) ^ (grp >> 1);
+    const uint32_t vlane = (4 * (grp >> 1) + (s16 >> 2)) * kRowBytes + slotl * 16 + (s16 & 1) * 8;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      klx[x] = (li * kRowBytes + ((g ^ ring_f(li)) * 16)) ^ (32 * x);
+      vlx[x] = vlane ^ (64 * (x >> 1) ^ 32 * (x & 1));
+    }
+  }
   // scratch: C[i = li][r - r_lo], P[jj = li][r - r_lo]; element (jj = 8q + 4g + e, i = li) reads index li + 31 - jj.
   // C's window of four elements starts at li + 28 - 4g - 8q = 4*chunk + (li & 3): two aligned chunks are
   // read and the window is cut out (a misaligned 8-byte LDS read is served lane by lane).
@@ -225,10 +235,10 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
     // ---- operands of the step out of LDS ------------------------------------------------------------------
     qfrag kf[KS];
 #pragma unroll
-    for (int x = 0; x < KS; ++x) kf[x] = QT::load(Kt + 16 * x * 2);
+    for (int x = 0; x < KS; ++x) kf[x] = QT::load(Ks + klx[x]);
     ring_read(PAR, slot0);
     // V of this step to LDS, V of the next one on its way
-    *(u32x4*)(Vs + srow * kKvStride + scc * 16) = vreg;
+    *(u32x4*)(Vs + ring_wr) = vreg;
     if (k + 1 < n_steps) v_load(s + 1);
     // ---- the five products, the position ones through the wave's scratch ------------------------------------
     // C, then the content product (independent work while C drains), C to the scratch; only then P, in the
@@ -270,7 +280,7 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
     // ---- B2: nobody reads K or the ring of this step from LDS any more --------------------------------------
     __syncthreads();
     if (k + 1 < n_steps) {
-      *(u32x4*)(Ks + srow * kKvStride + scc * 16) = kreg;
+      *(u32x4*)(Ks + ring_wr) = kreg;
       batch_store(k + 5);
       if (k + 2 < n_steps) {
         batch_load(dnext);  // its table value was loaded a step ago: no wait on the loads issued below
@@ -347,7 +357,9 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
       l_run = VT::sum8(pf, l_run);
 #pragma unroll
       for (int d = 0; d < DBLKS; ++d) {
-        const vfrag vf = VtLoad<VT>::get(Vs, kKvStride, c, d, lane);
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(Vs + vlx[2 * d] + 2048 * c));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(Vs + vlx[2 * d + 1] + 2048 * c + 1024));
+        const vfrag vf = __builtin_bit_cast(vfrag, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
         o_acc[d] = VT::mma(vf, pf, o_acc[d]);
       }
     }
