@@ -373,15 +373,19 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
     const int slotl = (2 * (grp & 1) + ((s16 & 3) >> 1)) ^ (4 * ((s16 >> 3) & 1)) ^ (grp >> 1);  // chunk ^ f, less (4db) ^ (2h)
     vlane = (4 * (grp >> 1) + (s16 >> 2)) * 128 + slotl * 16 + (s16 & 1) * 8;
   }
+  // The tile's first row travels as the scalar base of the load, the lane's place in the tile as
+  // its offset: the row is clamped to the last one of the sequence (rows past the end re-read it).
   auto dma_issue = [&](int tile, int bufoff) __attribute__((always_inline)) {
+    const char* kt = kb + (uint64_t)(uint32_t)(tile * FDB_BN) * k_rsb;
+    const char* vt = vb + (uint64_t)(uint32_t)(tile * FDB_BN) * v_rsb;
+    const int last = Lb - 1 - tile * FDB_BN;
 #pragma unroll
     for (int q2 = 0; q2 < 2; ++q2) {  // this wave's two 8-row groups of K and of V
-      const int row = 16 * wave + 8 * q2 + (lane >> 3);
-      const uint32_t c = (lane & 7) ^ (4 * ((lane >> 4) & 1)) ^ (lane >> 5) ^ (2 * q2);  // slot ^ f(row)
-      const uint32_t rg = (uint32_t)min(tile * FDB_BN + row, Lb - 1);  // rows past the end re-read the last one
+      const uint32_t row = (uint32_t)min(16 * wave + 8 * q2 + (lane >> 3), last);
+      const uint32_t c16 = ((lane & 7) ^ (4 * ((lane >> 4) & 1)) ^ (lane >> 5) ^ (2 * q2)) * 16;  // slot ^ f(row), unclamped row
       const uint32_t dst = lds0 + bufoff + (2 * wave + q2) * 1024;
-      dma16(kb + (uint64_t)rg * k_rsb + c * 16, dst);
-      dma16(vb + (uint64_t)rg * v_rsb + c * 16, dst + C::DMA_TILE);
+      dma16s(kt, row * k_rsb + c16, dst);
+      dma16s(vt, row * v_rsb + c16, dst + C::DMA_TILE);
     }
   };
   {

@@ -283,6 +283,15 @@ __device__ __forceinline__ void dma16(const void* g, uint32_t lds_base) {
   const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(base) : "memory");
 }
+// The same with the address split into a base that is the same in every lane (it travels in scalar
+// registers) and this lane's 32-bit byte offset from it.
+__device__ __forceinline__ void dma16s(const void* base, uint32_t lane_off, uint32_t lds_base) {
+  const uint32_t lb = __builtin_amdgcn_readfirstlane(lds_base);
+  const uint64_t b64 = (uint64_t)(uintptr_t)base;
+  const uint32_t blo = __builtin_amdgcn_readfirstlane((uint32_t)b64), bhi = __builtin_amdgcn_readfirstlane((uint32_t)(b64 >> 32));
+  const uint64_t sb = ((uint64_t)bhi << 32) | blo;
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(sb), "s"(lb) : "memory");
+}
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   static_assert(N == 0 || N == 4, "counts used by the kernels");
