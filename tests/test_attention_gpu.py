@@ -129,6 +129,25 @@ def test_one_kernel_and_two_kernel_paths_agree(dtype, B, L, pb, mr):
     assert (two.float() - one.float()).abs().max().item() <= TOL[dtype]
 
 
+@pytest.mark.parametrize("causal,c2p,p2c,D,L", [
+    (True, True, True, 64, 1400),    # causal across the far / near boundary
+    (False, True, False, 64, 1300),  # one position term only, both launches
+    (False, False, True, 64, 1300),
+    (False, True, True, 32, 1300),   # head_dim 32: far-only + ring mode
+    (True, True, True, 32, 700),
+    (False, True, True, 64, 1153),   # ragged last step of 32 keys (1153 = 36*32 + 1)
+])
+def test_two_launch_variants(causal, c2p, p2c, D, L):
+    """The far-only launch followed by the near launch, over the combinations that select different
+    kernels (one or two position terms, causal, head_dim 32 / 64, ragged tails)."""
+    q, k, v, pk, pq = _inputs(2, L, 2, D, 256, 512, torch.bfloat16, 31 + L, 1.0, c2p, p2c)
+    ref, ref_lse = _oracle_blhd(q, k, v, pk, pq, 256, 512, causal=causal, return_lse=True)
+    out, lse = ops.disentangled_attention_fwd(_dev(q), _dev(k), _dev(v), _dev(pk), _dev(pq), position_buckets=256,
+                                              max_relative_positions=512, causal=causal, return_lse=True)
+    _check(out, ref, TOL[torch.bfloat16], "out")
+    _check(lse.view(2, L, 2), ref_lse, 4 * TOL[torch.bfloat16], "lse")
+
+
 # ---- delta indices are bit-exact inside the kernel ----------------------------------------------
 @pytest.mark.parametrize("pb,mr,L", [(256, 512, 1200), (32, 64, 300), (0, 40, 130)])
 @pytest.mark.parametrize("term", ["c2p", "p2c"])
