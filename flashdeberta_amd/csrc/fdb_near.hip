@@ -16,8 +16,9 @@
 //   exactly 5 batches = 160 rows of 128 bytes, unpadded and XOR-swizzled;
 //   a wave's 32 x 32 sub-tile sees 63 relative positions, so both position products are 2 MFMA row
 //   blocks, private to the wave: C[i][r] = q_i . E_K[r] and P[j][r] = k_j . E_Q[r] go, one after
-//   the other, through one per-wave LDS scratch from which element (i, j) reads index r = i - j.
-// LDS: K 4 KB + V 4 KB + rings 40 KB + scratch 17 KB = 65 KB.
+//   the other, through one per-wave fp32 LDS scratch from which element (i, j) reads index r = i - j;
+//   C's values come back as the initial value of the content product's accumulator.
+// LDS: K 4 KB + V 4 KB + rings 40 KB + scratch 18.5 KB = 66.5 KB.
 //
 // Staging rides inside the step, between its two barriers B1 (top: K, the ring rows and V's buffer
 // are ready / free) and B2 (every wave has its operands of the step out of LDS):
@@ -38,14 +39,15 @@ namespace {
 constexpr int kNThreads = 256;
 constexpr int kStep = 32;        // keys per step
 constexpr int kRingRows = 160;   // 5 batches of 32 relative positions
-constexpr int kScrStride = 68;   // elements per row of a wave's [32][64] bias scratch
+constexpr int kScrW = 36;        // fp32 words between the rows of a wave's bias scratch (rows overlap, see below)
+constexpr int kScrWords = 32 * kScrW + 32;  // row 31 reaches column 63
 constexpr int kRowBytes = 128;   // head_dim 64, 16-bit
 
 struct NCfg {
   static constexpr int K_BYTES = kStep * kRowBytes;  // K and V rows are swizzled like the ring rows
   static constexpr int V_BYTES = kStep * kRowBytes;
   static constexpr int RING_BYTES = kRingRows * kRowBytes;
-  static constexpr int SCR_BYTES = 4 * 32 * kScrStride * 2;
+  static constexpr int SCR_BYTES = 4 * kScrWords * 4;
   static constexpr int lds_bytes(bool c2p, bool p2c) {
     return K_BYTES + V_BYTES + (c2p ? RING_BYTES : 0) + (p2c ? RING_BYTES : 0) + SCR_BYTES;
   }
@@ -58,7 +60,6 @@ __device__ __forceinline__ int ring_f(int row) { return 4 * ((row >> 1) & 1) | (
 template <class QT, class VT, bool C2P, bool P2C>
 __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams p) {
   constexpr int D = 64, KS = 4, DBLKS = 2;
-  using ST = typename QT::scratch_t;
   using qfrag = typename QT::frag;
   using vfrag = typename VT::frag;
   static_assert(QT::SZ == 2 && VT::SZ == 2, "16-bit element types only");
@@ -74,7 +75,7 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
   const int lane = tid & 63, li = lane & 31, g = lane >> 5;
   int xq, h;
   block_map((int)blockIdx.x, p.grid_x, p.H, p.tiles_per_seq, p.cu == nullptr, xq, h);
-  ST* scr = (ST*)scr_raw + wave * (32 * kScrStride);
+  float* scr = (float*)scr_raw + wave * kScrWords;
 
   int b, m0, tok0, Lb;
   int64_t qo, ko, vo, oo;
@@ -136,7 +137,9 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
   u32x4 kreg = {0, 0, 0, 0}, vreg = {0, 0, 0, 0}, ekreg = {0, 0, 0, 0}, eqreg = {0, 0, 0, 0};
   int dnext = 0;
   auto k_load = [&](int s) __attribute__((always_inline)) {
-    const int row = min(s * kStep + srow, Lb - 1);  // rows past the end re-read the last one; their scores are masked
+    // LDS row srow holds key srow ^ 3 of the step (see the scratch reads below); rows past the end
+    // re-read the last one, their scores are masked
+    const int row = min(s * kStep + (srow ^ 3), Lb - 1);
     kreg = *(const u32x4*)(kb + (uint64_t)(uint32_t)row * k_rsb + scc * 16);
   };
   auto v_load = [&](int s) __attribute__((always_inline)) {
@@ -145,7 +148,9 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
   };
   auto batch_delta = [&](int batch) __attribute__((always_inline)) {  // table row of this thread's ring row
     const int r = r_hi0 - (batch * 32 + srow);
-    return (int)p.lut[max(-p.R, min(p.R, r)) + p.R];
+    // table rows are indices >= 0: read unsigned, so that the loaded register is the value and nothing
+    // has to wait for the load before the next step uses it
+    return (int)((const uint16_t*)p.lut)[max(-p.R, min(p.R, r)) + p.R];
   };
   auto batch_load = [&](int delta) __attribute__((always_inline)) {
     if constexpr (C2P) ekreg = *(const u32x4*)(pkb + (int64_t)delta * p.pk_sr * 2 + scc * 16);
@@ -174,11 +179,9 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
       batch_store(bt);
     }
     v_load(s0);
-    if (n_steps > 1) {
-      k_load(s0 + 1);
-      batch_load(batch_delta(5));
-      dnext = batch_delta(6);
-    }
+    k_load(s0 + 1);
+    batch_load(batch_delta(5));
+    dnext = batch_delta(6);
   }
 
   // ---- per-lane constants ------------------------------------------------------------------------------
@@ -201,14 +204,31 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
       vlx[x] = vlane ^ (64 * (x >> 1) ^ 32 * (x & 1));
     }
   }
-  // scratch: C[i = li][r - r_lo], P[jj = li][r - r_lo]; element (jj = 8q + 4g + e, i = li) reads index li + 31 - jj.
-  // C's window of four elements starts at li + 28 - 4g - 8q = 4*chunk + (li & 3): two aligned chunks are
-  // read and the window is cut out (a misaligned 8-byte LDS read is served lane by lane).
-  const ST* c_rd = scr + li * kScrStride + 4 * ((li >> 2) + 7 - g);
-  const bool c_odd_chunk = (li & 2) != 0;
-  const uint32_t c_shift = 16 * (li & 1);
-  const ST* p_rd = scr + (4 * g) * kScrStride + (li + 31 - 4 * g);  // P[jj][.], plus cj * (stride - 1)
-  ST* scr_wr = scr + li * kScrStride + 4 * g;                       // row = this lane's MFMA column
+  // scratch (fp32, so no conversion and no sub-word extraction): C[i = li][rr], P[jj = li][rr] with
+  // rr = r - r_lo in 0..63; element (jj = 8q + 4g + e, i = li) reads C[li][li + 31 - jj] and
+  // P[jj][li + 31 - jj].  Only a band of 32 columns of each row is ever read (C: rr in [li, li + 31],
+  // P: rr in [31 - jj, 62 - jj]), so the rows are laid 36 words apart and overlap: the bands (plus the
+  // three columns a four-column group may stick out on either side) stay disjoint, and a lane does not
+  // write the groups of its row that lie wholly outside the band.
+  // K's rows sit in LDS with the low two bits of the row index inverted, so MFMA row m = 8q + 4g + e of
+  // the content product is key jj = 8q + 4g + 3 - e: the four C elements a lane adds to consecutive
+  // accumulator registers then lie at ascending addresses and can be read in pairs straight into the
+  // accumulator's registers.  P's column of lane li is therefore key li ^ 3.
+  const int lj = li ^ 3;
+  float* c_wrp = scr + li * kScrW + 4 * g;  // row = this lane's MFMA column; group (bk, q4) at + 32 bk + 8 q4
+  float* p_wrp = scr + lj * kScrW + 4 * g;
+  bool c_wr[2][4], p_wr[2][4];
+#pragma unroll
+  for (int q4 = 0; q4 < 4; ++q4) {
+    const int m = 8 * q4 + 4 * g;  // first column of the group within its block
+    c_wr[0][q4] = m + 3 >= li;
+    c_wr[1][q4] = m + 1 <= li;
+    p_wr[0][q4] = m + 3 >= 31 - lj;
+    p_wr[1][q4] = m <= 30 - lj;
+  }
+  LDS_AS const float* c_rd = (LDS_AS const float*)(scr + (kScrW + 1) * li + 4 - 4 * g);   // register 4q + e at + 8 (3 - q) + e
+  LDS_AS const float* p_rd = (LDS_AS const float*)(scr + (kScrW - 1) * 4 * g + 31 + li);  // register 4q + e at + 35 * (8q + 3 - e)
+  asm volatile("" : "+v"(c_rd), "+v"(p_rd));  // opaque bases: the reads keep small immediate offsets
 
   // Block 1 of a step holds the rows that were block 0 of the step before: the A operands stay in
   // registers for two steps, in two buffers that swap roles (the loop is unrolled over the parity),
@@ -239,18 +259,18 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
     ring_read(PAR, slot0);
     // V of this step to LDS, V of the next one on its way
     *(u32x4*)(Vs + ring_wr) = vreg;
-    if (k + 1 < n_steps) v_load(s + 1);
+    __builtin_amdgcn_sched_barrier(0);
+    v_load(s + 1);
     // ---- the five products, the position ones through the wave's scratch ------------------------------------
-    // C, then the content product (independent work while C drains), C to the scratch; only then P, in the
-    // registers C has left (the fence below keeps the two from being live together); after B2 and the
-    // staging, C's skewed diagonal is read, P is written over it and read.  The LDS unit runs one wave's
-    // operations in order, so the reads of C are served before the writes of P that follow them; only the
-    // compiler needs the fences.
-    f32x16 sacc, zero;
+    // C, C to the scratch and its skewed diagonal back as the initial value of the content product's
+    // accumulator; P runs while those reads are in flight, in the registers C has left (the fence keeps
+    // the two from being live together); after B2 and the staging, P is written over C and read.  The
+    // LDS unit runs one wave's operations in order, so the reads of C are served before the writes of P
+    // that follow them; only the compiler needs the fences.
+    f32x16 sacc;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) zero[v] = 0.f;
-    u32x4 cw[4];
-    uint32_t px[16];
+    for (int v = 0; v < 16; ++v) sacc[v] = 0.f;
+    const f32x16 zero = sacc;
     if constexpr (C2P) {
       f32x16 cacc[2];
 #pragma unroll
@@ -258,17 +278,17 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
 #pragma unroll
         for (int x = 0; x < KS; ++x) cacc[bk] = QT::mma(ac[PAR ^ bk][x], qf[x], x == 0 ? zero : cacc[bk]);
 #pragma unroll
-      for (int x = 0; x < KS; ++x) sacc = QT::mma(kf[x], qf[x], x == 0 ? zero : sacc);
-#pragma unroll
       for (int bk = 0; bk < 2; ++bk)
 #pragma unroll
         for (int q4 = 0; q4 < 4; ++q4)  // C[i = li][32*bk + 8*q4 + 4*g + 0..3]
-          store4_scratch<ST>(scr_wr + 32 * bk + 8 * q4, cacc[bk][4 * q4], cacc[bk][4 * q4 + 1], cacc[bk][4 * q4 + 2],
-                             cacc[bk][4 * q4 + 3]);
-      __builtin_amdgcn_sched_barrier(0);
-    } else {
+          if (__builtin_expect(c_wr[bk][q4], 1))
+            *(f32x4*)(c_wrp + 32 * bk + 8 * q4) =
+                f32x4{cacc[bk][4 * q4], cacc[bk][4 * q4 + 1], cacc[bk][4 * q4 + 2], cacc[bk][4 * q4 + 3]};
+      wave_lds_fence();
 #pragma unroll
-      for (int x = 0; x < KS; ++x) sacc = QT::mma(kf[x], qf[x], x == 0 ? zero : sacc);
+      for (int v = 0; v < 16; ++v) sacc[v] = c_rd[8 * (3 - (v >> 2)) + (v & 3)];
+      wave_lds_fence();
+      __builtin_amdgcn_sched_barrier(0);
     }
     f32x16 pacc[2];
     if constexpr (P2C) {
@@ -277,59 +297,42 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
 #pragma unroll
         for (int x = 0; x < KS; ++x) pacc[bk] = QT::mma(aq[PAR ^ bk][x], kf[x], x == 0 ? zero : pacc[bk]);
     }
+#pragma unroll
+    for (int x = 0; x < KS; ++x) sacc = QT::mma(kf[x], qf[x], sacc);
     // ---- B2: nobody reads K or the ring of this step from LDS any more --------------------------------------
     __syncthreads();
-    if (k + 1 < n_steps) {
-      *(u32x4*)(Ks + ring_wr) = kreg;
-      batch_store(k + 5);
-      if (k + 2 < n_steps) {
-        batch_load(dnext);  // its table value was loaded a step ago: no wait on the loads issued below
-        k_load(s + 2);
-        if (k + 3 < n_steps) dnext = batch_delta(k + 7);
-      }
-    }
-    if constexpr (C2P) {
-      wave_lds_fence();
-#pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        const u32x2 lo = *(const u32x2*)(c_rd - 8 * q4), hi = *(const u32x2*)(c_rd - 8 * q4 + 4);
-        cw[q4] = u32x4{lo[0], lo[1], hi[0], hi[1]};
-      }
-      wave_lds_fence();
-    }
+    // The staging runs unconditionally, past the last step too (row and table indices are clamped, and
+    // nobody reads what the last steps store): with a fixed sequence of loads the compiler waits at each
+    // use for exactly the loads that are older, instead of for every outstanding one.
+    *(u32x4*)(Ks + ring_wr) = kreg;
+    batch_store(k + 5);
+    __builtin_amdgcn_sched_barrier(0);  // the loads below reuse the registers just stored
+    const int dnew = batch_delta(k + 7);  // first: whatever consumes it waits for this load alone
+    batch_load(dnext);                    // its table value was loaded a step ago
+    k_load(s + 2);
+    dnext = dnew;
     if constexpr (P2C) {
+      wave_lds_fence();
 #pragma unroll
       for (int bk = 0; bk < 2; ++bk)
 #pragma unroll
         for (int q4 = 0; q4 < 4; ++q4)  // P[jj = li][32*bk + 8*q4 + 4*g + 0..3]
-          store4_scratch<ST>(scr_wr + 32 * bk + 8 * q4, pacc[bk][4 * q4], pacc[bk][4 * q4 + 1], pacc[bk][4 * q4 + 2],
-                             pacc[bk][4 * q4 + 3]);
+          if (__builtin_expect(p_wr[bk][q4], 1))
+            *(f32x4*)(p_wrp + 32 * bk + 8 * q4) =
+                f32x4{pacc[bk][4 * q4], pacc[bk][4 * q4 + 1], pacc[bk][4 * q4 + 2], pacc[bk][4 * q4 + 3]};
+      wave_lds_fence();
+      float px[16];
+#pragma unroll
+      for (int v = 0; v < 16; ++v) px[v] = p_rd[(kScrW - 1) * (8 * (v >> 2) + 3 - (v & 3))];
       wave_lds_fence();
 #pragma unroll
-      for (int v = 0; v < 16; ++v) px[v] = *(const uint16_t*)(p_rd + (8 * (v >> 2) + (v & 3)) * (kScrStride - 1));
-      wave_lds_fence();
-    }
-#pragma unroll
-    for (int q4 = 0; q4 < 4; ++q4) {
-      if constexpr (C2P) {
-        const u32x4 d = cw[q4];
-        const uint32_t wa = c_odd_chunk ? d[1] : d[0], wb = c_odd_chunk ? d[2] : d[1], wc = c_odd_chunk ? d[3] : d[2];
-        const uint32_t w0 = __builtin_amdgcn_alignbit(wb, wa, c_shift), w1 = __builtin_amdgcn_alignbit(wc, wb, c_shift);
-        sacc[4 * q4 + 0] = QT::add_hi(sacc[4 * q4 + 0], w1);  // window elements 3, 2, 1, 0 for jj offsets 0, 1, 2, 3
-        sacc[4 * q4 + 1] = QT::add_lo(sacc[4 * q4 + 1], w1);
-        sacc[4 * q4 + 2] = QT::add_hi(sacc[4 * q4 + 2], w0);
-        sacc[4 * q4 + 3] = QT::add_lo(sacc[4 * q4 + 3], w0);
-      }
-      if constexpr (P2C) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) sacc[4 * q4 + e] = QT::add_lo(sacc[4 * q4 + e], px[4 * q4 + e]);
-      }
+      for (int v = 0; v < 16; ++v) sacc[v] += px[v];
     }
     // ---- mask, online soft-max in base 2, O^T += V^T P^T ---------------------------------------------------
     if constexpr (MASK) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int j = j0 + 8 * (v >> 2) + 4 * g + (v & 3);
+        const int j = j0 + 8 * (v >> 2) + 4 * g + 3 - (v & 3);
         if (j >= Lb || (p.causal && j > i)) sacc[v] = -INFINITY;
       }
     }
@@ -352,7 +355,8 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
     for (int c = 0; c < 2; ++c) {
       f32x8 pv;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) pv[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[8 * c + e], x_scale, off));
+      for (int e = 0; e < 8; ++e)  // the V^T operand takes the keys in ascending order
+        pv[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[8 * c + (e ^ 3)], x_scale, off));
       const vfrag pf = VT::from_f32(pv);
       l_run = VT::sum8(pf, l_run);
 #pragma unroll
