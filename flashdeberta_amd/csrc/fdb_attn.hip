@@ -318,7 +318,8 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // in scalar registers: what depends on it alone stays scalar
   const int lane = tid & 63, li = lane & 31, g = lane >> 5;
   int xq, h;
-  block_map((int)blockIdx.x, p.grid_x, p.H, p.tiles_per_seq, p.cu == nullptr, xq, h);
+  block_map((int)blockIdx.x, p.grid_x, p.H, p.tiles_per_seq, p.cu == nullptr,
+            MODE == kFarOnly ? kEdgesFirst : (MODE == kNearRing ? kMiddleFirst : kNatural), xq, h);
 
   int b, m0, tok0, Lb;
   int64_t qo, ko, vo, oo;
