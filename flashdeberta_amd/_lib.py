@@ -32,7 +32,7 @@ class FdbAttnArgs(ctypes.Structure):
 EXPORTS = (
     "fdb_version", "fdb_attn_args_size", "fdb_strerror", "fdb_attn_check", "fdb_attn_fwd", "fdb_worklist_ints",
     "fdb_worklist_max_tiles", "fdb_tile_rows", "fdb_build_worklist", "fdb_delta_lut_radius", "fdb_delta_lut",
-    "fdb_quant_e4m3_per_head",
+    "fdb_quant_e4m3_per_head", "fdb_dequant_e4m3_per_head",
 )
 
 
@@ -67,6 +67,8 @@ def _load():
     lib.fdb_delta_lut.argtypes = [i32, i32, i32, vp]
     lib.fdb_quant_e4m3_per_head.restype = ctypes.c_int
     lib.fdb_quant_e4m3_per_head.argtypes = [vp, i64, i64, vp, i64, i64, vp, vp, i32, i32, i32, vp]
+    lib.fdb_dequant_e4m3_per_head.restype = ctypes.c_int
+    lib.fdb_dequant_e4m3_per_head.argtypes = [vp, i64, i64, vp, vp, i64, i64, i32, i32, i32, vp]
     return lib
 
 

@@ -231,4 +231,16 @@ int fdb_quant_e4m3_per_head(const void* x, int64_t x_stride_t, int64_t x_stride_
                           head_dim, stream);
 }
 
+int fdb_dequant_e4m3_per_head(const void* y, int64_t y_stride_t, int64_t y_stride_h, const float* scale, void* x,
+                              int64_t x_stride_t, int64_t x_stride_h, int32_t tokens, int32_t heads, int32_t head_dim,
+                              void* stream) {
+  if (!x || !y || !scale) return FDB_ERR_NULL;
+  if (head_dim != 32 && head_dim != 64 && head_dim != 128) return FDB_ERR_HEAD_DIM;
+  if (tokens < 1 || heads < 1 || heads > 65535) return FDB_ERR_SHAPE;
+  if (!aligned16(x) || (reinterpret_cast<uintptr_t>(y) & 7u) || (x_stride_t * 2) % 16 || (x_stride_h * 2) % 16 ||
+      y_stride_t % 8 || y_stride_h % 8)
+    return FDB_ERR_ALIGN;
+  return fdb_launch_dequant(y, y_stride_t, y_stride_h, scale, x, x_stride_t, x_stride_h, tokens, heads, head_dim, stream);
+}
+
 }  // extern "C"

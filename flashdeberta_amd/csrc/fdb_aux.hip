@@ -106,7 +106,54 @@ __global__ __launch_bounds__(256) void fdb_quant_kernel(const uint16_t* __restri
   }
 }
 
+// The inverse map, to bf16: x = bf16_rne(e4m3(y) * scale[h]).  Eight elements per thread.
+template <int D>
+__global__ __launch_bounds__(256) void fdb_dequant_kernel(const uint8_t* __restrict__ y, int64_t yst, int64_t ysh,
+                                                          const float* __restrict__ scale, uint16_t* __restrict__ x,
+                                                          int64_t st, int64_t sh, int32_t tokens) {
+  constexpr int CPT = D / 8;
+  const int h = blockIdx.y;
+  const float sc = scale[h];
+  for (int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; c < (int64_t)tokens * CPT;
+       c += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t t = c / CPT;
+    const int cc = (int)(c % CPT);
+    const uint2 raw = *(const uint2*)(y + t * yst + h * ysh + cc * 8);
+    const uint32_t w[2] = {raw.x, raw.y};
+    uint32_t o[4];
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const auto lo = __builtin_amdgcn_cvt_pk_f32_fp8(w[e], false), hi = __builtin_amdgcn_cvt_pk_f32_fp8(w[e], true);
+      typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+      typedef float f2 __attribute__((ext_vector_type(2)));
+      o[2 * e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f2{lo[0] * sc, lo[1] * sc}, bf2));
+      o[2 * e + 1] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f2{hi[0] * sc, hi[1] * sc}, bf2));
+    }
+    *(uint4*)(x + t * st + h * sh + cc * 8) = uint4{o[0], o[1], o[2], o[3]};
+  }
+}
+
 }  // namespace
+
+int fdb_launch_dequant(const void* y, int64_t y_st, int64_t y_sh, const float* scale, void* x, int64_t x_st, int64_t x_sh,
+                       int32_t tokens, int32_t heads, int32_t head_dim, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  const int64_t chunks = (int64_t)tokens * head_dim / 8;
+  int gx = (int)((chunks + 255) / 256);
+  if (gx > 2048) gx = 2048;
+  if (gx < 1) gx = 1;
+#define FDB_DQ(DD)                                                                                              \
+  hipLaunchKernelGGL(fdb_dequant_kernel<DD>, dim3(gx, heads), dim3(256), 0, stream, (const uint8_t*)y, y_st,    \
+                     y_sh, scale, (uint16_t*)x, x_st, x_sh, tokens);
+  switch (head_dim) {
+    case 32: FDB_DQ(32) break;
+    case 64: FDB_DQ(64) break;
+    case 128: FDB_DQ(128) break;
+    default: return -3;
+  }
+#undef FDB_DQ
+  return (int)hipGetLastError();
+}
 
 int fdb_launch_worklist(const int32_t* cu, int32_t batch, int32_t* wl, int32_t max_tiles, void* stream) {
   hipLaunchKernelGGL(fdb_worklist_kernel, dim3(1), dim3(kWlThreads), 0, (hipStream_t)stream, cu, batch, wl, max_tiles);

@@ -58,3 +58,5 @@ int fdb_launch_worklist(const int32_t* cu, int32_t batch, int32_t* wl, int32_t m
 int fdb_launch_quant(const void* x, int64_t x_st, int64_t x_sh, void* y, int64_t y_st, int64_t y_sh,
                      float* scale, uint32_t* absmax_ws, int32_t tokens, int32_t heads, int32_t head_dim,
                      void* stream);
+int fdb_launch_dequant(const void* y, int64_t y_st, int64_t y_sh, const float* scale, void* x, int64_t x_st, int64_t x_sh,
+                       int32_t tokens, int32_t heads, int32_t head_dim, void* stream);

@@ -116,6 +116,22 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
     if fp8:
         if k.dtype != _FP8 or v.dtype != torch.bfloat16:
             raise ValueError("fp8 path: q and k float8_e4m3fn, v bfloat16")
+        if q_scale is None or k_scale is None or (pos_key is not None and pos_key_scale is None) or (
+                pos_query is not None and pos_query_scale is None):
+            raise ValueError("fp8 path: q_scale, k_scale and a scale for each position tensor are required")
+        if D <= 64 and not single_kernel:
+            # At head_dim <= 64 a key tile is bound by its soft-max and LDS work, not by the MFMA rate, and the
+            # 16-bit kernels (direct-to-LDS staging, far / near pair of launches) are about three times faster
+            # than the fp8-MFMA kernel: FP8 operands are expanded to bf16 (scale applied, one rounding to eight
+            # bits) and take that route.  single_kernel=True keeps the fp8 MFMA contraction.
+            deq = lambda x, s: None if x is None else dequantize_e4m3_per_head(x, s)
+            return disentangled_attention_fwd(
+                deq(q, q_scale), deq(k, k_scale), v,
+                None if pos_key is None else deq(pos_key.transpose(0, 1), pos_key_scale).transpose(0, 1),
+                None if pos_query is None else deq(pos_query.transpose(0, 1), pos_query_scale).transpose(0, 1),
+                cu_seqlens=cu_seqlens, max_seqlen=max_seqlen, sm_scale=sm_scale, position_buckets=position_buckets,
+                max_relative_positions=max_relative_positions, causal=causal, return_lse=return_lse,
+                seq_start=seq_start, seq_len=seq_len, out=out)
         dt = _lib.FDB_FP8_E4M3
     else:
         if q.dtype not in _DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
@@ -236,3 +252,23 @@ def quantize_e4m3_per_head(x):
                                           _ptr(scale), _ptr(ws), x3.shape[0], H, D, _stream_ptr(x.device)),
               "fdb_quant_e4m3_per_head")
     return y.view(_FP8).reshape(x.shape), scale
+
+
+def dequantize_e4m3_per_head(y, scale):
+    """y: float8_e4m3fn [..., H, D] on the GPU, scale float32 [H] -> bfloat16 tensor of the same shape,
+    x = bf16_rne(y * scale[h])."""
+    if not y.is_cuda or y.dtype != _FP8:
+        raise ValueError("dequantize_e4m3_per_head expects a float8_e4m3fn GPU tensor")
+    H, D = y.shape[-2], y.shape[-1]
+    if scale.dtype != torch.float32 or scale.numel() != H or not scale.is_cuda:
+        raise ValueError("scale must be a float32 GPU tensor with one entry per head")
+    y3 = y.reshape(-1, H, D)
+    if y3.stride(2) != 1:
+        y3 = y3.contiguous()
+    x = torch.empty(y3.shape, dtype=torch.bfloat16, device=y.device)
+    with torch.cuda.device(y.device):
+        check(lib.fdb_dequant_e4m3_per_head(_ptr(y3), y3.stride(0), y3.stride(1), _ptr(scale.contiguous()), _ptr(x),
+                                            x.stride(0), x.stride(1), y3.shape[0], H, D, _stream_ptr(y.device)),
+              "fdb_dequant_e4m3_per_head")
+    return x.reshape(y.shape)
+

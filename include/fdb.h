@@ -22,7 +22,7 @@
  *                             (flash_attention.py:236-254, flash_attention_varlen.py:174-186), i.e.
  *                             make_log_bucket_position of transformers' modeling_deberta_v2.py:56-69
  *                             followed by clamp(. + S, 0, 2S-1) (:318, :336); host-side, integers out.
- *   fdb_quant_e4m3_per_head   no reference counterpart (FP8 Q/K variant).
+ *   fdb_quant_e4m3_per_head, fdb_dequant_e4m3_per_head   no reference counterpart (FP8 Q/K variant).
  */
 #ifndef FDB_H_
 #define FDB_H_
@@ -156,6 +156,16 @@ int fdb_quant_e4m3_per_head(const void* x, int64_t x_stride_t, int64_t x_stride_
                             void* y, int64_t y_stride_t, int64_t y_stride_h,
                             float* scale, uint32_t* absmax_ws,
                             int32_t tokens, int32_t heads, int32_t head_dim, void* stream);
+
+/*
+ * The inverse map to bf16, x = bf16_rne(e4m3(y) * scale[h]), same indexing as above (y: one byte per
+ * element, 8-byte aligned rows; x: bf16, 16-byte aligned rows).  No reference counterpart (FP8 Q/K
+ * variant): the host side uses it to run FP8 operands through the 16-bit kernels where those are the
+ * faster ones (head_dim <= 64).
+ */
+int fdb_dequant_e4m3_per_head(const void* y, int64_t y_stride_t, int64_t y_stride_h, const float* scale,
+                              void* x, int64_t x_stride_t, int64_t x_stride_h,
+                              int32_t tokens, int32_t heads, int32_t head_dim, void* stream);
 
 #ifdef __cplusplus
 }

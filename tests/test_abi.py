@@ -112,6 +112,8 @@ def test_argument_validation_codes():
     assert lib.fdb_attn_fwd(ctypes.byref(a), None) == -3
     assert lib.fdb_build_worklist(None, 1, 1, None, None) == -1
     assert lib.fdb_quant_e4m3_per_head(None, 0, 0, None, 0, 0, None, None, 1, 1, 64, None) == -1
+    assert lib.fdb_dequant_e4m3_per_head(None, 0, 0, None, None, 0, 0, 1, 1, 64, None) == -1
+    assert lib.fdb_dequant_e4m3_per_head(0x4000, 64, 64, 0x5000, 0x6000, 64, 64, 1, 1, 48, None) == -3
 
 
 def test_error_strings_and_python_mapping():

@@ -266,8 +266,25 @@ def test_fp8_quantisation_bit_exact():
     assert torch.equal(y2.view(torch.uint8), y.view(torch.uint8)) and torch.equal(s2, s)
 
 
+def test_fp8_dequantisation_exact():
+    # x = bf16_rne(e4m3(y) * scale[h]): torch's own float8 -> float32 conversion is the reference
+    g = torch.Generator().manual_seed(10)
+    x = _outliers(torch.randn(513, 12, 64, generator=g) * 0.02, g).to(torch.bfloat16)
+    y, s = ops.quantize_e4m3_per_head(x.cuda())
+    got = ops.dequantize_e4m3_per_head(y, s)
+    ref = (y.float() * s[:, None]).to(torch.bfloat16)
+    assert got.dtype == torch.bfloat16 and torch.equal(got, ref)
+    # a transposed view, as the position tensors arrive ([H, 2S, D] views of [2S, H, D])
+    yt = y.transpose(0, 1)
+    got_t = ops.dequantize_e4m3_per_head(yt.transpose(0, 1), s)
+    assert torch.equal(got_t, ref)
+
+
+# single=False: FP8 operands expanded to bf16 and run through the 16-bit kernels (the default at
+# head_dim <= 64); single=True: the fp8 MFMA contraction in the fused kernel
+@pytest.mark.parametrize("single", [False, True])
 @pytest.mark.parametrize("L,pb,mr", [(300, 32, 64), (1100, 256, 512)])
-def test_fp8_attention(L, pb, mr):
+def test_fp8_attention(L, pb, mr, single):
     B, H, D = 2, 3, 64
     g = torch.Generator().manual_seed(13)
     q, k, v, pk, pq = _inputs(B, L, H, D, pb, mr, torch.bfloat16, 14, 0.02)
@@ -278,7 +295,7 @@ def test_fp8_attention(L, pb, mr):
     pq8, pqs = ops.quantize_e4m3_per_head(pq.cuda().transpose(0, 1))
     out = ops.disentangled_attention_fwd(q8, k8, v.cuda(), pk8.transpose(0, 1), pq8.transpose(0, 1), position_buckets=pb,
                                          max_relative_positions=mr, q_scale=qs, k_scale=ks, pos_key_scale=pks,
-                                         pos_query_scale=pqs)
+                                         pos_query_scale=pqs, single_kernel=single)
     # (a) tight: the oracle on the de-quantised operands
     dq = lambda y, s: y.float().cpu() * s.cpu()[:, None]
     ref_dq = _oracle_blhd(dq(q8, qs), dq(k8, ks), v, dq(pk8, pks).transpose(0, 1), dq(pq8, pqs).transpose(0, 1), pb, mr)
@@ -294,7 +311,7 @@ def test_fp8_attention(L, pb, mr):
     pq8, pqs = ops.quantize_e4m3_per_head(pq.cuda().transpose(0, 1))
     out = ops.disentangled_attention_fwd(q8, k8, v.cuda(), pk8.transpose(0, 1), pq8.transpose(0, 1), position_buckets=pb,
                                          max_relative_positions=mr, q_scale=qs, k_scale=ks, pos_key_scale=pks,
-                                         pos_query_scale=pqs)
+                                         pos_query_scale=pqs, single_kernel=single)
     ref_dq = _oracle_blhd(dq(q8, qs), dq(k8, ks), v, dq(pk8, pks).transpose(0, 1), dq(pq8, pqs).transpose(0, 1), pb, mr)
     _check(out, ref_dq, TOL[torch.bfloat16], "unit scale vs de-quantised oracle")
 
