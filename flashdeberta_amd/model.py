@@ -9,9 +9,10 @@ Forward / inference only (the reference's varlen path has no backward either,
 src/flashdeberta/ops/flash_attention_varlen.py:480-483).
 """
 import math
+import weakref
 
 import torch
-from torch import nn
+import torch.nn.functional as F
 from transformers.models.deberta_v2.modeling_deberta_v2 import (
     DebertaV2Config,
     DebertaV2Model,
@@ -22,22 +23,101 @@ from . import ops
 from .padding import key_padding_mask, seq_bounds
 
 
+class _Memo:
+    """One remembered value, valid while the tensors it was computed from are the same objects and
+    have not been written in place (their version counters are unchanged) and `extra` compares equal.
+    The tensors are held weakly."""
+
+    def __init__(self):
+        self._refs, self._versions, self._extra, self._value = (), (), None, None
+
+    def get(self, tensors, extra=None):
+        if len(self._refs) != len(tensors) or extra != self._extra:
+            return None
+        for ref, ver, t in zip(self._refs, self._versions, tensors):
+            if ref() is not t or t._version != ver:
+                return None
+        return self._value
+
+    def put(self, tensors, value, extra=None):
+        self._refs = tuple(weakref.ref(t) for t in tensors)
+        self._versions = tuple(t._version for t in tensors)
+        self._extra, self._value = extra, value
+        return value
+
+
+_MASK_MEMO = _Memo()
+
+
+def _seq_bounds_of(attention_mask):
+    """(seq_start, seq_len) of a mask; every layer of an encoder receives the same mask object, so
+    the two reductions run once per forward instead of once per layer."""
+    hit = _MASK_MEMO.get((attention_mask,))
+    if hit is None:
+        hit = _MASK_MEMO.put((attention_mask,), seq_bounds(key_padding_mask(attention_mask)))
+    return hit
+
+
 class FlashDisentangledSelfAttention(DisentangledSelfAttention):
     """Same parameters as the eager module (query_proj, key_proj, value_proj[, pos_key_proj,
     pos_query_proj]), so `load_state_dict(eager.state_dict())` works (reference tests/attention.py:60).
 
     fp8_qk=True quantises Q, K and the projected relative embeddings to OCP e4m3 with per-head
-    absmax scales before the kernel (bf16 inputs only)."""
+    absmax scales before the kernel (bf16 inputs only).
+
+    Outside training the three input projections run as one GEMM over the concatenated weights
+    (a copy kept per module, rebuilt when a parameter is replaced or written in place), and K_r / Q_r
+    are remembered for as long as the relative embeddings handed in are the same tensor (an encoder
+    patched by `patch_model` hands in the same tensor until its embedding table changes)."""
 
     def __init__(self, config, fp8_qk=None):
         super().__init__(config)
         self.fp8_qk = bool(getattr(config, "fp8_qk", False)) if fp8_qk is None else bool(fp8_qk)
+        self._qkv_memo, self._pos_memo = _Memo(), _Memo()
+
+    def _fused_qkv(self):
+        """Concatenated [3*H*D, hidden] weight and bias of the query, key and value projections."""
+        projs = (self.query_proj, self.key_proj, self.value_proj)
+        params = tuple(p.weight for p in projs) + tuple(p.bias for p in projs if p.bias is not None)
+        if len(params) not in (3, 6):
+            return None
+        hit = self._qkv_memo.get(params)
+        if hit is None:
+            with torch.no_grad():
+                w = torch.cat([p.weight for p in projs], dim=0)
+                b = torch.cat([p.bias for p in projs], dim=0) if len(params) == 6 else None
+            hit = self._qkv_memo.put(params, (w, b))
+        return hit
+
+    def _qkv(self, hidden_states, query_states):
+        """q, k, v as [B, L, H, D] views (reference model.py:147-149)."""
+        B, L, _ = hidden_states.shape
+        H, D = self.num_attention_heads, self.attention_head_size
+        fused = None if (self.training or query_states is not hidden_states) else self._fused_qkv()
+        if fused is not None:
+            qkv = F.linear(hidden_states, fused[0], fused[1]).view(B, L, 3, H, D)
+            return qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
+        return (self.query_proj(query_states).view(B, L, H, D), self.key_proj(hidden_states).view(B, L, H, D),
+                self.value_proj(hidden_states).view(B, L, H, D))
 
     def _pos_layers(self, rel_embeddings):
         """K_r, Q_r as [H, 2S, D] views of the projected relative embeddings
         (reference model.py:159-177; the slice to 2S rows is transformers modeling_deberta_v2.py:295)."""
         if not self.relative_attention or rel_embeddings is None:
             return None, None
+        # the position projections exist only for the terms the module has (transformers :170-178)
+        kproj = qproj = None
+        if "c2p" in self.pos_att_type:
+            kproj = self.key_proj if self.share_att_key else self.pos_key_proj
+        if "p2c" in self.pos_att_type:
+            qproj = self.query_proj if self.share_att_key else self.pos_query_proj
+        key = None
+        if not self.training:
+            key = (rel_embeddings,) + tuple(p for m in (kproj, qproj) if m is not None for p in (m.weight, m.bias)
+                                            if p is not None)
+            hit = self._pos_memo.get(key, tuple(self.pos_att_type))
+            if hit is not None:
+                return hit
         H, D = self.num_attention_heads, self.attention_head_size
         span = self.pos_ebd_size
         rel = self.pos_dropout(rel_embeddings)[0:2 * span]
@@ -45,17 +125,10 @@ class FlashDisentangledSelfAttention(DisentangledSelfAttention):
         def heads(x):  # [2S, H*D] -> [H, 2S, D] without a copy
             return x.view(x.shape[0], H, D).transpose(0, 1)
 
-        pos_key = pos_query = None
-        if self.share_att_key:
-            if "c2p" in self.pos_att_type:
-                pos_key = heads(self.key_proj(rel))
-            if "p2c" in self.pos_att_type:
-                pos_query = heads(self.query_proj(rel))
-        else:
-            if "c2p" in self.pos_att_type:
-                pos_key = heads(self.pos_key_proj(rel))
-            if "p2c" in self.pos_att_type:
-                pos_query = heads(self.pos_query_proj(rel))
+        pos_key = heads(kproj(rel)) if kproj is not None else None
+        pos_query = heads(qproj(rel)) if qproj is not None else None
+        if key is not None:
+            self._pos_memo.put(key, (pos_key, pos_query), tuple(self.pos_att_type))
         return pos_key, pos_query
 
     def forward(self, hidden_states, attention_mask, output_attentions=False, query_states=None,
@@ -70,9 +143,7 @@ class FlashDisentangledSelfAttention(DisentangledSelfAttention):
         B, L, _ = hidden_states.shape
         H, D = self.num_attention_heads, self.attention_head_size
 
-        q = self.query_proj(query_states).view(B, L, H, D)
-        k = self.key_proj(hidden_states).view(B, L, H, D)
-        v = self.value_proj(hidden_states).view(B, L, H, D)
+        q, k, v = self._qkv(hidden_states, query_states)
         pos_key, pos_query = self._pos_layers(rel_embeddings)
 
         scale_factor = 1 + ("c2p" in self.pos_att_type and pos_key is not None) + \
@@ -84,7 +155,7 @@ class FlashDisentangledSelfAttention(DisentangledSelfAttention):
         seq_start = seq_len = None
         out = None
         if attention_mask is not None:
-            seq_start, seq_len = seq_bounds(key_padding_mask(attention_mask))
+            seq_start, seq_len = _seq_bounds_of(attention_mask)
             out = torch.zeros((B, L, H, D), dtype=v.dtype, device=v.device)  # padded rows stay zero
 
         kw = {}
@@ -145,6 +216,25 @@ def patch_model(model, attn_implementation="flash_attention_2", fp8_qk=False, sk
     else:
         encoder.__dict__.pop("get_rel_pos", None)
         encoder.__dict__.pop("get_attention_mask", None)
+    encoder.__dict__.pop("get_rel_embedding", None)
+    if flash and getattr(encoder, "relative_attention", False):
+        # outside training the (normalised) relative embeddings are the same from forward to forward: hand
+        # the layers one tensor object for as long as the table and its LayerNorm are unchanged, so that
+        # each layer's K_r / Q_r stay valid too
+        original, memo = encoder.get_rel_embedding, _Memo()
+
+        def get_rel_embedding():
+            if encoder.training:
+                return original()
+            norm = getattr(encoder, "LayerNorm", None) if "layer_norm" in getattr(encoder, "norm_rel_ebd", []) else None
+            key = (encoder.rel_embeddings.weight,) + (tuple(norm.parameters()) if norm is not None else ())
+            hit = memo.get(key)
+            if hit is None:
+                with torch.no_grad():
+                    hit = memo.put(key, original())
+            return hit
+
+        encoder.get_rel_embedding = get_rel_embedding
     return model
 
 

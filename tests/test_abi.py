@@ -176,6 +176,75 @@ def test_switch_builds_both_implementations():
         FlashDebertaV2Model(DebertaV2Config(attn_implementation="sdpa", **kw))
 
 
+def test_module_projection_memos():
+    """The one-GEMM input projection and the remembered K_r / Q_r equal the separate projections, and
+    are rebuilt when a parameter is written in place, replaced, or the module goes back to training."""
+    from flashdeberta_amd import DebertaV2Config, FlashDisentangledSelfAttention, patch_model
+    from flashdeberta_amd.model import _seq_bounds_of
+    from transformers.models.deberta_v2.modeling_deberta_v2 import DebertaV2Model
+
+    torch.manual_seed(3)
+    kw = dict(vocab_size=50, hidden_size=128, num_hidden_layers=2, num_attention_heads=2, intermediate_size=128,
+              relative_attention=True, pos_att_type="p2c|c2p", position_buckets=32, max_relative_positions=64,
+              share_att_key=True, norm_rel_ebd="layer_norm", position_biased_input=False)
+    att = FlashDisentangledSelfAttention(DebertaV2Config(**kw)).eval()
+    x = torch.randn(2, 7, 128)
+
+    def separate():
+        return [p(x).view(2, 7, 2, 64) for p in (att.query_proj, att.key_proj, att.value_proj)]
+
+    with torch.no_grad():
+        for got, ref in zip(att._qkv(x, x), separate()):
+            assert got.shape == ref.shape and got.stride(-1) == 1 and torch.allclose(got, ref, atol=1e-6)
+        w0 = att._fused_qkv()[0]
+        assert att._fused_qkv()[0] is w0                       # remembered
+        att.key_proj.weight.mul_(2.0)                          # in-place update -> rebuilt
+        assert att._fused_qkv()[0] is not w0
+        for got, ref in zip(att._qkv(x, x), separate()):
+            assert torch.allclose(got, ref, atol=1e-6)
+        att.load_state_dict({k: v * 0.5 for k, v in att.state_dict().items()})
+        for got, ref in zip(att._qkv(x, x), separate()):
+            assert torch.allclose(got, ref, atol=1e-6)
+        other = torch.randn(2, 7, 128)                         # cross-attention style call: no fusion
+        q, k, v = att._qkv(x, other)
+        assert torch.allclose(q, att.query_proj(other).view(2, 7, 2, 64)) and torch.allclose(k, separate()[1], atol=1e-6)
+        # K_r / Q_r
+        rel = torch.randn(64, 128)
+        pk, pq = att._pos_layers(rel)
+        assert att._pos_layers(rel)[0] is pk
+        assert torch.allclose(pk, att.key_proj(rel).view(64, 2, 64).transpose(0, 1))
+        assert torch.allclose(pq, att.query_proj(rel).view(64, 2, 64).transpose(0, 1))
+        att.query_proj.bias.add_(1.0)
+        pk2, pq2 = att._pos_layers(rel)
+        assert pq2 is not pq and torch.allclose(pq2, att.query_proj(rel).view(64, 2, 64).transpose(0, 1))
+        assert att._pos_layers(rel.clone())[0] is not pk2      # another tensor object
+    att.train()
+    assert att._pos_layers(rel)[0] is not att._pos_layers(rel)[0]
+
+    # the patched encoder hands out one relative-embedding tensor until the table changes
+    hf = patch_model(DebertaV2Model(DebertaV2Config(**kw))).eval()
+    r0 = hf.encoder.get_rel_embedding()
+    assert hf.encoder.get_rel_embedding() is r0
+    ref = hf.encoder.LayerNorm(hf.encoder.rel_embeddings.weight)
+    assert torch.allclose(r0, ref)
+    with torch.no_grad():
+        hf.encoder.rel_embeddings.weight.add_(0.1)
+    r1 = hf.encoder.get_rel_embedding()
+    assert r1 is not r0 and torch.allclose(r1, hf.encoder.LayerNorm(hf.encoder.rel_embeddings.weight))
+    hf.train()
+    assert hf.encoder.get_rel_embedding() is not hf.encoder.get_rel_embedding()
+    patch_model(hf, "eager")
+    assert "get_rel_embedding" not in hf.encoder.__dict__
+
+    # mask bounds: once per mask object and version
+    m = torch.tensor([[1, 1, 1, 0, 0], [0, 0, 1, 1, 1]])
+    s0, n0 = _seq_bounds_of(m)
+    assert _seq_bounds_of(m)[0] is s0 and s0.tolist() == [0, 2] and n0.tolist() == [3, 3]
+    m[0, 3] = 1
+    s1, n1 = _seq_bounds_of(m)
+    assert s1 is not s0 and n1.tolist() == [4, 3]
+
+
 def test_padding_helpers():
     from flashdeberta_amd.padding import get_unpad_data, key_padding_mask, pad_input, seq_bounds, unpad_input
 
