@@ -170,18 +170,31 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
   float m_run = -INFINITY, l_run = 0.f;
 
   // ---- prologue: step 0's K and ring batches 0..4 to LDS; V(0), K(1), batch 5 in the registers --------
+  // All table values first, then all rows: the loads of one kind are in flight together instead of five
+  // dependent round trips one after the other.
   if (n_steps > 0) {
+    int d0[7];
+#pragma unroll
+    for (int bt = 0; bt < 7; ++bt) d0[bt] = batch_delta(bt);
     k_load(s0);
-    *(u32x4*)(Ks + ring_wr) = kreg;
-#pragma unroll 1
+    u32x4 ek0[5], eq0[5];
+#pragma unroll
     for (int bt = 0; bt < 5; ++bt) {
-      batch_load(batch_delta(bt));
+      batch_load(d0[bt]);
+      ek0[bt] = ekreg;
+      eq0[bt] = eqreg;
+    }
+    *(u32x4*)(Ks + ring_wr) = kreg;
+#pragma unroll
+    for (int bt = 0; bt < 5; ++bt) {
+      ekreg = ek0[bt];
+      eqreg = eq0[bt];
       batch_store(bt);
     }
     v_load(s0);
     k_load(s0 + 1);
-    batch_load(batch_delta(5));
-    dnext = batch_delta(6);
+    batch_load(d0[5]);
+    dnext = d0[6];
   }
 
   // ---- per-lane constants ------------------------------------------------------------------------------
