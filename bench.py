@@ -115,8 +115,9 @@ def cpu_baseline(H, D, L):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    # defaults long enough for the clocks to settle: the first ~100 ms after idle run about 3 % slower
+    ap.add_argument("--steps", type=int, default=300)
+    ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--workload", default="v3base_L4096_B8_bf16", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
