@@ -15,6 +15,7 @@ import torch
 import torch.nn.functional as F
 from transformers.models.deberta_v2.modeling_deberta_v2 import (
     DebertaV2Config,
+    DebertaV2Encoder,
     DebertaV2Model,
     DisentangledSelfAttention,
 )
@@ -44,6 +45,9 @@ class _Memo:
         self._versions = tuple(t._version for t in tensors)
         self._extra, self._value = extra, value
         return value
+
+    def __reduce__(self):  # copies and pickles of a module start with nothing remembered
+        return (_Memo, ())
 
 
 _MASK_MEMO = _Memo()
@@ -185,6 +189,41 @@ DEBERTA_SELF_ATTENTION_CLASSES = {
 }
 
 
+class FlashDebertaV2Encoder(DebertaV2Encoder):
+    """transformers' encoder minus work the fused attention never reads: with `_fdb_skip_dense` it builds
+    neither the [1, L, L] int64 relative-position tensor nor the [B, 1, L, L] mask (transformers
+    modeling_deberta_v2.py:601-626), and outside training it hands the layers one relative-embedding tensor
+    object for as long as the table and its LayerNorm are unchanged, so that each layer's K_r / Q_r stay
+    valid from forward to forward.  Instances are made by `patch_model`, which switches the class of an
+    existing encoder."""
+
+    _fdb_skip_dense = True
+
+    def get_rel_pos(self, hidden_states, query_states=None, relative_pos=None):
+        if self._fdb_skip_dense:
+            return relative_pos
+        return super().get_rel_pos(hidden_states, query_states, relative_pos)
+
+    def get_attention_mask(self, attention_mask):
+        if self._fdb_skip_dense:
+            return attention_mask
+        return super().get_attention_mask(attention_mask)
+
+    def get_rel_embedding(self):
+        if self.training or not self.relative_attention:
+            return super().get_rel_embedding()
+        memo = self.__dict__.get("_fdb_rel_memo")
+        if memo is None:
+            memo = self._fdb_rel_memo = _Memo()
+        norm = self.LayerNorm if "layer_norm" in self.norm_rel_ebd else None
+        key = (self.rel_embeddings.weight,) + (tuple(norm.parameters()) if norm is not None else ())
+        hit = memo.get(key)
+        if hit is None:
+            with torch.no_grad():
+                hit = memo.put(key, super().get_rel_embedding())
+        return hit
+
+
 def patch_model(model, attn_implementation="flash_attention_2", fp8_qk=False, skip_dense_position_tensors=True):
     """Swap every `layer.attention.self` of a transformers DebertaV2 model (bare or with a head)
     for the class the key selects, keeping the weights.  With skip_dense_position_tensors the
@@ -210,31 +249,14 @@ def patch_model(model, attn_implementation="flash_attention_2", fp8_qk=False, sk
         new.train(old.training)
         layer.attention.self = new
     flash = cls is FlashDisentangledSelfAttention
-    if flash and skip_dense_position_tensors:
-        encoder.get_rel_pos = lambda hidden_states, query_states=None, relative_pos=None: relative_pos
-        encoder.get_attention_mask = lambda attention_mask: attention_mask
-    else:
-        encoder.__dict__.pop("get_rel_pos", None)
-        encoder.__dict__.pop("get_attention_mask", None)
-    encoder.__dict__.pop("get_rel_embedding", None)
-    if flash and getattr(encoder, "relative_attention", False):
-        # outside training the (normalised) relative embeddings are the same from forward to forward: hand
-        # the layers one tensor object for as long as the table and its LayerNorm are unchanged, so that
-        # each layer's K_r / Q_r stay valid too
-        original, memo = encoder.get_rel_embedding, _Memo()
-
-        def get_rel_embedding():
-            if encoder.training:
-                return original()
-            norm = getattr(encoder, "LayerNorm", None) if "layer_norm" in getattr(encoder, "norm_rel_ebd", []) else None
-            key = (encoder.rel_embeddings.weight,) + (tuple(norm.parameters()) if norm is not None else ())
-            hit = memo.get(key)
-            if hit is None:
-                with torch.no_grad():
-                    hit = memo.put(key, original())
-            return hit
-
-        encoder.get_rel_embedding = get_rel_embedding
+    # The encoder-side shortcuts live in a subclass that differs from transformers' encoder in three methods
+    # only; switching the instance's class keeps copies and pickles of the model working.
+    if flash and type(encoder) in (DebertaV2Encoder, FlashDebertaV2Encoder):
+        encoder.__class__ = FlashDebertaV2Encoder
+        encoder._fdb_skip_dense = bool(skip_dense_position_tensors)
+        encoder._fdb_rel_memo = _Memo()
+    elif type(encoder) is FlashDebertaV2Encoder:
+        encoder.__class__ = DebertaV2Encoder
     return model
 
 
@@ -258,4 +280,4 @@ class FlashDebertaV2Model(DebertaV2Model):
 
 
 __all__ = ["FlashDisentangledSelfAttention", "DEBERTA_SELF_ATTENTION_CLASSES", "FlashDebertaV2Model",
-           "DebertaV2Config", "patch_model"]
+           "FlashDebertaV2Encoder", "DebertaV2Config", "patch_model"]

@@ -233,8 +233,19 @@ def test_module_projection_memos():
     assert r1 is not r0 and torch.allclose(r1, hf.encoder.LayerNorm(hf.encoder.rel_embeddings.weight))
     hf.train()
     assert hf.encoder.get_rel_embedding() is not hf.encoder.get_rel_embedding()
+    # copies and pickles of a patched model work and remember nothing of the original
+    import copy, io, pickle
+    hf.eval()
+    r2 = hf.encoder.get_rel_embedding()
+    twin = copy.deepcopy(hf)
+    with torch.no_grad():
+        twin.encoder.rel_embeddings.weight.mul_(3.0)
+    assert hf.encoder.get_rel_embedding() is r2
+    assert torch.allclose(twin.encoder.get_rel_embedding(), twin.encoder.LayerNorm(twin.encoder.rel_embeddings.weight))
+    again = pickle.loads(pickle.dumps(hf))
+    assert type(again.encoder) is type(hf.encoder) and torch.allclose(again.encoder.get_rel_embedding(), r2)
     patch_model(hf, "eager")
-    assert "get_rel_embedding" not in hf.encoder.__dict__
+    assert type(hf.encoder).__name__ == "DebertaV2Encoder"
 
     # mask bounds: once per mask object and version
     m = torch.tensor([[1, 1, 1, 0, 0], [0, 0, 1, 1, 1]])
