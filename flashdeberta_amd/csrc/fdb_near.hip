@@ -243,20 +243,33 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
   LDS_AS const float* p_rd = (LDS_AS const float*)(scr + (kScrW - 1) * 4 * g + 31 + li);  // register 4q + e at + 35 * (8q + 3 - e)
   asm volatile("" : "+v"(c_rd), "+v"(p_rd));  // opaque bases: the reads keep small immediate offsets
 
-  // Block 1 of a step holds the rows that were block 0 of the step before: the A operands stay in
-  // registers for two steps, in two buffers that swap roles (the loop is unrolled over the parity),
-  // and a step reads only its new block 0 from the rings.
-  qfrag ac[2][C2P ? KS : 1], aq[2][P2C ? KS : 1];
+  // Block 1 of a step holds the rows that were block 0 of the step before, and a step reads only its
+  // new block 0 from the rings.  C[r][i] does not depend on the keys, so C's block 1 IS the block 0 the
+  // step before computed: its accumulator is kept (two that swap roles; the loop is unrolled over the
+  // parity) and only block 0 is contracted.  P depends on the step's keys: there the A operands are
+  // kept instead, in two buffers that swap roles the same way.
+  qfrag ac[C2P ? KS : 1], aq[2][P2C ? KS : 1];
+  f32x16 ckeep[2];
   auto ring_read = [&](int buf, int slot) __attribute__((always_inline)) {
 #pragma unroll
     for (int x = 0; x < KS; ++x) {
-      if constexpr (C2P) ac[buf][x] = QT::load(EK + slot * kRowBytes + rlx[x]);
+      if constexpr (C2P) ac[x] = QT::load(EK + slot * kRowBytes + rlx[x]);
       if constexpr (P2C) aq[buf][x] = QT::load(EQ + slot * kRowBytes + rlx[x]);
     }
   };
   if (n_steps > 0) {
     __syncthreads();  // the prologue's ring rows
     ring_read(1, slot0 >= 32 ? slot0 - 32 : slot0 + (kRingRows - 32));  // block 1 of step 0
+    if constexpr (C2P) {
+#pragma unroll
+      for (int x = 0; x < KS; ++x) {
+        if (x == 0) {
+#pragma unroll
+          for (int v = 0; v < 16; ++v) ckeep[1][v] = 0.f;
+        }
+        ckeep[1] = QT::mma(ac[x], qf[x], ckeep[1]);
+      }
+    }
   }
 
   auto step = [&](auto mask_tag, auto par_tag, int k) __attribute__((always_inline)) {
@@ -285,18 +298,17 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
     for (int v = 0; v < 16; ++v) sacc[v] = 0.f;
     const f32x16 zero = sacc;
     if constexpr (C2P) {
-      f32x16 cacc[2];
 #pragma unroll
-      for (int bk = 0; bk < 2; ++bk)
-#pragma unroll
-        for (int x = 0; x < KS; ++x) cacc[bk] = QT::mma(ac[PAR ^ bk][x], qf[x], x == 0 ? zero : cacc[bk]);
+      for (int x = 0; x < KS; ++x) ckeep[PAR] = QT::mma(ac[x], qf[x], x == 0 ? zero : ckeep[PAR]);
+      const f32x16(&cacc)[2] = ckeep;  // block bk of this step sits in ckeep[PAR ^ bk]
 #pragma unroll
       for (int bk = 0; bk < 2; ++bk)
 #pragma unroll
         for (int q4 = 0; q4 < 4; ++q4)  // C[i = li][32*bk + 8*q4 + 4*g + 0..3]
           if (__builtin_expect(c_wr[bk][q4], 1))
             *(f32x4*)(c_wrp + 32 * bk + 8 * q4) =
-                f32x4{cacc[bk][4 * q4], cacc[bk][4 * q4 + 1], cacc[bk][4 * q4 + 2], cacc[bk][4 * q4 + 3]};
+                f32x4{cacc[PAR ^ bk][4 * q4], cacc[PAR ^ bk][4 * q4 + 1], cacc[PAR ^ bk][4 * q4 + 2],
+                      cacc[PAR ^ bk][4 * q4 + 3]};
       wave_lds_fence();
 #pragma unroll
       for (int v = 0; v < 16; ++v) sacc[v] = c_rd[8 * (3 - (v >> 2)) + (v & 3)];
