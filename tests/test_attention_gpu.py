@@ -148,6 +148,45 @@ def test_two_launch_variants(causal, c2p, p2c, D, L):
     _check(lse.view(2, L, 2), ref_lse, 4 * TOL[torch.bfloat16], "lse")
 
 
+@pytest.mark.parametrize("seed", [1, 2])
+def test_seeded_random_shapes(seed):
+    """Sixteen shapes per seed drawn around the boundaries that change the code path (one query tile,
+    the far / near split at R + 63 keys, 32-key step tails, packed sequences), all dtypes of the
+    two-launch path, against the oracle."""
+    import random
+
+    rng = random.Random(seed)
+    for it in range(16):
+        dtype = rng.choice([torch.bfloat16, torch.float16])
+        D = rng.choice([64, 64, 64, 32])
+        pb, mr = rng.choice([(256, 512), (32, 64), (0, 48), (64, 512), (16, 32), (128, 256)])
+        L = rng.choice([rng.randint(1, 200), rng.randint(200, 700), rng.randint(560, 680), rng.randint(700, 1300)])
+        B, H = rng.choice([(1, 1), (2, 1), (1, 2)])
+        causal = rng.random() < 0.2
+        c2p, p2c = rng.choice([(True, True), (True, True), (True, False), (False, True)])
+        scale = rng.choice([1.0, 0.02])
+        what = "seed %d #%d %s D%d buckets %d/%d L%d B%d H%d causal %d terms %d%d scale %g" % (
+            seed, it, str(dtype)[6:], D, pb, mr, L, B, H, causal, c2p, p2c, scale)
+        if rng.random() < 0.3:  # packed: three random lengths and L itself
+            lens = [rng.randint(1, L) for _ in range(3)] + [L]
+            q, k, v, pk, pq = _inputs(1, sum(lens), H, D, pb, mr, dtype, 100 * seed + it, scale, c2p, p2c)
+            cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+            out = ops.disentangled_attention_fwd(_dev(q[0]), _dev(k[0]), _dev(v[0]), _dev(pk), _dev(pq), cu_seqlens=cu.cuda(),
+                                                 max_seqlen=max(lens), position_buckets=pb, max_relative_positions=mr,
+                                                 causal=causal)
+            off = 0
+            for n in lens:
+                sl = slice(off, off + n)
+                ref = _oracle_blhd(q[:, sl], k[:, sl], v[:, sl], pk, pq, pb, mr, causal=causal)
+                _check(out[sl][None], ref, TOL[dtype], what + " length %d" % n)
+                off += n
+        else:
+            q, k, v, pk, pq = _inputs(B, L, H, D, pb, mr, dtype, 100 * seed + it, scale, c2p, p2c)
+            out = ops.disentangled_attention_fwd(_dev(q), _dev(k), _dev(v), _dev(pk), _dev(pq), position_buckets=pb,
+                                                 max_relative_positions=mr, causal=causal)
+            _check(out, _oracle_blhd(q, k, v, pk, pq, pb, mr, causal=causal), TOL[dtype], what)
+
+
 # ---- delta indices are bit-exact inside the kernel ----------------------------------------------
 @pytest.mark.parametrize("pb,mr,L", [(256, 512, 1200), (32, 64, 300), (0, 40, 130)])
 @pytest.mark.parametrize("term", ["c2p", "p2c"])
