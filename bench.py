@@ -107,9 +107,46 @@ def cpu_baseline(H, D, L):
         run()
     dt = time.perf_counter() - t0
     fl = flops([L], heads, D)
-    return {"value": round(fl / dt / 1e12, 5), "unit": "TFLOP/s", "cores": int(threads), "kind": "port",
-            "sample": "numpy fp32 oracle, %d of %d heads of one batch element at L=%d (%.1f s), %.0f tokens/s per layer"
-                      % (heads, H, L, dt, L / (dt / heads * H))}
+    rec = {"value": round(fl / dt / 1e12, 5), "unit": "TFLOP/s", "cores": int(threads), "kind": "port",
+           "sample": "numpy fp32 oracle, %d of %d heads of one batch element at L=%d (%.1f s), %.0f tokens/s per layer"
+                     % (heads, H, L, dt, L / (dt / heads * H))}
+    eager = eager_module_cpu(H, D, L)
+    if eager is not None:
+        rec["eager_module"] = eager
+    return rec
+
+
+def eager_module_cpu(H, D, L):
+    """transformers' DisentangledSelfAttention -- the class behind the reference's "eager" key
+    (src/flashdeberta/model.py:255) -- on the host cores: one fp32 forward of one batch element, module
+    level (its three input projections and the two relative-embedding projections included), priced with
+    the attention FLOPs only.  None where transformers is not importable."""
+    try:
+        from transformers.models.deberta_v2.modeling_deberta_v2 import DisentangledSelfAttention
+    except Exception:
+        return None
+
+    class Cfg:
+        hidden_size, num_attention_heads = H * D, H
+        attention_probs_dropout_prob = hidden_dropout_prob = 0.0
+        pos_att_type = ["c2p", "p2c"]
+        relative_attention, position_buckets, max_relative_positions = True, 256, 512
+        max_position_embeddings, share_att_key = 512, True
+
+    torch.manual_seed(0)
+    att = DisentangledSelfAttention(Cfg()).eval()
+    x = torch.randn(1, L, H * D) * 0.02
+    rel = torch.randn(S2, H * D) * 0.02
+    mask = torch.ones(1, 1, L, L, dtype=torch.bool)
+    with torch.no_grad():
+        small = slice(0, 256)
+        att(x[:, small], mask[:, :, small, small], rel_embeddings=rel)  # warm-up
+        t0 = time.perf_counter()
+        att(x, mask, rel_embeddings=rel)  # builds its own relative positions, as the encoder would once per forward
+        dt = time.perf_counter() - t0
+    return {"value": round(flops([L], H, D) / dt / 1e12, 5), "unit": "TFLOP/s", "cores": int(torch.get_num_threads()),
+            "sample": "transformers %s DisentangledSelfAttention.forward, fp32, one batch element at L=%d, all %d heads "
+                      "(%.1f s), %.0f tokens/s per layer" % (__import__("transformers").__version__, L, H, dt, L / dt)}
 
 
 def main():
