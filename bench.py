@@ -110,7 +110,10 @@ def cpu_baseline(H, D, L):
     rec = {"value": round(fl / dt / 1e12, 5), "unit": "TFLOP/s", "cores": int(threads), "kind": "port",
            "sample": "numpy fp32 oracle, %d of %d heads of one batch element at L=%d (%.1f s), %.0f tokens/s per layer"
                      % (heads, H, L, dt, L / (dt / heads * H))}
-    eager = eager_module_cpu(H, D, L)
+    try:
+        eager = eager_module_cpu(H, D, L)
+    except Exception as e:  # a transformers release with another module signature: report, do not lose the line
+        eager = {"error": "%s: %s" % (type(e).__name__, str(e)[:200])}
     if eager is not None:
         rec["eager_module"] = eager
     return rec
