@@ -395,12 +395,22 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
   for (int v = 0; v < 16; ++v) negm[v] = 0.f;
   auto setup_far = [&](int side) __attribute__((always_inline)) {  // side 0: far-left (delta(+R)), 1: far-right (delta(-R))
     const int delta = kHasPos ? p.lut[side == 0 ? 2 * p.R : 0] : 0;
+    // A far-only run needs the plain query only here, twice per workgroup: it is loaded again instead of
+    // being held in sixteen registers through the loops.
+    qfrag qs[C::KSTEPS];
+#pragma unroll
+    for (int s = 0; s < C::KSTEPS; ++s) {
+      if constexpr (MODE == kFarOnly)
+        qs[s] = (i < Lb) ? QT::load(qb + ((int64_t)i * p.q_st + 16 * s + 8 * g) * QT::SZ) : QT::zero();
+      else
+        qs[s] = qf[s];
+    }
     if constexpr (C2P) {
       const char* row = pkb + (int64_t)delta * p.pk_sr * QT::SZ;
       float acc = 0.f;
 #pragma unroll
       for (int s = 0; s < C::KSTEPS; ++s) {
-        const f32x8 a = QT::to_f32(QT::load(row + (16 * s + 8 * g) * QT::SZ)), q8 = QT::to_f32(qf[s]);
+        const f32x8 a = QT::to_f32(QT::load(row + (16 * s + 8 * g) * QT::SZ)), q8 = QT::to_f32(qs[s]);
 #pragma unroll
         for (int e = 0; e < 8; ++e) acc = __builtin_fmaf(a[e], q8[e], acc);
       }
@@ -410,10 +420,10 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
       const char* row = pqb + (int64_t)delta * p.pq_sr * QT::SZ;
 #pragma unroll
       for (int s = 0; s < C::KSTEPS; ++s)
-        qfar[s] = QT::from_f32((QT::to_f32(qf[s]) + QT::to_f32(QT::load(row + (16 * s + 8 * g) * QT::SZ))) * x_scale);
+        qfar[s] = QT::from_f32((QT::to_f32(qs[s]) + QT::to_f32(QT::load(row + (16 * s + 8 * g) * QT::SZ))) * x_scale);
     } else {
 #pragma unroll
-      for (int s = 0; s < C::KSTEPS; ++s) qfar[s] = QT::from_f32(QT::to_f32(qf[s]) * x_scale);
+      for (int s = 0; s < C::KSTEPS; ++s) qfar[s] = QT::from_f32(QT::to_f32(qs[s]) * x_scale);
     }
     const float nm = a_far - (m_run == -INFINITY ? 0.f : m_run);
 #pragma unroll
@@ -522,14 +532,26 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
 #pragma unroll
   for (int v = 0; v < 16; ++v) zero16[v] = 0.f;
   auto qk = [&](f32x16 (&sacc)[2], const qfrag (&qq)[C::KSTEPS], const f32x16& init) __attribute__((always_inline)) {
+    if constexpr (DMA) {
+      // every K fragment of the tile is requested before the first MFMA waits for one
+      qfrag kf[2][C::KSTEPS];
 #pragma unroll
-    for (int jb = 0; jb < 2; ++jb) {
+      for (int jb = 0; jb < 2; ++jb)
 #pragma unroll
-      for (int s = 0; s < C::KSTEPS; ++s) {
-        qfrag kf;
-        if constexpr (DMA) kf = QT::load(smem + kcur[s] + jb * 4096);
-        else kf = QT::load(Ks + (jb * 32 + li) * C::K_RS + (16 * s + 8 * g) * QT::SZ);
-        sacc[jb] = QT::mma(kf, qq[s], s == 0 ? init : sacc[jb]);
+        for (int s = 0; s < C::KSTEPS; ++s) kf[jb][s] = QT::load(smem + kcur[s] + jb * 4096);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s = 0; s < C::KSTEPS; ++s)
+#pragma unroll
+        for (int jb = 0; jb < 2; ++jb) sacc[jb] = QT::mma(kf[jb][s], qq[s], s == 0 ? init : sacc[jb]);
+    } else {
+#pragma unroll
+      for (int jb = 0; jb < 2; ++jb) {
+#pragma unroll
+        for (int s = 0; s < C::KSTEPS; ++s) {
+          const qfrag kf = QT::load(Ks + (jb * 32 + li) * C::K_RS + (16 * s + 8 * g) * QT::SZ);
+          sacc[jb] = QT::mma(kf, qq[s], s == 0 ? init : sacc[jb]);
+        }
       }
     }
   };
