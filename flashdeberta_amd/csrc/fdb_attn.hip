@@ -464,17 +464,37 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
   }
   // The tile's first row travels as the scalar base of the load, the lane's place in the tile as
   // its offset: the row is clamped to the last one of the sequence (rows past the end re-read it).
+  // A tile inside the sequence uses lane offsets computed once; only the last, ragged tile clamps its rows.
+  uint32_t dma_koff[2] = {0, 0}, dma_voff[2] = {0, 0};
+  if constexpr (DMA) {
+#pragma unroll
+    for (int q2 = 0; q2 < 2; ++q2) {
+      const uint32_t row = (uint32_t)(16 * wave + 8 * q2 + (lane >> 3));
+      const uint32_t c16 = ((lane & 7) ^ (4 * ((lane >> 4) & 1)) ^ (lane >> 5) ^ (2 * q2)) * 16;
+      dma_koff[q2] = row * k_rsb + c16;
+      dma_voff[q2] = row * v_rsb + c16;
+    }
+  }
   auto dma_issue = [&](int tile, int bufoff) __attribute__((always_inline)) {
     const char* kt = kb + (uint64_t)(uint32_t)(tile * FDB_BN) * k_rsb;
     const char* vt = vb + (uint64_t)(uint32_t)(tile * FDB_BN) * v_rsb;
     const int last = Lb - 1 - tile * FDB_BN;
+    if (last >= FDB_BN - 1) {
 #pragma unroll
-    for (int q2 = 0; q2 < 2; ++q2) {  // this wave's two 8-row groups of K and of V
-      const uint32_t row = (uint32_t)min(16 * wave + 8 * q2 + (lane >> 3), last);
-      const uint32_t c16 = ((lane & 7) ^ (4 * ((lane >> 4) & 1)) ^ (lane >> 5) ^ (2 * q2)) * 16;  // slot ^ f(row), unclamped row
-      const uint32_t dst = lds0 + bufoff + (2 * wave + q2) * 1024;
-      dma16s(kt, row * k_rsb + c16, dst);
-      dma16s(vt, row * v_rsb + c16, dst + C::DMA_TILE);
+      for (int q2 = 0; q2 < 2; ++q2) {  // this wave's two 8-row groups of K and of V
+        const uint32_t dst = lds0 + bufoff + (2 * wave + q2) * 1024;
+        dma16s(kt, dma_koff[q2], dst);
+        dma16s(vt, dma_voff[q2], dst + C::DMA_TILE);
+      }
+    } else {
+#pragma unroll
+      for (int q2 = 0; q2 < 2; ++q2) {
+        const uint32_t row = (uint32_t)min(16 * wave + 8 * q2 + (lane >> 3), last);
+        const uint32_t c16 = ((lane & 7) ^ (4 * ((lane >> 4) & 1)) ^ (lane >> 5) ^ (2 * q2)) * 16;  // slot ^ f(row), unclamped row
+        const uint32_t dst = lds0 + bufoff + (2 * wave + q2) * 1024;
+        dma16s(kt, row * k_rsb + c16, dst);
+        dma16s(vt, row * v_rsb + c16, dst + C::DMA_TILE);
+      }
     }
   };
   {
@@ -504,8 +524,8 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
       }
 #pragma unroll
       for (int x = 0; x < 4; ++x) {
-        kcur[x] = (klane ^ (32 * x)) + dma_cur;
-        vcur[x] = (vlane ^ (64 * (x >> 1) ^ 32 * (x & 1))) + dma_cur + C::DMA_TILE;
+        kcur[x] = (klane ^ (32 * x)) + (dma_cur + lds0);  // absolute LDS addresses
+        vcur[x] = (vlane ^ (64 * (x >> 1) ^ 32 * (x & 1))) + (dma_cur + lds0 + C::DMA_TILE);
       }
     } else {
       __syncthreads();  // every wave is done with the previous tile and its bias scratch
@@ -521,8 +541,8 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
   };
   auto vload = [&](int c, int d) __attribute__((always_inline)) {
     if constexpr (DMA) {
-      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(smem + vcur[2 * d] + 2048 * c));
-      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(smem + vcur[2 * d + 1] + 2048 * c + 1024));
+      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)((LDS_AS char*)(uintptr_t)vcur[2 * d] + 2048 * c));
+      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)((LDS_AS char*)(uintptr_t)vcur[2 * d + 1] + 2048 * c + 1024));
       return __builtin_bit_cast(typename VT::frag, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
     } else {
       return VtLoad<VT>::get(Vs, C::V_RS, c, d, lane);
@@ -538,7 +558,7 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
 #pragma unroll
       for (int jb = 0; jb < 2; ++jb)
 #pragma unroll
-        for (int s = 0; s < C::KSTEPS; ++s) kf[jb][s] = QT::load(smem + kcur[s] + jb * 4096);
+        for (int s = 0; s < C::KSTEPS; ++s) kf[jb][s] = *(LDS_AS const qfrag*)((LDS_AS const char*)(uintptr_t)kcur[s] + jb * 4096);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int s = 0; s < C::KSTEPS; ++s)
