@@ -269,3 +269,25 @@ def test_padding_helpers():
     assert idx.tolist() == ref_idx.tolist() and cu.tolist() == ref_cu.tolist() and int(mx) == ref_mx
     x = torch.arange(15.0).view(3, 5, 1)
     assert torch.equal(pad_input(unpad_input(x, idx), idx, 3, 5), x * m[:, :, None])
+
+
+def test_bench_contract_without_a_gpu():
+    """bench.py refuses more than one GPU with a message, prices the workloads with the stated FLOP
+    count, and its CPU leg returns the fields the measurement contract names."""
+    import subprocess
+    import sys
+
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0 and "ONE GPU" in (r.stderr + r.stdout)
+    sys.path.insert(0, ROOT)
+    import bench
+
+    # F = B*H*(4 L^2 D + 4 L 2S D): 463.86 GFLOP at the default workload
+    B, L, H, D, _, _ = bench.WORKLOADS["v3base_L4096_B8_bf16"]
+    assert abs(bench.flops([L] * B, H, D) / 1e9 - 463.86) < 0.01
+    assert bench.flops([512], 12, 64, pos=False) == 12 * 4 * 512 * 512 * 64
+    rec = bench.cpu_baseline(2, 64, 256)
+    assert rec["kind"] == "port" and rec["cores"] >= 1 and rec["value"] > 0 and rec["unit"] == "TFLOP/s"
+    assert "sample" in rec and ("eager_module" not in rec or "value" in rec["eager_module"] or "error" in rec["eager_module"])
+    t = bench.measured_traffic("v3base_L4096_B8_bf16")
+    assert t is None or t > 2e8
