@@ -14,10 +14,11 @@
 //   a step sees 159 relative positions (5 batches of 32), and since the rows of the next step are
 //   stored after every wave has finished reading the ring in the current one, the rings hold
 //   exactly 5 batches = 160 rows of 128 bytes, unpadded and XOR-swizzled;
-//   a wave's 32 x 32 sub-tile sees 63 relative positions, so both position products are 2 MFMA row
-//   blocks, private to the wave: C[i][r] = q_i . E_K[r] and P[j][r] = k_j . E_Q[r] go, one after
-//   the other, through one per-wave fp32 LDS scratch from which element (i, j) reads index r = i - j;
-//   C's values come back as the initial value of the content product's accumulator.
+//   a wave's 32 x 32 sub-tile sees 63 relative positions, so both position products are 2 MFMA
+//   blocks, private to the wave: C[i][r] = q_i . E_K[r] and P[j][r] = k_j . E_Q[r], of which element
+//   (i, j) wants index r = i - j.  C goes through a per-wave fp32 LDS scratch and comes back as the
+//   initial value of the content product's accumulator; P is computed with the keys as MFMA rows, so
+//   its skew is a permutation of lanes within a register (ds_bpermute) and needs no scratch.
 // LDS: K 4 KB + V 4 KB + rings 40 KB + scratch 18.5 KB = 66.5 KB.
 //
 // Staging rides inside the step, between its two barriers B1 (top: K, the ring rows and V's buffer
@@ -49,7 +50,7 @@ struct NCfg {
   static constexpr int RING_BYTES = kRingRows * kRowBytes;
   static constexpr int SCR_BYTES = 4 * kScrWords * 4;
   static constexpr int lds_bytes(bool c2p, bool p2c) {
-    return K_BYTES + V_BYTES + (c2p ? RING_BYTES : 0) + (p2c ? RING_BYTES : 0) + SCR_BYTES;
+    return K_BYTES + V_BYTES + (c2p ? RING_BYTES + SCR_BYTES : 0) + (p2c ? RING_BYTES : 0);
   }
 };
 
@@ -68,7 +69,7 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
   char* Vs = Ks + NCfg::K_BYTES;        // [32][128]
   char* EK = Vs + NCfg::V_BYTES;        // [160][128] rows K_r[delta(r)], slot = (r_hi0 - r) mod 160
   char* EQ = EK + (C2P ? NCfg::RING_BYTES : 0);
-  char* scr_raw = EQ + (P2C ? NCfg::RING_BYTES : 0);
+  char* scr_raw = EQ + (P2C ? NCfg::RING_BYTES : 0);  // C's scratch (absent without the c2p term)
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -217,31 +218,27 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
       vlx[x] = vlane ^ (64 * (x >> 1) ^ 32 * (x & 1));
     }
   }
-  // scratch (fp32, so no conversion and no sub-word extraction): C[i = li][rr], P[jj = li][rr] with
-  // rr = r - r_lo in 0..63; element (jj = 8q + 4g + e, i = li) reads C[li][li + 31 - jj] and
-  // P[jj][li + 31 - jj].  Only a band of 32 columns of each row is ever read (C: rr in [li, li + 31],
-  // P: rr in [31 - jj, 62 - jj]), so the rows are laid 36 words apart and overlap: the bands (plus the
-  // three columns a four-column group may stick out on either side) stay disjoint, and a lane does not
-  // write the groups of its row that lie wholly outside the band.
+  // scratch (fp32, so no conversion and no sub-word extraction): C[i = li][rr] with rr = r - r_lo in
+  // 0..63; element (jj = 8q + 4g + e, i = li) reads C[li][li + 31 - jj].  Only a band of 32 columns of
+  // each row is ever read (rr in [li, li + 31]), so the rows are laid 36 words apart and overlap: the
+  // bands (plus the three columns a four-column group may stick out on either side) stay disjoint, and
+  // a lane does not write the groups of its row that lie wholly outside the band.
   // K's rows sit in LDS with the low two bits of the row index inverted, so MFMA row m = 8q + 4g + e of
   // the content product is key jj = 8q + 4g + 3 - e: the four C elements a lane adds to consecutive
   // accumulator registers then lie at ascending addresses and can be read in pairs straight into the
-  // accumulator's registers.  P's column of lane li is therefore key li ^ 3.
-  const int lj = li ^ 3;
+  // accumulator's registers.
   float* c_wrp = scr + li * kScrW + 4 * g;  // row = this lane's MFMA column; group (bk, q4) at + 32 bk + 8 q4
-  float* p_wrp = scr + lj * kScrW + 4 * g;
-  bool c_wr[2][4], p_wr[2][4];
+  bool c_wr[2][4];
 #pragma unroll
   for (int q4 = 0; q4 < 4; ++q4) {
     const int m = 8 * q4 + 4 * g;  // first column of the group within its block
     c_wr[0][q4] = m + 3 >= li;
     c_wr[1][q4] = m + 1 <= li;
-    p_wr[0][q4] = m + 3 >= 31 - lj;
-    p_wr[1][q4] = m <= 30 - lj;
   }
   LDS_AS const float* c_rd = (LDS_AS const float*)(scr + (kScrW + 1) * li + 4 - 4 * g);   // register 4q + e at + 8 (3 - q) + e
-  LDS_AS const float* p_rd = (LDS_AS const float*)(scr + (kScrW - 1) * 4 * g + 31 + li);  // register 4q + e at + 35 * (8q + 3 - e)
-  asm volatile("" : "+v"(c_rd), "+v"(p_rd));  // opaque bases: the reads keep small immediate offsets
+  asm volatile("" : "+v"(c_rd));  // opaque base: the reads keep small immediate offsets
+  // P's lane permutation: register v (key jj = 4g + c) of lane (g, li) comes from lane (g, (li + 31 - jj) mod 32)
+  const int p_nj = li + 4 * g, p_src = 4 * (li + 31 - 4 * g), p_half = 128 * g;
 
   // Block 1 of a step holds the rows that were block 0 of the step before, and a step reads only its
   // new block 0 from the rings.  C[r][i] does not depend on the keys, so C's block 1 IS the block 0 the
@@ -287,12 +284,11 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
     *(u32x4*)(Vs + ring_wr) = vreg;
     __builtin_amdgcn_sched_barrier(0);
     v_load(s + 1);
-    // ---- the five products, the position ones through the wave's scratch ------------------------------------
+    // ---- the five products -------------------------------------------------------------------------------
     // C, C to the scratch and its skewed diagonal back as the initial value of the content product's
-    // accumulator; P runs while those reads are in flight, in the registers C has left (the fence keeps
-    // the two from being live together); after B2 and the staging, P is written over C and read.  The
-    // LDS unit runs one wave's operations in order, so the reads of C are served before the writes of P
-    // that follow them; only the compiler needs the fences.
+    // accumulator; P runs while those reads are in flight (the scheduling fence keeps it behind them).
+    // The LDS unit runs one wave's operations in order, so the reads of C are served before the writes
+    // of the next step; only the compiler needs the fences.
     f32x16 sacc;
 #pragma unroll
     for (int v = 0; v < 16; ++v) sacc[v] = 0.f;
@@ -315,15 +311,32 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
       wave_lds_fence();
       __builtin_amdgcn_sched_barrier(0);
     }
+    // P with the keys as MFMA rows, like the content product: register v of lane (g, n) holds
+    // P[jj(v, g)][32 bk + n], and element (jj, i = li) wants column li + 31 - jj of that row, i.e. the same
+    // register of another lane of its own half.  Each source lane is read by exactly one lane, which
+    // wants block 1 from it if n + jj < 31 and block 0 otherwise: the source picks, one lane permutation
+    // per register moves it.
     f32x16 pacc[2];
     if constexpr (P2C) {
 #pragma unroll
       for (int bk = 0; bk < 2; ++bk)
 #pragma unroll
-        for (int x = 0; x < KS; ++x) pacc[bk] = QT::mma(aq[PAR ^ bk][x], kf[x], x == 0 ? zero : pacc[bk]);
+        for (int x = 0; x < KS; ++x) pacc[bk] = QT::mma(kf[x], aq[PAR ^ bk][x], x == 0 ? zero : pacc[bk]);
     }
 #pragma unroll
     for (int x = 0; x < KS; ++x) sacc = QT::mma(kf[x], qf[x], sacc);
+    float px[16];
+    if constexpr (P2C) {
+      int nj = p_nj, src = p_src;
+      asm volatile("" : "+v"(nj), "+v"(src));  // per-register masks and addresses are made here, not kept
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int c = 8 * (v >> 2) + 3 - (v & 3);  // jj - 4g
+        const float x = (nj + c < 31) ? pacc[1][v] : pacc[0][v];
+        const int addr = ((src - 4 * c) & 124) | p_half;
+        px[v] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(addr, __builtin_bit_cast(int, x)));
+      }
+    }
     // ---- B2: nobody reads K or the ring of this step from LDS any more --------------------------------------
     __syncthreads();
     // The staging runs unconditionally, past the last step too (row and table indices are clamped, and
@@ -337,19 +350,6 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
     k_load(s + 2);
     dnext = dnew;
     if constexpr (P2C) {
-      wave_lds_fence();
-#pragma unroll
-      for (int bk = 0; bk < 2; ++bk)
-#pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4)  // P[jj = li][32*bk + 8*q4 + 4*g + 0..3]
-          if (__builtin_expect(p_wr[bk][q4], 1))
-            *(f32x4*)(p_wrp + 32 * bk + 8 * q4) =
-                f32x4{pacc[bk][4 * q4], pacc[bk][4 * q4 + 1], pacc[bk][4 * q4 + 2], pacc[bk][4 * q4 + 3]};
-      wave_lds_fence();
-      float px[16];
-#pragma unroll
-      for (int v = 0; v < 16; ++v) px[v] = p_rd[(kScrW - 1) * (8 * (v >> 2) + 3 - (v & 3))];
-      wave_lds_fence();
 #pragma unroll
       for (int v = 0; v < 16; ++v) sacc[v] += px[v];
     }
