@@ -18,19 +18,20 @@ class FdbAttnArgs(ctypes.Structure):
     _fields_ = (
         [(n, ctypes.c_void_p) for n in (
             "q", "k", "v", "pos_key", "pos_query", "out", "lse", "cu_seqlens", "worklist", "seq_start", "seq_len", "delta_lut",
-            "q_scale", "k_scale", "pk_scale", "pq_scale")]
+            "q_scale", "k_scale", "pk_scale", "pq_scale", "workspace")]
         + [(n, ctypes.c_int64) for n in (
             "q_stride_b", "q_stride_t", "q_stride_h", "k_stride_b", "k_stride_t", "k_stride_h",
             "v_stride_b", "v_stride_t", "v_stride_h", "o_stride_b", "o_stride_t", "o_stride_h",
-            "pk_stride_h", "pk_stride_r", "pq_stride_h", "pq_stride_r")]
+            "pk_stride_h", "pk_stride_r", "pq_stride_h", "pq_stride_r", "workspace_bytes")]
         + [(n, ctypes.c_int32) for n in (
-            "batch", "heads", "head_dim", "max_seqlen", "total_tokens", "att_span", "lut_radius", "dtype", "causal")]
+            "batch", "heads", "head_dim", "max_seqlen", "total_tokens", "att_span", "lut_radius", "dtype", "causal", "far_splits")]
         + [("sm_scale", ctypes.c_float)]
     )
 
 
 EXPORTS = (
-    "fdb_version", "fdb_attn_args_size", "fdb_strerror", "fdb_attn_check", "fdb_attn_fwd", "fdb_worklist_ints",
+    "fdb_version", "fdb_attn_args_size", "fdb_strerror", "fdb_attn_check", "fdb_attn_fwd", "fdb_attn_workspace_bytes",
+    "fdb_worklist_ints",
     "fdb_worklist_max_tiles", "fdb_tile_rows", "fdb_build_worklist", "fdb_delta_lut_radius", "fdb_delta_lut",
     "fdb_quant_e4m3_per_head", "fdb_dequant_e4m3_per_head",
 )
@@ -54,6 +55,8 @@ def _load():
     lib.fdb_attn_check.argtypes = [ctypes.POINTER(FdbAttnArgs)]
     lib.fdb_attn_fwd.restype = ctypes.c_int
     lib.fdb_attn_fwd.argtypes = [ctypes.POINTER(FdbAttnArgs), vp]
+    lib.fdb_attn_workspace_bytes.restype = i64
+    lib.fdb_attn_workspace_bytes.argtypes = [ctypes.POINTER(FdbAttnArgs)]
     lib.fdb_worklist_ints.restype = i64
     lib.fdb_worklist_ints.argtypes = [i32, i32]
     lib.fdb_worklist_max_tiles.restype = i32

@@ -4,6 +4,8 @@
 #include <stdint.h>
 #include <string.h>
 
+#include <atomic>
+
 #include <hip/hip_runtime_api.h>
 
 #include "../../include/fdb.h"
@@ -67,6 +69,60 @@ bool lut_config_ok(int32_t position_buckets, int32_t max_position) {
 
 constexpr int32_t kRadiusCap = 1 << 22;
 
+static_assert(FDB_MAX_FAR_SPLITS == FDB_MAX_FAR_PARTS, "public and internal limit of the far splits");
+
+// Compute units of the current device (256 if it cannot be asked).
+int cu_count() {
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) n = 256;
+    cached[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
+
+int64_t query_tiles(const fdb_attn_args* a) {
+  return a->cu_seqlens ? fdb_worklist_max_tiles(a->total_tokens, a->batch)
+                       : (int64_t)a->batch * ((a->max_seqlen + FDB_BM - 1) / FDB_BM);
+}
+
+// Does the call take the far / near pair of launches with a far launch in it?
+bool has_far_launch(const fdb_attn_args* a) {
+  const int32_t radius = a->lut_radius > 0 ? a->lut_radius : 1;
+  return (a->pos_key || a->pos_query) && a->lse && fdb_near_supported(a->dtype, a->head_dim) &&
+         a->max_seqlen > radius + FDB_BN - 1;
+}
+
+// Workgroups per query tile of the far-only launch.  That launch keeps three workgroups on a CU; when
+// the query tiles fill at most half of those slots, the far keys of a tile are shared out among as many
+// workgroups as still fit in one round, every share keeping at least eight tiles.  (Measured: 384 query
+// tiles on 768 slots gain 9 % of the whole call from two shares; shares that need a second round of
+// workgroups, e.g. three for 512 query tiles, gain nothing.)
+int far_parts_wanted(const fdb_attn_args* a) {
+  if (!has_far_launch(a) || !fdb_near32_supported(a->dtype, a->head_dim)) return 1;
+  if (a->far_splits > 0) return a->far_splits;
+  if (a->cu_seqlens) return 1;  // the lengths, and with them the far tiles per query tile, are on the device
+  const int64_t wgs = query_tiles(a) * a->heads, slots = 3 * (int64_t)cu_count();
+  if (wgs >= slots) return 1;
+  const int n64 = (a->max_seqlen + FDB_BN - 1) / FDB_BN;
+  const int near64 = (FDB_BM + 2 * a->lut_radius + 3 * (FDB_BN - 1)) / FDB_BN;  // of a query tile in mid-sequence
+  const int most = (n64 - near64) / 8 < FDB_MAX_FAR_PARTS ? (n64 - near64) / 8 : FDB_MAX_FAR_PARTS;
+  const int64_t fit = slots / wgs;
+  const int n = (int)(fit < most ? fit : most);
+  return n > 1 ? n : 1;
+}
+
+int64_t lse_rows(const fdb_attn_args* a) {
+  return a->cu_seqlens ? (int64_t)a->total_tokens : (int64_t)a->batch * a->max_seqlen;
+}
+
+int64_t far_part_bytes(const fdb_attn_args* a) {
+  return lse_rows(a) * a->heads * ((int64_t)a->head_dim * v_elem_size(a->dtype) + 4);
+}
+
 }  // namespace
 
 extern "C" {
@@ -118,6 +174,8 @@ int fdb_attn_check(const fdb_attn_args* a) {
   if (a->dtype == FDB_F32 && a->head_dim == 128) return FDB_ERR_UNSUPPORTED;
   if (a->batch < 1 || a->heads < 1 || a->heads > 65535 || a->max_seqlen < 1 || a->total_tokens < 1)
     return FDB_ERR_SHAPE;
+  if (a->far_splits < 0 || a->far_splits > FDB_MAX_FAR_SPLITS || a->workspace_bytes < 0) return FDB_ERR_SHAPE;
+  if (a->workspace && !aligned16(a->workspace)) return FDB_ERR_ALIGN;
   if (!a->cu_seqlens && (int64_t)a->batch * a->max_seqlen != a->total_tokens) return FDB_ERR_SHAPE;
   if (a->cu_seqlens && !a->worklist) return FDB_ERR_WORKLIST;
   const bool has_pos = a->pos_key || a->pos_query;
@@ -141,6 +199,11 @@ int fdb_attn_check(const fdb_attn_args* a) {
   for (int64_t s : v_strides)
     if ((s * vsz) % 16 != 0) return FDB_ERR_ALIGN;
   return FDB_OK;
+}
+
+int64_t fdb_attn_workspace_bytes(const fdb_attn_args* a) {
+  if (fdb_attn_check(a) != FDB_OK) return 0;
+  return (far_parts_wanted(a) - 1) * far_part_bytes(a);
 }
 
 int fdb_attn_fwd(const fdb_attn_args* a, void* stream) {
@@ -172,16 +235,22 @@ int fdb_attn_fwd(const fdb_attn_args* a, void* stream) {
   p.R = a->lut_radius > 0 ? a->lut_radius : 1;
   p.causal = a->causal ? 1 : 0;
   p.scale_log2 = a->sm_scale * 1.4426950408889634f;
-  int64_t grid_x = a->cu_seqlens ? fdb_worklist_max_tiles(a->total_tokens, a->batch)
-                                 : (int64_t)a->batch * p.tiles_per_seq;
+  const int64_t grid_x = query_tiles(a);
   if (grid_x < 1 || grid_x * a->heads > INT32_MAX) return FDB_ERR_SHAPE;
   p.grid_x = (int32_t)grid_x;
   // Split path: the far tiles in a far-only run of the kernel (three workgroups per CU), the near
   // tiles in a second launch, which merges the two.  It needs the log-sum-exp buffer as the
   // hand-over between the two launches.
   if ((a->pos_key || a->pos_query) && a->lse && fdb_near_supported(a->dtype, a->head_dim)) {
-    const bool need_far = a->max_seqlen > p.R + FDB_BN - 1;  // otherwise no tile of any query tile is far
+    const bool need_far = has_far_launch(a);  // otherwise no tile of any query tile is far
+    p.far_parts = 1;
     if (need_far) {
+      // as many workgroups per query tile as wanted and as the workspace holds partial results for
+      p.far_parts = far_parts_wanted(a);
+      const int64_t part_bytes = far_part_bytes(a);
+      while (p.far_parts > 1 && (!a->workspace || a->workspace_bytes / part_bytes < p.far_parts - 1)) --p.far_parts;
+      p.ws = (char*)a->workspace;
+      p.ws_rows = lse_rows(a);
       const int rc_far = fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, FDB_MODE_FAR_ONLY, stream);
       if (rc_far != 0) return rc_far;
     }

@@ -431,10 +431,23 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
   };
 
 
+  // The far tiles of this workgroup: [zl0, zl1) left of the near range and [zr0, zr1) right of it.  A
+  // far-only run may be split over p.far_parts workgroups per query tile (blockIdx.y), each taking an equal
+  // share of the far tiles in walking order and leaving a partial result of its own.
+  int zl0 = 0, zl1 = t_near0, zr0 = t_near1, zr1 = n_tiles;
+  const int part = FAR_ONLY ? (int)blockIdx.y : 0;
+  if (FAR_ONLY && p.far_parts > 1) {
+    const int n_far = t_near0 + (n_tiles - t_near1);
+    const int o_lo = (int)((int64_t)n_far * part / p.far_parts), o_hi = (int)((int64_t)n_far * (part + 1) / p.far_parts);
+    zl0 = min(o_lo, t_near0);
+    zl1 = min(o_hi, t_near0);
+    zr0 = t_near1 + max(o_lo - t_near0, 0);
+    zr1 = t_near1 + max(o_hi - t_near0, 0);
+  }
   // the tile walked after tile t (far-only runs jump over the near range, ring runs walk nothing else)
-  const int t_end = RING ? t_near1 : n_tiles;
+  const int t_end = RING ? t_near1 : zr1;
   auto next_tile = [&](int t) __attribute__((always_inline)) {
-    return (FAR_ONLY && t + 1 >= t_near0 && t + 1 < t_near1) ? t_near1 : t + 1;
+    return (FAR_ONLY && t + 1 >= zl1 && t + 1 < zr0) ? zr0 : t + 1;
   };
   // Two ways of staging the K and V tiles.
   //
@@ -498,7 +511,7 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
     }
   };
   {
-    const int first = RING ? t_near0 : next_tile(-1);
+    const int first = RING ? t_near0 : next_tile(zl0 - 1);
     if (first < t_end) {
       if constexpr (DMA) {
         dma_issue(first, 0);
@@ -604,7 +617,7 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
   };
 
   // ---- far-left ------------------------------------------------------------------------------
-  if constexpr (!RING) far_range(0, t_near0, 0);
+  if constexpr (!RING) far_range(zl0, zl1, 0);
 
   // ---- near ----------------------------------------------------------------------------------
   if constexpr (RING) {
@@ -929,7 +942,7 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
   }
 
   // ---- far-right -----------------------------------------------------------------------------
-  if constexpr (!RING) far_range(t_near1, n_tiles, 1);
+  if constexpr (!RING) far_range(zr0, zr1, 1);
 
   // ---- epilogue ------------------------------------------------------------------------------
   const float l_tot = wave_half_sum(l_run);
@@ -969,7 +982,13 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
   }
   const float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
   if (i < Lb) {
+    const int64_t tok = p.cu ? (int64_t)tok0 + i : (int64_t)b * p.L + tok0 + i;
     char* orow = ob + (int64_t)i * p.o_st * VT::SZ;
+    float* lse_row = p.lse;
+    if (FAR_ONLY && part > 0) {  // the partial results after the first go to the workspace, token-major
+      orow = far_part_out(p, part, D * VT::SZ) + (tok * p.H + h) * (D * VT::SZ);
+      lse_row = far_part_lse(p, part, D * VT::SZ);
+    }
 #pragma unroll
     for (int d = 0; d < C::DBLKS; ++d)
 #pragma unroll
@@ -978,10 +997,7 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
         VT::store4(orow + dd * VT::SZ, o_acc[d][4 * q4] * inv, o_acc[d][4 * q4 + 1] * inv,
                    o_acc[d][4 * q4 + 2] * inv, o_acc[d][4 * q4 + 3] * inv);
       }
-    if (p.lse && g == 0) {
-      const int64_t tok = p.cu ? (int64_t)tok0 + i : (int64_t)b * p.L + tok0 + i;
-      p.lse[tok * p.H + h] = (m_run + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
-    }
+    if (lse_row && g == 0) lse_row[tok * p.H + h] = (m_run + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
   }
 }
 
@@ -993,7 +1009,8 @@ int launch_one(const FdbKParams& p, int grid_x, hipStream_t stream) {
   static_assert(lds <= 160 * 1024, "LDS budget");
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
   if (e != hipSuccess) return (int)e;
-  hipLaunchKernelGGL(kern, dim3((unsigned)grid_x * p.H, 1, 1), dim3(kThreads), lds, stream, p);
+  const unsigned parts = MODE == kFarOnly && p.far_parts > 1 ? (unsigned)p.far_parts : 1u;
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid_x * p.H, parts, 1), dim3(kThreads), lds, stream, p);
   return (int)hipGetLastError();
 }
 

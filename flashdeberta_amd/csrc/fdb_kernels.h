@@ -33,10 +33,27 @@ struct FdbKParams {
   int32_t B, H, L, tiles_per_seq;
   int32_t grid_x;   // query tiles in the launch (the grid is grid_x * H workgroups)
   int32_t R;        // LUT radius
-  int32_t far_done; // ring mode only: the far tiles' partial result is already in out / lse
+  int32_t far_done;  // near launches: the far tiles' partial results (far_parts of them) are to be merged
+  int32_t far_parts; // workgroups per query tile of the far-only launch, each with its share of the far tiles and a
+                     // partial result of its own (the first in out / lse)
+  char* ws;          // partial results 1 .. far_parts-1: [far_parts-1][ws_rows][H][D] elements of v's type,
+  int64_t ws_rows;   // then [far_parts-1][ws_rows][H] float log-sum-exps; ws_rows = rows of the lse buffer
   int32_t causal;
   float scale_log2; // sm_scale * log2(e)
 };
+
+// Where far partial result `part` >= 1 lives in the workspace (row_bytes = head_dim * element size).
+#if defined(__HIPCC__)
+__device__ __forceinline__ char* far_part_out(const FdbKParams& p, int part, int row_bytes) {
+  return p.ws + (int64_t)(part - 1) * p.ws_rows * p.H * row_bytes;
+}
+__device__ __forceinline__ float* far_part_lse(const FdbKParams& p, int part, int row_bytes) {
+  return (float*)(p.ws + (int64_t)(p.far_parts - 1) * p.ws_rows * p.H * row_bytes) + (int64_t)(part - 1) * p.ws_rows * p.H;
+}
+#endif
+
+// Most workgroups per query tile a far-only launch is split into.
+#define FDB_MAX_FAR_PARTS 4
 
 // Launchers return the hipError_t of the launch as int.
 // fdb_launch_attn, by mode:

@@ -424,28 +424,49 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
   if (i < Lb) {
     char* orow = ob + (int64_t)i * p.o_st * 2;
     const int64_t tok = p.cu ? (int64_t)tok0 + i : (int64_t)b * p.L + tok0 + i;
-    float w_far = 0.f, w_near = 1.f, m_out = m_run;
-    if (p.far_done) {
-      const float lf = p.lse[tok * p.H + h] * 1.4426950408889634f;  // far log-sum-exp, base 2 (-inf: no far tile)
-      const float ln_ = m_run + __builtin_amdgcn_logf(l_tot);
-      m_out = fmaxf(lf, ln_);
-      w_far = __builtin_amdgcn_exp2f(lf - m_out);
+    // far partial results: part 0 in out / lse, the others in the workspace (rows normalised over their
+    // keys, log-sum-exp -inf where a row had none)
+    const int n_far = p.far_done ? p.far_parts : 0;
+    float w_far[FDB_MAX_FAR_PARTS], w_near = 1.f, m_out = m_run;
+    const char* far_row[FDB_MAX_FAR_PARTS];
+#pragma unroll
+    for (int s = 0; s < FDB_MAX_FAR_PARTS; ++s) {
+      w_far[s] = -INFINITY;  // log-sum-exp in base 2 until the maximum is known
+      far_row[s] = orow;
+      if (s < n_far) {
+        const float* lp = s == 0 ? p.lse : far_part_lse(p, s, D * 2);
+        w_far[s] = lp[tok * p.H + h] * 1.4426950408889634f;
+        if (s > 0) far_row[s] = far_part_out(p, s, D * 2) + (tok * p.H + h) * (D * 2);
+      }
+    }
+    if (n_far > 0) {
+      m_out = m_run + __builtin_amdgcn_logf(l_tot);
+#pragma unroll
+      for (int s = 0; s < FDB_MAX_FAR_PARTS; ++s) m_out = fmaxf(m_out, w_far[s]);
       w_near = __builtin_amdgcn_exp2f(m_run - m_out);
     }
-    const float denom = w_far + w_near * l_tot;
+    float denom = w_near * l_tot;
+#pragma unroll
+    for (int s = 0; s < FDB_MAX_FAR_PARTS; ++s) {
+      w_far[s] = (s < n_far && w_far[s] != -INFINITY) ? __builtin_amdgcn_exp2f(w_far[s] - m_out) : 0.f;
+      denom += w_far[s];
+    }
     const float inv = denom > 0.f ? 1.f / denom : 0.f;
-    const float sn = w_near * inv, sf = w_far * inv;
+    const float sn = w_near * inv;
 #pragma unroll
     for (int d = 0; d < DBLKS; ++d)
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
-        char* dst = orow + (32 * d + 8 * q4 + 4 * g) * 2;
+        const int off = (32 * d + 8 * q4 + 4 * g) * 2;
         float f0 = 0.f, f1 = 0.f, f2 = 0.f, f3 = 0.f;
-        if (p.far_done) {
-          const f32x4 far4 = VT::load4(dst);
-          f0 = far4[0] * sf; f1 = far4[1] * sf; f2 = far4[2] * sf; f3 = far4[3] * sf;
-        }
-        VT::store4(dst, o_acc[d][4 * q4] * sn + f0, o_acc[d][4 * q4 + 1] * sn + f1, o_acc[d][4 * q4 + 2] * sn + f2,
+#pragma unroll
+        for (int s = 0; s < FDB_MAX_FAR_PARTS; ++s)
+          if (s < n_far) {
+            const f32x4 far4 = VT::load4(far_row[s] + off);
+            const float sf = w_far[s] * inv;
+            f0 += far4[0] * sf; f1 += far4[1] * sf; f2 += far4[2] * sf; f3 += far4[3] * sf;
+          }
+        VT::store4(orow + off, o_acc[d][4 * q4] * sn + f0, o_acc[d][4 * q4 + 1] * sn + f1, o_acc[d][4 * q4 + 2] * sn + f2,
                    o_acc[d][4 * q4 + 3] * sn + f3);
       }
     if (p.lse && g == 0) p.lse[tok * p.H + h] = (m_out + __builtin_amdgcn_logf(denom)) * 0.6931471805599453f;

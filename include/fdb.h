@@ -4,8 +4,8 @@
  * The library is a plain shared object (libfdb_hip.so): C linkage, raw device pointers,
  * integer sizes and strides, no C++ or torch types in any signature.  It never allocates or
  * frees device memory and keeps no pointer after a call returns; every buffer, including the
- * output, the optional log-sum-exp, the varlen work-list and the delta look-up table, is
- * owned by the caller.  All launches are asynchronous on the stream passed in.
+ * output, the optional log-sum-exp, the varlen work-list, the delta look-up table and the
+ * optional workspace, is owned by the caller.  All launches are asynchronous on the stream passed in.
  *
  * Reference interfaces replaced (paths relative to the FlashDeBERTa repository):
  *   fdb_attn_fwd           <- flash_attention_with_disentangled
@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define FDB_VERSION 1
+#define FDB_VERSION 2
 
 /* element types of q/k/pos_key/pos_query (v and out: see fdb_attn_args.dtype) */
 enum fdb_dtype {
@@ -93,12 +93,14 @@ typedef struct fdb_attn_args {
   const float* k_scale;
   const float* pk_scale;
   const float* pq_scale;
+  void* workspace;         /* device scratch of workspace_bytes bytes, 16-byte aligned, or NULL: see fdb_attn_workspace_bytes */
   int64_t q_stride_b, q_stride_t, q_stride_h;
   int64_t k_stride_b, k_stride_t, k_stride_h;
   int64_t v_stride_b, v_stride_t, v_stride_h;
   int64_t o_stride_b, o_stride_t, o_stride_h;
   int64_t pk_stride_h, pk_stride_r;
   int64_t pq_stride_h, pq_stride_r;
+  int64_t workspace_bytes;
   int32_t batch;
   int32_t heads;
   int32_t head_dim;
@@ -108,8 +110,11 @@ typedef struct fdb_attn_args {
   int32_t lut_radius;
   int32_t dtype;           /* enum fdb_dtype                                                 */
   int32_t causal;          /* nonzero: key j visible to query i only if j <= i               */
+  int32_t far_splits;      /* 0: the library decides; 1 .. FDB_MAX_FAR_SPLITS: workgroups that share the far keys of a query tile */
   float sm_scale;
 } fdb_attn_args;
+
+#define FDB_MAX_FAR_SPLITS 4
 
 int fdb_version(void);
 /* sizeof(fdb_attn_args) as the library was built: lets a foreign-language binding check its struct mirror. */
@@ -121,6 +126,18 @@ int fdb_attn_check(const fdb_attn_args* a);
 
 /* Enqueue the fused forward on `stream` (a hipStream_t). */
 int fdb_attn_fwd(const fdb_attn_args* a, void* stream);
+
+/*
+ * Bytes of workspace the call would use (0: none), for the device that is current.  A launch whose
+ * query tiles fill at most half of the workgroups the GPU holds shares the far keys of each query tile (those
+ * whose bucketed relative position is constant) among up to FDB_MAX_FAR_SPLITS workgroups, whose partial results go
+ * through the workspace: (splits - 1) * rows * heads * (head_dim * sizeof(v element) + 4) bytes, rows being
+ * the rows of the lse buffer.  The workspace is optional: without it (or with a smaller one) the call
+ * uses as many splits as fit, down to one, with the same result up to rounding.  far_splits and the
+ * workspace fields of `a` are read (far_splits) and ignored (workspace, workspace_bytes) here.  No
+ * counterpart in the reference, whose kernels have one program per query tile (flash_attention.py:465-488).
+ */
+int64_t fdb_attn_workspace_bytes(const fdb_attn_args* a);
 
 /* Number of int32 the varlen work-list needs for (total_tokens, batch): 2 ints per possible
  * q-tile plus a header.  Depends on shapes only, so no device sync is needed to size it. */

@@ -33,7 +33,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_struct_mirror_and_version():
     assert lib.fdb_attn_args_size() == ctypes.sizeof(FdbAttnArgs)
-    assert lib.fdb_version() == 1
+    assert lib.fdb_version() == 2
     assert lib.fdb_tile_rows() == 128
 
 
@@ -114,6 +114,36 @@ def test_argument_validation_codes():
     assert lib.fdb_quant_e4m3_per_head(None, 0, 0, None, 0, 0, None, None, 1, 1, 64, None) == -1
     assert lib.fdb_dequant_e4m3_per_head(None, 0, 0, None, None, 0, 0, 1, 1, 64, None) == -1
     assert lib.fdb_dequant_e4m3_per_head(0x4000, 64, 64, 0x5000, 0x6000, 64, 64, 1, 1, 48, None) == -3
+
+
+def test_far_split_policy_and_workspace_size():
+    """Host-only: how many workgroups share a query tile's far keys, and the workspace that takes (without a
+    GPU the library assumes 256 compute units, i.e. 768 far workgroups in flight)."""
+    ws = lambda a: lib.fdb_attn_workspace_bytes(ctypes.byref(a))
+    chk = lambda a: lib.fdb_attn_check(ctypes.byref(a))
+    part = lambda rows, heads: rows * heads * (64 * 2 + 4)
+
+    def args(batch, seqlen, heads=12, lse=0x5000):
+        a = _good_args()
+        a.batch, a.heads, a.max_seqlen, a.total_tokens, a.lse = batch, heads, seqlen, batch * seqlen, lse
+        return a
+
+    assert ws(args(1, 4096)) == part(4096, 12)            # 384 query tiles -> 2 x 384 = one full round
+    assert ws(args(1, 4096, heads=16)) == 0               # 512: two shares would need a second round
+    assert ws(args(1, 4096, heads=8)) == 2 * part(4096, 8)  # 256 -> 3 x 256
+    assert ws(args(2, 4096)) == 0 and ws(args(8, 4096)) == 0  # the launch fills the slots by itself
+    assert ws(args(1, 2048)) == 0                         # too few far tiles to share out
+    assert ws(args(8, 512)) == 0                          # no far tile at all
+    assert ws(args(1, 4096, lse=None)) == 0               # one fused kernel without the lse buffer
+    a = args(8, 4096); a.far_splits = 4; assert ws(a) == 3 * part(8 * 4096, 12)
+    a = args(1, 4096); a.far_splits = 1; assert ws(a) == 0
+    a = args(1, 4096); a.dtype = _lib.FDB_F32; a.far_splits = 3; assert ws(a) == 0   # fp32 takes the fused kernel
+    a = args(1, 4096); a.cu_seqlens, a.worklist = 0x6000, 0x7000; assert ws(a) == 0   # lengths unknown to the host
+    a.far_splits = 2; assert ws(a) == part(4096, 12)
+    a = args(1, 4096); a.far_splits = 5; assert chk(a) == -5 and ws(a) == 0
+    a = args(1, 4096); a.far_splits = -1; assert chk(a) == -5
+    a = args(1, 4096); a.workspace, a.workspace_bytes = 0x8008, 1 << 20; assert chk(a) == -4
+    a = args(1, 4096); a.workspace, a.workspace_bytes = 0x8000, -1; assert chk(a) == -5
 
 
 def test_error_strings_and_python_mapping():

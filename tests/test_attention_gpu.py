@@ -148,6 +148,52 @@ def test_two_launch_variants(causal, c2p, p2c, D, L):
     _check(lse.view(2, L, 2), ref_lse, 4 * TOL[torch.bfloat16], "lse")
 
 
+@pytest.mark.parametrize("splits", [2, 3, 4])
+@pytest.mark.parametrize("L,pb,mr,causal,c2p,p2c,dtype", [
+    (1500, 256, 512, False, True, True, torch.bfloat16),   # three to six far tiles per query tile: empty shares too
+    (900, 32, 64, False, True, True, torch.float16),       # small radius: most tiles far, on both sides
+    (900, 32, 64, True, True, True, torch.bfloat16),       # causal: far tiles on the left only
+    (1100, 16, 32, False, False, True, torch.bfloat16),    # one position term
+    (833, 32, 64, False, True, False, torch.bfloat16),     # ragged last tile in the far zone
+])
+def test_far_keys_shared_among_workgroups(splits, L, pb, mr, causal, c2p, p2c, dtype):
+    """The far-only launch with several workgroups per query tile, each leaving a partial result that the
+    near launch merges: same result as with one, and both match the oracle (output and log-sum-exp)."""
+    q, k, v, pk, pq = _inputs(2, L, 2, 64, pb, mr, dtype, 500 + L + splits, 1.0, c2p, p2c)
+    ref, ref_lse = _oracle_blhd(q, k, v, pk, pq, pb, mr, causal=causal, return_lse=True)
+    args = [_dev(x) for x in (q, k, v, pk, pq)]
+    kw = dict(position_buckets=pb, max_relative_positions=mr, causal=causal, return_lse=True)
+    out, lse = ops.disentangled_attention_fwd(*args, far_splits=splits, **kw)
+    one, _ = ops.disentangled_attention_fwd(*args, far_splits=1, **kw)
+    _check(out, ref, TOL[dtype], "out")
+    _check(lse.view(2, L, 2), ref_lse, 4 * TOL[dtype], "lse")
+    assert (out.float() - one.float()).abs().max().item() <= TOL[dtype]
+
+
+def test_far_keys_shared_packed_and_padded():
+    """Shared far keys with packed sequences (work-list launch) and with a padded batch."""
+    pb, mr, H, D = 32, 64, 2, 64
+    lens = [700, 130, 1, 1000]
+    q, k, v, pk, pq = _inputs(1, sum(lens), H, D, pb, mr, torch.bfloat16, 611, 1.0)
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+    kw = dict(position_buckets=pb, max_relative_positions=mr)
+    out = ops.disentangled_attention_fwd(_dev(q[0]), _dev(k[0]), _dev(v[0]), _dev(pk), _dev(pq), cu_seqlens=cu.cuda(),
+                                         max_seqlen=max(lens), far_splits=3, **kw)
+    Lmax = max(lens)
+    pad = lambda x: torch.stack([torch.nn.functional.pad(x[0, cu[b]:cu[b + 1]], (0, 0, 0, 0, 0, Lmax - lens[b]))
+                                 for b in range(len(lens))])
+    padded = torch.zeros(len(lens), Lmax, H, D, dtype=torch.bfloat16, device="cuda")
+    ops.disentangled_attention_fwd(_dev(pad(q)), _dev(pad(k)), _dev(pad(v)), _dev(pk), _dev(pq), out=padded,
+                                   seq_len=torch.tensor(lens, dtype=torch.int32).cuda(), far_splits=4, **kw)
+    off = 0
+    for b, n in enumerate(lens):
+        sl = slice(off, off + n)
+        ref = _oracle_blhd(q[:, sl], k[:, sl], v[:, sl], pk, pq, pb, mr)
+        _check(out[sl][None], ref, TOL[torch.bfloat16], "packed, length %d" % n)
+        _check(padded[b, :n][None], ref, TOL[torch.bfloat16], "padded, length %d" % n)
+        off += n
+
+
 @pytest.mark.parametrize("seed", [1, 2])
 def test_seeded_random_shapes(seed):
     """Sixteen shapes per seed drawn around the boundaries that change the code path (one query tile,
