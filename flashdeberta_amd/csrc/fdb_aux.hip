@@ -10,12 +10,41 @@
 namespace {
 
 constexpr int kWlThreads = 256;
+constexpr int kWlSortMax = 1024;  // batches up to this size get their tiles ordered by sequence length
 
-// wl[0] = number of tiles, wl[1] = 0, then (sequence, first row) pairs in sequence order.
+// wl[0] = number of tiles, wl[1] = 0, then (sequence, first row) pairs: the tiles of the longest
+// sequence first (ties in sequence order), so that a launch starts on the workgroups with the most
+// key tiles and ends on the short ones.  Each thread places its sequences by summing the tiles of
+// all sequences that come before them in that order (batch^2 / 256 steps per thread, the lengths in
+// LDS); larger batches keep the sequence order and a prefix sum.
 __global__ __launch_bounds__(kWlThreads) void fdb_worklist_kernel(const int32_t* __restrict__ cu, int32_t batch,
                                                                   int32_t* __restrict__ wl, int32_t max_tiles) {
   __shared__ int32_t part[kWlThreads];
+  __shared__ int32_t lens[kWlSortMax];
   const int t = threadIdx.x;
+  if (batch <= kWlSortMax) {
+    for (int b = t; b < batch; b += kWlThreads) lens[b] = max(cu[b + 1] - cu[b], 0);
+    __syncthreads();
+    for (int b = t; b < batch; b += kWlThreads) {
+      const int len = lens[b];
+      int32_t pos = 0, total = 0;
+      for (int c = 0; c < batch; ++c) {
+        const int lc = lens[c], tiles = (lc + FDB_BM - 1) / FDB_BM;
+        total += tiles;
+        if (lc > len || (lc == len && c < b)) pos += tiles;
+      }
+      if (b == 0) {
+        wl[0] = min(total, max_tiles);
+        wl[1] = 0;
+      }
+      for (int m0 = 0; m0 < len; m0 += FDB_BM, ++pos)
+        if (pos < max_tiles) {
+          wl[2 + 2 * pos] = b;
+          wl[3 + 2 * pos] = m0;
+        }
+    }
+    return;
+  }
   const int per = (batch + kWlThreads - 1) / kWlThreads;
   const int b_lo = min(batch, t * per), b_hi = min(batch, b_lo + per);
   int32_t cnt = 0;

@@ -277,9 +277,14 @@ __device__ __forceinline__ void block_map(int n, int nx, int heads, int tiles_pe
     }
     xq = (grp / heads) * tiles_per_seq + t;
     h = grp % heads;
-  } else {
+  } else if (fixed) {
     xq = n % nx;
     h = n / nx;
+  } else {
+    // packed sequences: the work-list holds the tiles longest sequence first; all heads of a tile are
+    // dealt before the next tile, so the whole launch runs from long workgroups to short ones
+    xq = n / heads;
+    h = n % heads;
   }
 }
 

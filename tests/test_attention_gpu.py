@@ -297,7 +297,7 @@ def test_worklist_on_device():
     from flashdeberta_amd._lib import lib
     import ctypes
     rng = np.random.default_rng(3)
-    for B in (1, 7, 300, 1000):
+    for B in (1, 7, 300, 1000, 1500):
         lens = rng.integers(0, 600, size=B)
         cu = torch.from_numpy(np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)).cuda()
         T = int(lens.sum())
@@ -306,7 +306,9 @@ def test_worklist_on_device():
                                     ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
         assert rc == 0
         w = wl.cpu().numpy()
-        want = [(b, m0) for b in range(B) for m0 in range(0, int(lens[b]), 128)]
+        # the tiles of the longest sequence first, ties in sequence order (batches above 1024: sequence order)
+        order = sorted(range(B), key=lambda b: (-int(lens[b]), b)) if B <= 1024 else range(B)
+        want = [(b, m0) for b in order for m0 in range(0, int(lens[b]), 128)]
         assert w[0] == len(want)
         assert w[2:2 + 2 * len(want)].reshape(-1, 2).tolist() == [list(x) for x in want]
 
