@@ -80,7 +80,9 @@ __global__ void fdb_fill_u32(uint32_t* p, int n, uint32_t v) {
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __builtin_bit_cast(float, (uint32_t)b << 16); }
 
-// grid (token blocks, heads); each thread owns 8 consecutive d of one token.
+// grid (token blocks, heads); each thread owns 8 consecutive d of one token.  One atomic per
+// workgroup: all of a head's atomics hit one address and are served one after the other (one per wave
+// from 1024 workgroups per head took 560 us for 50 MB), so the launch also keeps the workgroups few.
 template <int D>
 __global__ __launch_bounds__(256) void fdb_absmax_kernel(const uint16_t* __restrict__ x, int64_t st, int64_t sh,
                                                          uint32_t* __restrict__ absmax, int32_t tokens) {
@@ -100,7 +102,13 @@ __global__ __launch_bounds__(256) void fdb_absmax_kernel(const uint16_t* __restr
     }
   }
   for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
-  if ((threadIdx.x & 63) == 0) atomicMax(absmax + h, __builtin_bit_cast(uint32_t, m));  // m >= 0: bit order = value order
+  __shared__ float wave_max[4];
+  if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    m = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
+    atomicMax(absmax + h, __builtin_bit_cast(uint32_t, m));  // m >= 0: bit order = value order
+  }
 }
 
 template <int D>
@@ -197,8 +205,10 @@ int fdb_launch_quant(const void* x, int64_t x_st, int64_t x_sh, void* y, int64_t
   int gx = (int)((chunks + 255) / 256);
   if (gx > 1024) gx = 1024;
   if (gx < 1) gx = 1;
+  int gx_max = 2048 / heads > 1 ? 2048 / heads : 1;  // about 2048 workgroups, i.e. atomics, in all
+  if (gx_max > gx) gx_max = gx;
 #define FDB_Q(DD)                                                                                              \
-  hipLaunchKernelGGL(fdb_absmax_kernel<DD>, dim3(gx, heads), dim3(256), 0, stream, (const uint16_t*)x, x_st,   \
+  hipLaunchKernelGGL(fdb_absmax_kernel<DD>, dim3(gx_max, heads), dim3(256), 0, stream, (const uint16_t*)x, x_st, \
                      x_sh, absmax_ws, tokens);                                                                 \
   hipLaunchKernelGGL(fdb_quant_kernel<DD>, dim3(gx, heads), dim3(256), 0, stream, (const uint16_t*)x, x_st,    \
                      x_sh, (uint8_t*)y, y_st, y_sh, absmax_ws, scale, tokens);
