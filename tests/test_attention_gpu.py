@@ -194,6 +194,36 @@ def test_far_keys_shared_packed_and_padded():
         off += n
 
 
+@pytest.mark.parametrize("B,L,splits", [(2, 700, 0), (1, 1500, 2)])
+def test_operator_replays_from_a_hip_graph(B, L, splits):
+    """The operator enqueues only kernels on the current stream and allocates through torch, so it can be
+    captured into a HIP graph: three replays on fresh input values, with eager calls and synchronisations
+    in between, each equal to the eager result on the same values."""
+    pb, mr, H, D = 32, 64, 2, 64
+    kw = dict(position_buckets=pb, max_relative_positions=mr, far_splits=splits)
+    q, k, v, pk, pq = [_dev(x) for x in _inputs(B, L, H, D, pb, mr, torch.bfloat16, 900, 1.0)]
+    ops.disentangled_attention_fwd(q, k, v, pk, pq, **kw)  # the delta table reaches the device outside the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            out = ops.disentangled_attention_fwd(q, k, v, pk, pq, **kw)
+    torch.cuda.current_stream().wait_stream(side)
+    g = torch.Generator().manual_seed(901)
+    for it in range(3):
+        for x in (q, k, v):
+            x.copy_(torch.randn(x.shape, generator=g).to(torch.bfloat16))
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = ops.disentangled_attention_fwd(q, k, v, pk, pq, **kw)
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), "replay %d differs from the eager call" % it
+    ref = _oracle_blhd(q.cpu(), k.cpu(), v.cpu(), pk.cpu(), pq.cpu(), pb, mr)
+    _check(out, ref, TOL[torch.bfloat16], "last replay")
+
+
 @pytest.mark.parametrize("seed", [1, 2])
 def test_seeded_random_shapes(seed):
     """Sixteen shapes per seed drawn around the boundaries that change the code path (one query tile,
