@@ -24,7 +24,8 @@ class FdbAttnArgs(ctypes.Structure):
             "v_stride_b", "v_stride_t", "v_stride_h", "o_stride_b", "o_stride_t", "o_stride_h",
             "pk_stride_h", "pk_stride_r", "pq_stride_h", "pq_stride_r", "workspace_bytes")]
         + [(n, ctypes.c_int32) for n in (
-            "batch", "heads", "head_dim", "max_seqlen", "total_tokens", "att_span", "lut_radius", "dtype", "causal", "far_splits")]
+            "batch", "heads", "head_dim", "max_seqlen", "total_tokens", "att_span", "lut_radius", "dtype", "causal", "far_splits",
+            "near_splits")]
         + [("sm_scale", ctypes.c_float)]
     )
 

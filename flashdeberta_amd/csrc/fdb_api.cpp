@@ -115,6 +115,26 @@ int far_parts_wanted(const fdb_attn_args* a) {
   return n > 1 ? n : 1;
 }
 
+// The same for the near launch, which keeps two workgroups on a CU.  Every share repeats the prologue
+// (five batches of table rows) and a merge kernel follows, so a share keeps at least sixteen 32-key
+// steps, or eight when all shares together fill at most half of the slots.  (Measured, 12 heads: one
+// sequence of 1024: 0.056 -> 0.040 ms; one of 512: 0.025 -> 0.022; four of 512 in shares of eight
+// steps would go from 0.025 to 0.028.)
+int near_parts_wanted(const fdb_attn_args* a) {
+  if (!(a->pos_key || a->pos_query) || !a->lse || !fdb_near32_supported(a->dtype, a->head_dim)) return 1;
+  if (a->near_splits > 0) return a->near_splits;
+  if (a->cu_seqlens) return 1;
+  const int64_t wgs = query_tiles(a) * a->heads, slots = 2 * (int64_t)cu_count();
+  const int steps_all = (a->max_seqlen + 31) / 32, steps_near = (FDB_BM + 2 * a->lut_radius + 3 * (FDB_BN - 1)) / 32;
+  const int steps = steps_all < steps_near ? steps_all : steps_near;
+  int best = 1;
+  for (int n = 2; n <= FDB_MAX_FAR_PARTS && wgs * n <= slots; ++n) {
+    const int per = steps / n;
+    if (per >= 16 || (per >= 8 && wgs * n <= slots / 2)) best = n;
+  }
+  return best;
+}
+
 int64_t lse_rows(const fdb_attn_args* a) {
   return a->cu_seqlens ? (int64_t)a->total_tokens : (int64_t)a->batch * a->max_seqlen;
 }
@@ -174,7 +194,9 @@ int fdb_attn_check(const fdb_attn_args* a) {
   if (a->dtype == FDB_F32 && a->head_dim == 128) return FDB_ERR_UNSUPPORTED;
   if (a->batch < 1 || a->heads < 1 || a->heads > 65535 || a->max_seqlen < 1 || a->total_tokens < 1)
     return FDB_ERR_SHAPE;
-  if (a->far_splits < 0 || a->far_splits > FDB_MAX_FAR_SPLITS || a->workspace_bytes < 0) return FDB_ERR_SHAPE;
+  if (a->far_splits < 0 || a->far_splits > FDB_MAX_FAR_SPLITS || a->near_splits < 0 ||
+      a->near_splits > FDB_MAX_FAR_SPLITS || a->workspace_bytes < 0)
+    return FDB_ERR_SHAPE;
   if (a->workspace && !aligned16(a->workspace)) return FDB_ERR_ALIGN;
   if (!a->cu_seqlens && (int64_t)a->batch * a->max_seqlen != a->total_tokens) return FDB_ERR_SHAPE;
   if (a->cu_seqlens && !a->worklist) return FDB_ERR_WORKLIST;
@@ -203,7 +225,8 @@ int fdb_attn_check(const fdb_attn_args* a) {
 
 int64_t fdb_attn_workspace_bytes(const fdb_attn_args* a) {
   if (fdb_attn_check(a) != FDB_OK) return 0;
-  return (far_parts_wanted(a) - 1) * far_part_bytes(a);
+  const int near = near_parts_wanted(a);
+  return (far_parts_wanted(a) - 1 + (near > 1 ? near : 0)) * far_part_bytes(a);
 }
 
 int fdb_attn_fwd(const fdb_attn_args* a, void* stream) {
@@ -243,20 +266,26 @@ int fdb_attn_fwd(const fdb_attn_args* a, void* stream) {
   // hand-over between the two launches.
   if ((a->pos_key || a->pos_query) && a->lse && fdb_near_supported(a->dtype, a->head_dim)) {
     const bool need_far = has_far_launch(a);  // otherwise no tile of any query tile is far
-    p.far_parts = 1;
+    // as many workgroups per query tile as wanted and as the workspace holds partial results for
+    p.far_parts = need_far ? far_parts_wanted(a) : 1;
+    p.near_parts = near_parts_wanted(a);
+    const int64_t ws_slots_have = a->workspace ? a->workspace_bytes / far_part_bytes(a) : 0;
+    if (p.near_parts > 1 && ws_slots_have < p.far_parts - 1 + p.near_parts) p.near_parts = 1;
+    while (p.far_parts > 1 && ws_slots_have < p.far_parts - 1 + (p.near_parts > 1 ? p.near_parts : 0)) --p.far_parts;
+    p.ws_slots = p.far_parts - 1 + (p.near_parts > 1 ? p.near_parts : 0);
+    p.ws = (char*)a->workspace;
+    p.ws_rows = lse_rows(a);
     if (need_far) {
-      // as many workgroups per query tile as wanted and as the workspace holds partial results for
-      p.far_parts = far_parts_wanted(a);
-      const int64_t part_bytes = far_part_bytes(a);
-      while (p.far_parts > 1 && (!a->workspace || a->workspace_bytes / part_bytes < p.far_parts - 1)) --p.far_parts;
-      p.ws = (char*)a->workspace;
-      p.ws_rows = lse_rows(a);
       const int rc_far = fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, FDB_MODE_FAR_ONLY, stream);
       if (rc_far != 0) return rc_far;
     }
     p.far_done = need_far ? 1 : 0;
     // head_dim 64: the near kernel (32-key steps, two workgroups per CU); head_dim 32: the fused kernel's ring mode
-    if (fdb_near32_supported(a->dtype, a->head_dim)) return fdb_launch_near32(p, a->dtype, (int)grid_x, stream);
+    if (fdb_near32_supported(a->dtype, a->head_dim)) {
+      const int rc_near = fdb_launch_near32(p, a->dtype, (int)grid_x, stream);
+      if (rc_near != 0 || p.near_parts <= 1) return rc_near;
+      return fdb_launch_merge(p, a->dtype, stream);
+    }
     return fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, FDB_MODE_NEAR_RING, stream);
   }
   return fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, FDB_MODE_FUSED, stream);

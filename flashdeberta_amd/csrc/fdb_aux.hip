@@ -5,7 +5,9 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "fdb_device.h"
 #include "fdb_kernels.h"
+#include "../../include/fdb.h"
 
 namespace {
 
@@ -194,6 +196,90 @@ int fdb_launch_dequant(const void* y, int64_t y_st, int64_t y_sh, const float* s
 
 int fdb_launch_worklist(const int32_t* cu, int32_t batch, int32_t* wl, int32_t max_tiles, void* stream) {
   hipLaunchKernelGGL(fdb_worklist_kernel, dim3(1), dim3(kWlThreads), 0, (hipStream_t)stream, cu, batch, wl, max_tiles);
+  return (int)hipGetLastError();
+}
+
+// ---- merge of partial results -------------------------------------------------------------------------
+// After a near launch whose workgroups each took a share of a query tile's steps: every partial result is
+// a set of rows normalised over the keys it saw plus their log-sum-exp (-inf: none seen).  The far ones
+// (when p.far_done: the first in out / lse, the others in workspace slots 0 .. far_parts-2) and the near
+// ones (slots far_parts-1 ..) are combined with weights exp(lse_s - max) into out and lse.  One thread
+// per eight elements of a (token, head) row; padded rows of a fixed-layout batch are left alone.
+namespace {
+
+template <class VT>
+__global__ __launch_bounds__(256) void fdb_merge_kernel(const FdbKParams p) {
+  constexpr int D = 64, CPR = D / 8, RB = D * 2;
+  const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= p.ws_rows * p.H * CPR) return;
+  const int cc = (int)(c % CPR);
+  const int64_t row = c / CPR;  // tok * H + h
+  const int h = (int)(row % p.H);
+  const int64_t tok = row / p.H;
+  char* dst;
+  if (p.cu) {
+    dst = p.out + (tok * p.o_st + (int64_t)h * p.o_sh) * 2;
+  } else {
+    const int b = (int)(tok / p.L), l = (int)(tok % p.L);
+    const int t0 = p.seq_start ? min(max(p.seq_start[b], 0), p.L) : 0;
+    const int len = p.seq_len ? min(max(p.seq_len[b], 0), p.L - t0) : p.L;
+    if (l < t0 || l >= t0 + len) return;
+    dst = p.out + ((int64_t)b * p.o_sb + (int64_t)l * p.o_st + (int64_t)h * p.o_sh) * 2;
+  }
+  dst += cc * 16;
+  constexpr int kMax = 2 * FDB_MAX_FAR_PARTS;
+  const int n_far = p.far_done ? p.far_parts : 0, n = n_far + p.near_parts;
+  float w[kMax], m = -INFINITY;
+  const char* src[kMax];
+#pragma unroll
+  for (int s = 0; s < kMax; ++s) {
+    w[s] = -INFINITY;
+    src[s] = dst;
+    if (s < n) {
+      // source s: far part s (s < n_far), else near part s - n_far
+      const int slot = s < n_far ? s - 1 : p.far_parts - 1 + (s - n_far);
+      const float* lp = slot < 0 ? p.lse : ws_slot_lse(p, slot, RB);
+      w[s] = lp[row] * 1.4426950408889634f;
+      if (slot >= 0) src[s] = ws_slot_out(p, slot, RB) + row * RB + cc * 16;
+      m = fmaxf(m, w[s]);
+    }
+  }
+  float denom = 0.f;
+#pragma unroll
+  for (int s = 0; s < kMax; ++s) {
+    w[s] = (s < n && w[s] != -INFINITY) ? __builtin_amdgcn_exp2f(w[s] - m) : 0.f;
+    denom += w[s];
+  }
+  const float inv = denom > 0.f ? 1.f / denom : 0.f;
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int s = 0; s < kMax; ++s)
+    if (s < n && w[s] > 0.f) {
+      const f32x4 lo = VT::load4(src[s]);
+      const f32x4 hi = VT::load4(src[s] + 8);
+      const float f = w[s] * inv;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        acc[e] = __builtin_fmaf(lo[e], f, acc[e]);
+        acc[4 + e] = __builtin_fmaf(hi[e], f, acc[4 + e]);
+      }
+    }
+  VT::store4(dst, acc[0], acc[1], acc[2], acc[3]);
+  VT::store4(dst + 8, acc[4], acc[5], acc[6], acc[7]);
+  if (cc == 0) p.lse[row] = denom > 0.f ? (m + __builtin_amdgcn_logf(denom)) * 0.6931471805599453f : -INFINITY;
+}
+
+}  // namespace
+
+int fdb_launch_merge(const FdbKParams& p, int dtype, void* stream) {
+  const int64_t chunks = p.ws_rows * p.H * 8;
+  const unsigned blocks = (unsigned)((chunks + 255) / 256);
+  if (dtype == FDB_BF16)
+    hipLaunchKernelGGL(fdb_merge_kernel<fdb::Bf16Tr>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, p);
+  else if (dtype == FDB_F16)
+    hipLaunchKernelGGL(fdb_merge_kernel<fdb::F16Tr>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, p);
+  else
+    return FDB_ERR_UNSUPPORTED;
   return (int)hipGetLastError();
 }
 

@@ -35,20 +35,30 @@ struct FdbKParams {
   int32_t R;        // LUT radius
   int32_t far_done;  // near launches: the far tiles' partial results (far_parts of them) are to be merged
   int32_t far_parts; // workgroups per query tile of the far-only launch, each with its share of the far tiles and a
-                     // partial result of its own (the first in out / lse)
-  char* ws;          // partial results 1 .. far_parts-1: [far_parts-1][ws_rows][H][D] elements of v's type,
-  int64_t ws_rows;   // then [far_parts-1][ws_rows][H] float log-sum-exps; ws_rows = rows of the lse buffer
+                     // partial result of its own (the first in out / lse, the others in workspace slots 0 ..)
+  int32_t near_parts; // workgroups per query tile of the near launch; above 1 each leaves the partial result of
+                      // its share of the steps in workspace slot far_parts-1 + part, and fdb_launch_merge follows
+  int32_t ws_slots;  // partial results in the workspace: far_parts-1, plus near_parts if that is above 1
+  char* ws;          // [ws_slots][ws_rows][H][D] elements of v's type (rows normalised over the keys seen), then
+  int64_t ws_rows;   // [ws_slots][ws_rows][H] float log-sum-exps (-inf: no key seen); ws_rows = rows of the lse buffer
   int32_t causal;
   float scale_log2; // sm_scale * log2(e)
 };
 
-// Where far partial result `part` >= 1 lives in the workspace (row_bytes = head_dim * element size).
+// Workspace slot `slot`: its output rows and its log-sum-exps (row_bytes = head_dim * element size).
 #if defined(__HIPCC__)
+__device__ __forceinline__ char* ws_slot_out(const FdbKParams& p, int slot, int row_bytes) {
+  return p.ws + (int64_t)slot * p.ws_rows * p.H * row_bytes;
+}
+__device__ __forceinline__ float* ws_slot_lse(const FdbKParams& p, int slot, int row_bytes) {
+  return (float*)(p.ws + (int64_t)p.ws_slots * p.ws_rows * p.H * row_bytes) + (int64_t)slot * p.ws_rows * p.H;
+}
+// far partial result `part` >= 1 sits in slot part - 1
 __device__ __forceinline__ char* far_part_out(const FdbKParams& p, int part, int row_bytes) {
-  return p.ws + (int64_t)(part - 1) * p.ws_rows * p.H * row_bytes;
+  return ws_slot_out(p, part - 1, row_bytes);
 }
 __device__ __forceinline__ float* far_part_lse(const FdbKParams& p, int part, int row_bytes) {
-  return (float*)(p.ws + (int64_t)(p.far_parts - 1) * p.ws_rows * p.H * row_bytes) + (int64_t)(part - 1) * p.ws_rows * p.H;
+  return ws_slot_lse(p, part - 1, row_bytes);
 }
 #endif
 
@@ -71,6 +81,9 @@ bool fdb_near_supported(int dtype, int head_dim);
 // (16-bit element types, head_dim 64); merges the far partial like the ring mode.
 bool fdb_near32_supported(int dtype, int head_dim);
 int fdb_launch_near32(const FdbKParams& p, int dtype, int grid_x, void* stream);
+// fdb_launch_merge: after a near launch with near_parts > 1: out / lse from the far partial results (when
+// p.far_done) and the near ones (16-bit element types, head_dim 64).
+int fdb_launch_merge(const FdbKParams& p, int dtype, void* stream);
 int fdb_launch_worklist(const int32_t* cu, int32_t batch, int32_t* wl, int32_t max_tiles, void* stream);
 int fdb_launch_quant(const void* x, int64_t x_st, int64_t x_sh, void* y, int64_t y_st, int64_t y_sh,
                      float* scale, uint32_t* absmax_ws, int32_t tokens, int32_t heads, int32_t head_dim,

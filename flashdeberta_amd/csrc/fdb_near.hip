@@ -123,8 +123,13 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
   const int lim = m0 - (FDB_BN - 1) - p.R;
   const int t0 = lim >= 0 ? min(n_tiles, lim / FDB_BN + 1) : 0;
   const int t1 = max(t0, min(n_tiles, (m0 + FDB_BM - 1 + p.R + FDB_BN - 1) / FDB_BN));
-  const int s0 = 2 * t0;                                                   // first 32-key step
-  const int s1 = max(s0, min(2 * t1, (j_end + kStep - 1) / kStep));        // one past the last
+  int s0 = 2 * t0;                                                         // first 32-key step
+  int s1 = max(s0, min(2 * t1, (j_end + kStep - 1) / kStep));              // one past the last
+  if (p.near_parts > 1) {  // this workgroup's share of the steps
+    const int all = s1 - s0, part = (int)blockIdx.y;
+    s1 = s0 + (int)((int64_t)all * (part + 1) / p.near_parts);
+    s0 = s0 + (int)((int64_t)all * part / p.near_parts);
+  }
   const int n_steps = s1 - s0;
   const int n_full = p.causal ? 0 : max(0, min(n_steps, Lb / kStep - s0));  // steps k < n_full need no mask
 
@@ -424,6 +429,22 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
   if (i < Lb) {
     char* orow = ob + (int64_t)i * p.o_st * 2;
     const int64_t tok = p.cu ? (int64_t)tok0 + i : (int64_t)b * p.L + tok0 + i;
+    if (p.near_parts > 1) {
+      // a share of the steps: the partial result goes to its workspace slot, fdb_merge_kernel does the rest
+      const int slot = p.far_parts - 1 + (int)blockIdx.y;
+      char* dst = ws_slot_out(p, slot, D * 2) + (tok * p.H + h) * (D * 2);
+      const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+#pragma unroll
+      for (int d = 0; d < DBLKS; ++d)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4)
+          VT::store4(dst + (32 * d + 8 * q4 + 4 * g) * 2, o_acc[d][4 * q4] * inv, o_acc[d][4 * q4 + 1] * inv,
+                     o_acc[d][4 * q4 + 2] * inv, o_acc[d][4 * q4 + 3] * inv);
+      if (g == 0)
+        ws_slot_lse(p, slot, D * 2)[tok * p.H + h] =
+            l_tot > 0.f ? (m_run + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f : -INFINITY;
+      return;
+    }
     // far partial results: part 0 in out / lse, the others in the workspace (rows normalised over their
     // keys, log-sum-exp -inf where a row had none)
     const int n_far = p.far_done ? p.far_parts : 0;
@@ -480,7 +501,8 @@ int launch_near_one(const FdbKParams& p, int grid_x, hipStream_t stream) {
   static_assert(lds <= 80 * 1024, "two workgroups per CU");
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
   if (e != hipSuccess) return (int)e;
-  hipLaunchKernelGGL(kern, dim3((unsigned)grid_x * p.H, 1, 1), dim3(kNThreads), lds, stream, p);
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid_x * p.H, p.near_parts > 1 ? (unsigned)p.near_parts : 1u, 1), dim3(kNThreads),
+                     lds, stream, p);
   return (int)hipGetLastError();
 }
 

@@ -111,6 +111,7 @@ typedef struct fdb_attn_args {
   int32_t dtype;           /* enum fdb_dtype                                                 */
   int32_t causal;          /* nonzero: key j visible to query i only if j <= i               */
   int32_t far_splits;      /* 0: the library decides; 1 .. FDB_MAX_FAR_SPLITS: workgroups that share the far keys of a query tile */
+  int32_t near_splits;     /* the same for the near keys (those whose bucketed relative position varies)                  */
   float sm_scale;
 } fdb_attn_args;
 
@@ -129,13 +130,15 @@ int fdb_attn_fwd(const fdb_attn_args* a, void* stream);
 
 /*
  * Bytes of workspace the call would use (0: none), for the device that is current.  A launch whose
- * query tiles fill at most half of the workgroups the GPU holds shares the far keys of each query tile (those
- * whose bucketed relative position is constant) among up to FDB_MAX_FAR_SPLITS workgroups, whose partial results go
- * through the workspace: (splits - 1) * rows * heads * (head_dim * sizeof(v element) + 4) bytes, rows being
- * the rows of the lse buffer.  The workspace is optional: without it (or with a smaller one) the call
- * uses as many splits as fit, down to one, with the same result up to rounding.  far_splits and the
- * workspace fields of `a` are read (far_splits) and ignored (workspace, workspace_bytes) here.  No
- * counterpart in the reference, whose kernels have one program per query tile (flash_attention.py:465-488).
+ * query tiles fill at most half of the workgroups the GPU holds shares the keys of each query tile among up
+ * to FDB_MAX_FAR_SPLITS workgroups, separately for the far keys (those whose bucketed relative position is
+ * constant; launch of their own) and the near keys; the partial results go through the workspace, one slot of
+ * rows * heads * (head_dim * sizeof(v element) + 4) bytes each (rows: those of the lse buffer): far_splits - 1
+ * slots, plus near_splits slots if near_splits > 1 (a small merge kernel then follows the two launches).
+ * The workspace is optional: without it (or with a smaller one) the call first gives up the near splits,
+ * then uses as many far splits as fit, down to one, with the same result up to rounding.  far_splits and
+ * near_splits of `a` are read, its workspace fields ignored here.  No counterpart in the reference, whose
+ * kernels have one program per query tile (flash_attention.py:465-488).
  */
 int64_t fdb_attn_workspace_bytes(const fdb_attn_args* a);
 

@@ -128,20 +128,28 @@ def test_far_split_policy_and_workspace_size():
         a.batch, a.heads, a.max_seqlen, a.total_tokens, a.lse = batch, heads, seqlen, batch * seqlen, lse
         return a
 
-    assert ws(args(1, 4096)) == part(4096, 12)            # 384 query tiles -> 2 x 384 = one full round
+    # far launch: 3 workgroups per CU = 768 slots; near launch: 2 per CU = 512 slots
+    assert ws(args(1, 4096)) == part(4096, 12)            # 384 query tiles: 2 far shares (1 slot), near unshared
     assert ws(args(1, 4096, heads=16)) == 0               # 512: two shares would need a second round
-    assert ws(args(1, 4096, heads=8)) == 2 * part(4096, 8)  # 256 -> 3 x 256
+    assert ws(args(1, 4096, heads=8)) == (2 + 2) * part(4096, 8)  # 256: 3 far shares (2 slots) + 2 near shares (2 slots)
     assert ws(args(2, 4096)) == 0 and ws(args(8, 4096)) == 0  # the launch fills the slots by itself
-    assert ws(args(1, 2048)) == 0                         # too few far tiles to share out
-    assert ws(args(8, 512)) == 0                          # no far tile at all
+    assert ws(args(1, 2048)) == 2 * part(2048, 12)        # 192: too few far tiles to share, 2 near shares
+    assert ws(args(1, 1024)) == 2 * part(1024, 12)        # 96: 32 steps in two shares of sixteen
+    assert ws(args(1, 512)) == 2 * part(512, 12)          # 48, no far tile at all: shares of eight steps, 96 workgroups
+    assert ws(args(2, 512)) == 2 * part(2 * 512, 12)      # 96 -> 192
+    assert ws(args(4, 512)) == 0                          # 192 -> 384: more than half of the slots in shares of eight
+    assert ws(args(8, 512)) == 0
     assert ws(args(1, 4096, lse=None)) == 0               # one fused kernel without the lse buffer
     a = args(8, 4096); a.far_splits = 4; assert ws(a) == 3 * part(8 * 4096, 12)
+    a = args(8, 4096); a.near_splits = 3; assert ws(a) == 3 * part(8 * 4096, 12)
     a = args(1, 4096); a.far_splits = 1; assert ws(a) == 0
-    a = args(1, 4096); a.dtype = _lib.FDB_F32; a.far_splits = 3; assert ws(a) == 0   # fp32 takes the fused kernel
+    a = args(1, 2048); a.near_splits = 1; assert ws(a) == 0
+    a = args(1, 4096); a.dtype = _lib.FDB_F32; a.far_splits = a.near_splits = 3; assert ws(a) == 0   # fp32 takes the fused kernel
     a = args(1, 4096); a.cu_seqlens, a.worklist = 0x6000, 0x7000; assert ws(a) == 0   # lengths unknown to the host
     a.far_splits = 2; assert ws(a) == part(4096, 12)
     a = args(1, 4096); a.far_splits = 5; assert chk(a) == -5 and ws(a) == 0
     a = args(1, 4096); a.far_splits = -1; assert chk(a) == -5
+    a = args(1, 4096); a.near_splits = 5; assert chk(a) == -5
     a = args(1, 4096); a.workspace, a.workspace_bytes = 0x8008, 1 << 20; assert chk(a) == -4
     a = args(1, 4096); a.workspace, a.workspace_bytes = 0x8000, -1; assert chk(a) == -5
 

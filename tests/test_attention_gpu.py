@@ -170,6 +170,29 @@ def test_far_keys_shared_among_workgroups(splits, L, pb, mr, causal, c2p, p2c, d
     assert (out.float() - one.float()).abs().max().item() <= TOL[dtype]
 
 
+@pytest.mark.parametrize("far,near", [(1, 2), (1, 3), (1, 4), (2, 2), (4, 3), (3, 4)])
+@pytest.mark.parametrize("L,pb,mr,causal,c2p,p2c,dtype", [
+    (1500, 256, 512, False, True, True, torch.bfloat16),   # far tiles on both sides, forty near steps
+    (300, 256, 512, False, True, True, torch.float16),     # no far launch at all; ten steps: shares of two or three
+    (900, 32, 64, True, True, True, torch.bfloat16),       # causal, ragged last step
+    (1100, 16, 32, False, False, True, torch.bfloat16),    # one position term
+    (45, 32, 64, False, True, False, torch.bfloat16),      # two steps: some shares are empty
+])
+def test_near_steps_shared_among_workgroups(far, near, L, pb, mr, causal, c2p, p2c, dtype):
+    """The near launch with several workgroups per query tile, each leaving the partial result of its share
+    of the steps in the workspace, and the merge kernel that combines them with the far ones: same result
+    as unshared, and both match the oracle (output and log-sum-exp)."""
+    q, k, v, pk, pq = _inputs(2, L, 2, 64, pb, mr, dtype, 700 + L + 10 * far + near, 1.0, c2p, p2c)
+    ref, ref_lse = _oracle_blhd(q, k, v, pk, pq, pb, mr, causal=causal, return_lse=True)
+    args = [_dev(x) for x in (q, k, v, pk, pq)]
+    kw = dict(position_buckets=pb, max_relative_positions=mr, causal=causal, return_lse=True)
+    out, lse = ops.disentangled_attention_fwd(*args, far_splits=far, near_splits=near, **kw)
+    one, _ = ops.disentangled_attention_fwd(*args, far_splits=1, near_splits=1, **kw)
+    _check(out, ref, TOL[dtype], "out")
+    _check(lse.view(2, L, 2), ref_lse, 4 * TOL[dtype], "lse")
+    assert (out.float() - one.float()).abs().max().item() <= TOL[dtype]
+
+
 def test_far_keys_shared_packed_and_padded():
     """Shared far keys with packed sequences (work-list launch) and with a padded batch."""
     pb, mr, H, D = 32, 64, 2, 64
@@ -178,13 +201,14 @@ def test_far_keys_shared_packed_and_padded():
     cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
     kw = dict(position_buckets=pb, max_relative_positions=mr)
     out = ops.disentangled_attention_fwd(_dev(q[0]), _dev(k[0]), _dev(v[0]), _dev(pk), _dev(pq), cu_seqlens=cu.cuda(),
-                                         max_seqlen=max(lens), far_splits=3, **kw)
+                                         max_seqlen=max(lens), far_splits=3, near_splits=2, **kw)
     Lmax = max(lens)
     pad = lambda x: torch.stack([torch.nn.functional.pad(x[0, cu[b]:cu[b + 1]], (0, 0, 0, 0, 0, Lmax - lens[b]))
                                  for b in range(len(lens))])
     padded = torch.zeros(len(lens), Lmax, H, D, dtype=torch.bfloat16, device="cuda")
     ops.disentangled_attention_fwd(_dev(pad(q)), _dev(pad(k)), _dev(pad(v)), _dev(pk), _dev(pq), out=padded,
-                                   seq_len=torch.tensor(lens, dtype=torch.int32).cuda(), far_splits=4, **kw)
+                                   seq_len=torch.tensor(lens, dtype=torch.int32).cuda(), far_splits=4, near_splits=3, **kw)
+    assert (padded[1, lens[1]:] == 0).all() and (padded[2, 1:] == 0).all()  # the merge leaves padded rows alone
     off = 0
     for b, n in enumerate(lens):
         sl = slice(off, off + n)
@@ -194,13 +218,13 @@ def test_far_keys_shared_packed_and_padded():
         off += n
 
 
-@pytest.mark.parametrize("B,L,splits", [(2, 700, 0), (1, 1500, 2)])
-def test_operator_replays_from_a_hip_graph(B, L, splits):
+@pytest.mark.parametrize("B,L,splits,near", [(2, 700, 0, 1), (1, 1500, 2, 0), (1, 1500, 2, 3)])
+def test_operator_replays_from_a_hip_graph(B, L, splits, near):
     """The operator enqueues only kernels on the current stream and allocates through torch, so it can be
     captured into a HIP graph: three replays on fresh input values, with eager calls and synchronisations
     in between, each equal to the eager result on the same values."""
     pb, mr, H, D = 32, 64, 2, 64
-    kw = dict(position_buckets=pb, max_relative_positions=mr, far_splits=splits)
+    kw = dict(position_buckets=pb, max_relative_positions=mr, far_splits=splits, near_splits=near)
     q, k, v, pk, pq = [_dev(x) for x in _inputs(B, L, H, D, pb, mr, torch.bfloat16, 900, 1.0)]
     ops.disentangled_attention_fwd(q, k, v, pk, pq, **kw)  # the delta table reaches the device outside the capture
     torch.cuda.synchronize()
