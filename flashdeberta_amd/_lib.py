@@ -12,6 +12,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libfdb_hip.so")
 
 FDB_F32, FDB_BF16, FDB_F16, FDB_FP8_E4M3 = 0, 1, 2, 3
+FDB_VERSION = 3  # of include/fdb.h as mirrored below
 
 
 class FdbAttnArgs(ctypes.Structure):
@@ -50,6 +51,9 @@ def _load():
     if lib.fdb_attn_args_size() != ctypes.sizeof(FdbAttnArgs):
         raise ImportError("flashdeberta_amd: %s was built from a different include/fdb.h (struct size %d, binding %d); rebuild it"
                           % (LIB_PATH, lib.fdb_attn_args_size(), ctypes.sizeof(FdbAttnArgs)))
+    if lib.fdb_version() != FDB_VERSION:  # the struct can change its layout and keep its size
+        raise ImportError("flashdeberta_amd: %s is version %d of the C ABI, this binding is version %d; rebuild it"
+                          % (LIB_PATH, lib.fdb_version(), FDB_VERSION))
     lib.fdb_strerror.restype = ctypes.c_char_p
     lib.fdb_strerror.argtypes = [ctypes.c_int]
     lib.fdb_attn_check.restype = ctypes.c_int

@@ -34,7 +34,8 @@
 extern "C" {
 #endif
 
-#define FDB_VERSION 2
+/* bumped whenever fdb_attn_args or the meaning of an entry point changes: a binding checks it next to the struct size */
+#define FDB_VERSION 3
 
 /* element types of q/k/pos_key/pos_query (v and out: see fdb_attn_args.dtype) */
 enum fdb_dtype {
