@@ -457,6 +457,28 @@ def test_fp8_attention(L, pb, mr, single):
     _check(out, ref_dq, TOL[torch.bfloat16], "unit scale vs de-quantised oracle")
 
 
+def test_fp8_full_length_one_head():
+    """The FP8 Q/K configuration at its full sequence length (8192, position_buckets 256) on one head, so
+    that the oracle finishes in seconds: 108 far tiles and 40 near steps per query tile, 64 query tiles, i.e.
+    a launch small enough that the far and the near keys are shared out and the merge kernel runs."""
+    L, H, D, pb, mr = 8192, 1, 64, 256, 512
+    g = torch.Generator().manual_seed(23)
+    q, k, v, pk, pq = _inputs(1, L, H, D, pb, mr, torch.bfloat16, 24, 0.02)
+    q, k = _outliers(q.float(), g).to(torch.bfloat16), _outliers(k.float(), g).to(torch.bfloat16)
+    q8, qs = ops.quantize_e4m3_per_head(q.cuda())
+    k8, ks = ops.quantize_e4m3_per_head(k.cuda())
+    pk8, pks = ops.quantize_e4m3_per_head(pk.cuda().transpose(0, 1))
+    pq8, pqs = ops.quantize_e4m3_per_head(pq.cuda().transpose(0, 1))
+    out = ops.disentangled_attention_fwd(q8, k8, v.cuda(), pk8.transpose(0, 1), pq8.transpose(0, 1), position_buckets=pb,
+                                         max_relative_positions=mr, q_scale=qs, k_scale=ks, pos_key_scale=pks,
+                                         pos_query_scale=pqs)
+    dq = lambda y, s: y.float().cpu() * s.cpu()[:, None]
+    ref_dq = _oracle_blhd(dq(q8, qs), dq(k8, ks), v, dq(pk8, pks).transpose(0, 1), dq(pq8, pqs).transpose(0, 1), pb, mr)
+    err = np.abs(out.float().cpu().numpy() - ref_dq).max()
+    assert err <= 1e-3, err  # outputs are averages of 0.02-scale values: an absolute bound that means something here
+    _check(out, ref_dq, TOL[torch.bfloat16], "vs de-quantised oracle")
+
+
 # ---- module: golden vectors and the live eager class ---------------------------------------------------
 def _module_from_golden(g, dtype=torch.float32):
     from flashdeberta_amd import FlashDisentangledSelfAttention
