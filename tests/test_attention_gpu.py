@@ -347,6 +347,31 @@ def test_varlen_matches_per_sequence_oracle(dtype):
     assert torch.equal(out3, out[torch.from_numpy(perm).cuda()])
 
 
+def test_varlen_full_size_matches_dense_calls():
+    """The packed-batch configuration at full size (64 sequences, lengths log-uniform in [32, 2048], 12 heads):
+    every sequence's rows of the packed result equal a fixed-layout call on that sequence alone, and two
+    heads of the longest and of the shortest sequence match the oracle."""
+    H, D, pb, mr = 12, 64, 256, 512
+    g = torch.Generator().manual_seed(1004)
+    lens = torch.exp(torch.empty(64).uniform_(np.log(32.0), np.log(2048.0), generator=g)).round().int().tolist()
+    T = sum(lens)
+    q, k, v, pk, pq = _inputs(1, T, H, D, pb, mr, torch.bfloat16, 1005, 1.0)
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+    kw = dict(position_buckets=pb, max_relative_positions=mr)
+    dq, dk, dv, dpk, dpq = [_dev(x) for x in (q, k, v, pk, pq)]
+    out = ops.disentangled_attention_fwd(dq[0], dk[0], dv[0], dpk, dpq, cu_seqlens=cu.cuda(), max_seqlen=max(lens), **kw)
+    worst = 0.0
+    for b, n in enumerate(lens):
+        sl = slice(int(cu[b]), int(cu[b + 1]))
+        alone = ops.disentangled_attention_fwd(dq[:, sl], dk[:, sl], dv[:, sl], dpk, dpq, **kw)
+        worst = max(worst, (out[sl].float() - alone[0].float()).abs().max().item())
+    assert worst <= TOL[torch.bfloat16], worst
+    for b in (int(np.argmax(lens)), int(np.argmin(lens))):
+        sl = slice(int(cu[b]), int(cu[b + 1]))
+        ref = _oracle_blhd(q[:, sl, :2], k[:, sl, :2], v[:, sl, :2], pk[:2], pq[:2], pb, mr)
+        _check(out[sl][None, :, :2], ref, TOL[torch.bfloat16], "sequence %d of %d tokens" % (b, lens[b]))
+
+
 def test_worklist_on_device():
     from flashdeberta_amd._lib import lib
     import ctypes
