@@ -590,6 +590,38 @@ def test_patched_encoder_matches_eager_encoder():
     assert err < 0.1, err  # two bf16 encoder layers; hidden states are O(1) after LayerNorm
 
 
+def test_full_v3_base_encoder_bf16_against_fp32_eager():
+    """The full-encoder configuration (DeBERTa-v3-base: 12 layers, hidden 768, vocabulary 128100, random weights
+    N(0, 0.02), batch 8 x 512, all-ones mask): the patched bf16 model is as close to the fp32 eager model as the
+    bf16 eager model is."""
+    import copy
+
+    from transformers.models.deberta_v2.modeling_deberta_v2 import DebertaV2Config, DebertaV2Model
+
+    from flashdeberta_amd import patch_model
+
+    torch.manual_seed(1002)
+    cfg = DebertaV2Config(vocab_size=128100, hidden_size=768, num_hidden_layers=12, num_attention_heads=12,
+                          intermediate_size=3072, relative_attention=True, pos_att_type="p2c|c2p", position_buckets=256,
+                          share_att_key=True, norm_rel_ebd="layer_norm", position_biased_input=False,
+                          max_position_embeddings=512, hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0,
+                          initializer_range=0.02)
+    fp32 = DebertaV2Model(cfg).eval().cuda()
+    bf16 = copy.deepcopy(fp32).to(torch.bfloat16)
+    ids = torch.randint(0, 128100, (8, 512), device="cuda")
+    mask = torch.ones(8, 512, dtype=torch.long, device="cuda")
+    with torch.no_grad():
+        ref = fp32(input_ids=ids, attention_mask=mask).last_hidden_state
+        eager = bf16(input_ids=ids, attention_mask=mask).last_hidden_state.float()
+        patch_model(bf16)
+        ours = bf16(input_ids=ids, attention_mask=mask).last_hidden_state.float()
+    err_eager, err_ours = (eager - ref).abs().max().item(), (ours - ref).abs().max().item()
+    assert not torch.isnan(ours).any()
+    assert err_ours <= 1.5 * err_eager + 0.02, (err_ours, err_eager)
+    rms = lambda x: x.pow(2).mean().sqrt().item()
+    assert rms(ours - ref) <= 1.5 * rms(eager - ref) + 1e-3, (rms(ours - ref), rms(eager - ref))
+
+
 # ---- full-size properties (metric shape: v3-base heads, seq 4096, bf16) ----------------------------------
 def test_full_size_properties():
     B, L, H, D, pb, mr = 1, 4096, 12, 64, 256, 512
