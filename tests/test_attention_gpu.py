@@ -567,6 +567,37 @@ def test_module_matches_live_eager(dtype, share):
     _check(out, ref, 2e-4 if dtype == torch.float32 else 3e-2)
 
 
+def test_cpu_runnable_configuration_fp32():
+    """The reference's own CPU-runnable case at its size: one v3-base attention layer, batch 1, 512 tokens,
+    12 heads x 64, hidden 768, fp32; inputs, weights and the (layer-normed) relative embeddings N(0, 0.02),
+    share_att_key, c2p|p2c, 256 buckets, no mask; against the eager class on the host."""
+    from transformers.models.deberta_v2.modeling_deberta_v2 import DisentangledSelfAttention
+
+    from flashdeberta_amd import FlashDisentangledSelfAttention
+
+    class Cfg:
+        hidden_size, num_attention_heads = 768, 12
+        attention_probs_dropout_prob = hidden_dropout_prob = 0.1
+        pos_att_type = ["c2p", "p2c"]
+        relative_attention, position_buckets, max_relative_positions = True, 256, 512
+        max_position_embeddings, share_att_key = 512, True
+
+    torch.manual_seed(1001)
+    eager = DisentangledSelfAttention(Cfg()).eval()
+    with torch.no_grad():
+        for prm in eager.parameters():
+            prm.normal_(0.0, 0.02)
+    flash = FlashDisentangledSelfAttention(Cfg()).eval()
+    flash.load_state_dict(eager.state_dict())
+    hidden = torch.randn(1, 512, 768) * 0.02
+    rel = torch.nn.functional.layer_norm(torch.randn(512, 768) * 0.02, (768,), eps=1e-7)
+    with torch.no_grad():
+        ref = eager(hidden, torch.ones(1, 1, 512, 512), rel_embeddings=rel)[0].numpy()
+        out = flash.cuda()(hidden.cuda(), None, rel_embeddings=rel.cuda())[0]
+    err = np.abs(out.cpu().numpy() - ref).max()
+    assert err <= 1e-4 and err <= 2e-3 * np.abs(ref).max(), (err, np.abs(ref).max())
+
+
 def test_patched_encoder_matches_eager_encoder():
     from transformers.models.deberta_v2.modeling_deberta_v2 import DebertaV2Config, DebertaV2Model
 
