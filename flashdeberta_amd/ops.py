@@ -80,7 +80,7 @@ def _pos_arg(x, H, D, span, name):
 def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seqlens=None, max_seqlen=None,
                                sm_scale=None, position_buckets=0, max_relative_positions=0, causal=False,
                                return_lse=False, seq_start=None, seq_len=None, q_scale=None, k_scale=None, pos_key_scale=None,
-                               pos_query_scale=None, out=None, single_kernel=False, far_splits=0, near_splits=0):
+                               pos_query_scale=None, out=None, single_kernel=False, far_splits=0, near_splits=0, workspace=None):
     """Fused forward.  Layouts (strides are free except a unit stride on D):
          fixed length : q, k, v  [B, L, H, D]   -> out [B, L, H, D] (contiguous: a free view of [B, L, H*D])
          packed varlen: q, k, v  [T, H, D] + cu_seqlens int32 [B+1] (+ max_seqlen upper bound) -> out [T, H, D]
@@ -94,6 +94,9 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
        one kernel instead of the far-tile / near-tile pair of launches (same result; for comparison).
        far_splits, near_splits: workgroups that share the far / the near keys of a query tile (0: the library
        decides from the size of the launch; it matters for launches that do not fill the GPU, e.g. one sequence).
+       workspace: a uint8 GPU tensor for the partial results of such shared launches, to reuse one buffer across
+       calls; by default one of the size the library asks for is allocated per call.  A smaller one is fine: the
+       library then shares less.
     """
     if not q.is_cuda:
         raise RuntimeError("disentangled_attention_fwd runs on the GPU only; got device %s" % q.device)
@@ -133,7 +136,8 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
                 None if pos_query is None else deq(pos_query.transpose(0, 1), pos_query_scale).transpose(0, 1),
                 cu_seqlens=cu_seqlens, max_seqlen=max_seqlen, sm_scale=sm_scale, position_buckets=position_buckets,
                 max_relative_positions=max_relative_positions, causal=causal, return_lse=return_lse,
-                seq_start=seq_start, seq_len=seq_len, out=out, far_splits=far_splits, near_splits=near_splits)
+                seq_start=seq_start, seq_len=seq_len, out=out, far_splits=far_splits, near_splits=near_splits,
+                workspace=workspace)
         dt = _lib.FDB_FP8_E4M3
     else:
         if q.dtype not in _DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
@@ -204,11 +208,17 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
     a.dtype, a.causal, a.sm_scale, a.far_splits = dt, int(bool(causal)), float(sm_scale), int(far_splits)
     a.near_splits = int(near_splits)
     with torch.cuda.device(q.device):
-        ws_bytes = lib.fdb_attn_workspace_bytes(ctypes.byref(a))
-        if ws_bytes > 0:
-            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
-            keep.append(ws)
-            a.workspace, a.workspace_bytes = ws.data_ptr(), ws_bytes
+        if workspace is not None:
+            if workspace.dtype != torch.uint8 or not workspace.is_cuda or not workspace.is_contiguous():
+                raise ValueError("workspace must be a contiguous uint8 GPU tensor")
+            if workspace.numel() > 0:
+                a.workspace, a.workspace_bytes = workspace.data_ptr(), workspace.numel()
+        else:
+            ws_bytes = lib.fdb_attn_workspace_bytes(ctypes.byref(a))
+            if ws_bytes > 0:
+                ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+                keep.append(ws)
+                a.workspace, a.workspace_bytes = ws.data_ptr(), ws_bytes
         check(lib.fdb_attn_fwd(ctypes.byref(a), _stream_ptr(q.device)), "fdb_attn_fwd")
     return (out, lse) if return_lse else out
 

@@ -193,6 +193,26 @@ def test_near_steps_shared_among_workgroups(far, near, L, pb, mr, causal, c2p, p
     assert (out.float() - one.float()).abs().max().item() <= TOL[dtype]
 
 
+@pytest.mark.parametrize("slots", [0, 1, 2, 4, 5])
+def test_caller_owned_workspace_of_any_size(slots):
+    """A caller-owned workspace smaller than what three far and three near shares need (five slots): the
+    library shares less, writes nothing outside the bytes it was given, and the result does not change."""
+    L, H, D, pb, mr = 1500, 2, 64, 256, 512
+    q, k, v, pk, pq = _inputs(1, L, H, D, pb, mr, torch.bfloat16, 800, 1.0)
+    args = [_dev(x) for x in (q, k, v, pk, pq)]
+    kw = dict(position_buckets=pb, max_relative_positions=mr, far_splits=3, near_splits=3)
+    slot = L * H * (D * 2 + 4)
+    guard = 4096
+    buf = torch.full((guard + slots * slot + guard,), 0xA5, dtype=torch.uint8, device="cuda")
+    out = ops.disentangled_attention_fwd(*args, workspace=buf[guard:guard + slots * slot], **kw)
+    torch.cuda.synchronize()
+    assert (buf[:guard] == 0xA5).all() and (buf[guard + slots * slot:] == 0xA5).all()
+    _check(out, _oracle_blhd(q, k, v, pk, pq, pb, mr), TOL[torch.bfloat16])
+    if slots < 5:  # the near shares were given up: no merge kernel, the last slots stay untouched
+        used = min(slots, 2) * slot
+        assert (buf[guard + used:guard + slots * slot] == 0xA5).all()
+
+
 def test_far_keys_shared_packed_and_padded():
     """Shared far keys with packed sequences (work-list launch) and with a padded batch."""
     pb, mr, H, D = 32, 64, 2, 64
