@@ -119,7 +119,9 @@ int far_parts_wanted(const fdb_attn_args* a) {
 // (five batches of table rows) and a merge kernel follows, so a share keeps at least sixteen 32-key
 // steps, or eight when all shares together fill at most half of the slots.  (Measured, 12 heads: one
 // sequence of 1024: 0.056 -> 0.040 ms; one of 512: 0.025 -> 0.022; four of 512 in shares of eight
-// steps would go from 0.025 to 0.028.)
+// steps would go from 0.025 to 0.028.)  Two shares also pay when they need a partial second round, as
+// long as the query tiles alone fill at most 70 % of the slots (288 to 352 tiles: 5 to 8 % of the call;
+// 384: between +2 and -4 %).
 int near_parts_wanted(const fdb_attn_args* a) {
   if (!(a->pos_key || a->pos_query) || !a->lse || !fdb_near32_supported(a->dtype, a->head_dim)) return 1;
   if (a->near_splits > 0) return a->near_splits;
@@ -128,7 +130,7 @@ int near_parts_wanted(const fdb_attn_args* a) {
   const int steps_all = (a->max_seqlen + 31) / 32, steps_near = (FDB_BM + 2 * a->lut_radius + 3 * (FDB_BN - 1)) / 32;
   const int steps = steps_all < steps_near ? steps_all : steps_near;
   int best = 1;
-  for (int n = 2; n <= FDB_MAX_FAR_PARTS && wgs * n <= slots; ++n) {
+  for (int n = 2; n <= FDB_MAX_FAR_PARTS && (wgs * n <= slots || (n == 2 && wgs * 10 <= slots * 7)); ++n) {
     const int per = steps / n;
     if (per >= 16 || (per >= 8 && wgs * n <= slots / 2)) best = n;
   }

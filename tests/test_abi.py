@@ -131,6 +131,7 @@ def test_far_split_policy_and_workspace_size():
     # far launch: 3 workgroups per CU = 768 slots; near launch: 2 per CU = 512 slots
     assert ws(args(1, 4096)) == part(4096, 12)            # 384 query tiles: 2 far shares (1 slot), near unshared
     assert ws(args(1, 4096, heads=16)) == 0               # 512: two shares would need a second round
+    assert ws(args(1, 4096, heads=10)) == (1 + 2) * part(4096, 10)  # 320: 2 far shares; 2 near shares in 1.25 rounds
     assert ws(args(1, 4096, heads=8)) == (2 + 2) * part(4096, 8)  # 256: 3 far shares (2 slots) + 2 near shares (2 slots)
     assert ws(args(2, 4096)) == 0 and ws(args(8, 4096)) == 0  # the launch fills the slots by itself
     assert ws(args(1, 2048)) == 2 * part(2048, 12)        # 192: too few far tiles to share, 2 near shares
