@@ -432,6 +432,29 @@ def test_padded_batch_matches_packed(side):
         assert (out[b, rest.cuda()] == 0).all()
 
 
+@pytest.mark.parametrize("near", [1, 2])
+def test_empty_rows_and_empty_sequences(near):
+    """A padded batch with a row of no real tokens and a packed batch with an empty sequence in the middle:
+    nothing is written for them, the other sequences are unaffected (also through the merge kernel)."""
+    pb, mr, H, D = 32, 64, 2, 64
+    lens = [300, 0, 77]
+    q, k, v, pk, pq = _inputs(3, 300, H, D, pb, mr, torch.bfloat16, 41, 1.0)
+    kw = dict(position_buckets=pb, max_relative_positions=mr, near_splits=near)
+    out = torch.full((3, 300, H, D), 7.0, dtype=torch.bfloat16, device="cuda")
+    ops.disentangled_attention_fwd(_dev(q), _dev(k), _dev(v), _dev(pk), _dev(pq), out=out,
+                                   seq_len=torch.tensor(lens, dtype=torch.int32).cuda(), **kw)
+    assert (out[1] == 7).all() and (out[2, 77:] == 7).all()
+    cu = torch.tensor([0, 300, 300, 377], dtype=torch.int32)
+    packed = torch.cat([q[0], q[2, :77]]), torch.cat([k[0], k[2, :77]]), torch.cat([v[0], v[2, :77]])
+    outp = ops.disentangled_attention_fwd(*[_dev(x) for x in packed], _dev(pk), _dev(pq), cu_seqlens=cu.cuda(),
+                                          max_seqlen=300, **kw)
+    for b, sl in ((0, slice(0, 300)), (2, slice(300, 377))):
+        n = lens[b]
+        ref = _oracle_blhd(q[b:b + 1, :n], k[b:b + 1, :n], v[b:b + 1, :n], pk, pq, pb, mr)
+        _check(out[b:b + 1, :n], ref, TOL[torch.bfloat16], "padded row %d" % b)
+        _check(outp[sl][None], ref, TOL[torch.bfloat16], "packed sequence %d" % b)
+
+
 # ---- fp8 Q/K ---------------------------------------------------------------------------------------
 def _outliers(x, g):
     m = torch.rand(x.shape, generator=g) < 0.01
