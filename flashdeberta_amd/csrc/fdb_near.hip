@@ -366,37 +366,56 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
         if (j >= Lb || (p.causal && j > i)) sacc[v] = -INFINITY;
       }
     }
-    float mx = sacc[0];
+    // The probabilities are formed against the row's current reference point first; the half-row sum of a
+    // step bounds its largest one, so while it stays under 2^kLazyTau nothing has to move and no maximum is
+    // taken.  Otherwise (or before a row has a reference point) the wave takes the maximum, moves the
+    // reference points of the rows that need it and forms the probabilities again.
+    vfrag pf[2];
+    float l_blk = 0.f;
+    auto probs = [&](float off) __attribute__((always_inline)) {
+      l_blk = 0.f;
 #pragma unroll
-    for (int v = 1; v < 16; ++v) mx = fmaxf(mx, sacc[v]);
-    mx = wave_half_max(mx) * x_scale;  // x_scale > 0
-    if (__any(mx > m_run + kLazyTau)) {
-      const float m_new = (mx > m_run + kLazyTau) ? mx : m_run;
-      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // m_run = -inf before the first visible key: 0
-      l_run *= alpha;
-      m_run = m_new;
+      for (int c = 0; c < 2; ++c) {
+        f32x8 pv;
 #pragma unroll
-      for (int d = 0; d < DBLKS; ++d)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) o_acc[d][v] *= alpha;
+        for (int e = 0; e < 8; ++e)  // the V^T operand takes the keys in ascending order
+          pv[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[8 * c + (e ^ 3)], x_scale, off));
+        pf[c] = VT::from_f32(pv);
+        l_blk = VT::sum8(pf[c], l_blk);
+      }
+    };
+    bool slow = __any(m_run == -INFINITY);
+    if (!slow) {
+      probs(-m_run);
+      slow = __any(!(l_blk <= 256.f));  // 2^kLazyTau; also true for an overflow
     }
-    const float off = (MASK && m_run == -INFINITY) ? 0.f : -m_run;  // a row that has seen no visible key yet
+    if (slow) {
+      float mx = sacc[0];
 #pragma unroll
-    for (int c = 0; c < 2; ++c) {
-      f32x8 pv;
+      for (int v = 1; v < 16; ++v) mx = fmaxf(mx, sacc[v]);
+      mx = wave_half_max(mx) * x_scale;  // x_scale > 0
+      if (__any(mx > m_run + kLazyTau)) {
+        const float m_new = (mx > m_run + kLazyTau) ? mx : m_run;
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // m_run = -inf before the first visible key: 0
+        l_run *= alpha;
+        m_run = m_new;
 #pragma unroll
-      for (int e = 0; e < 8; ++e)  // the V^T operand takes the keys in ascending order
-        pv[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[8 * c + (e ^ 3)], x_scale, off));
-      const vfrag pf = VT::from_f32(pv);
-      l_run = VT::sum8(pf, l_run);
+        for (int d = 0; d < DBLKS; ++d)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) o_acc[d][v] *= alpha;
+      }
+      probs((MASK && m_run == -INFINITY) ? 0.f : -m_run);  // a row that has seen no visible key yet
+    }
+    l_run += l_blk;
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
 #pragma unroll
       for (int d = 0; d < DBLKS; ++d) {
         const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(Vs + vlx[2 * d] + 2048 * c));
         const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(Vs + vlx[2 * d + 1] + 2048 * c + 1024));
         const vfrag vf = __builtin_bit_cast(vfrag, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-        o_acc[d] = VT::mma(vf, pf, o_acc[d]);
+        o_acc[d] = VT::mma(vf, pf[c], o_acc[d]);
       }
-    }
     slot0 = slot0 + 32 >= kRingRows ? slot0 + 32 - kRingRows : slot0 + 32;
   };
   {
