@@ -90,10 +90,14 @@ int64_t query_tiles(const fdb_attn_args* a) {
 }
 
 // Does the call take the far / near pair of launches with a far launch in it?
+// A packed call's max_seqlen is the caller's word; the one bound the library can trust there is the
+// token count (no sequence is longer), so an under-estimate cannot make the far keys disappear: a far
+// launch that finds no far tile leaves "no far keys" (-inf) for every row and costs a few microseconds.
 bool has_far_launch(const fdb_attn_args* a) {
   const int32_t radius = a->lut_radius > 0 ? a->lut_radius : 1;
+  const int32_t longest = a->cu_seqlens ? a->total_tokens : a->max_seqlen;
   return (a->pos_key || a->pos_query) && a->lse && fdb_near_supported(a->dtype, a->head_dim) &&
-         a->max_seqlen > radius + FDB_BN - 1;
+         longest > radius + FDB_BN - 1;
 }
 
 // Workgroups per query tile of the far-only launch.  That launch keeps three workgroups on a CU; when
@@ -193,7 +197,6 @@ int fdb_attn_check(const fdb_attn_args* a) {
   if (qsz == 0) return FDB_ERR_DTYPE;
   const int vsz = v_elem_size(a->dtype);
   if (a->head_dim != 32 && a->head_dim != 64 && a->head_dim != 128) return FDB_ERR_HEAD_DIM;
-  if (a->dtype == FDB_F32 && a->head_dim == 128) return FDB_ERR_UNSUPPORTED;
   if (a->batch < 1 || a->heads < 1 || a->heads > 65535 || a->max_seqlen < 1 || a->total_tokens < 1)
     return FDB_ERR_SHAPE;
   if (a->far_splits < 0 || a->far_splits > FDB_MAX_FAR_SPLITS || a->near_splits < 0 ||

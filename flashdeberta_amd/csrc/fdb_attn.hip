@@ -66,8 +66,13 @@ struct Cfg {
   // three K/V buffers deep (see the kernel).
   static constexpr bool DMA_OK = QT::SZ == 2 && VT::SZ == 2 && D == 64;
   static constexpr int DMA_TILE = FDB_BN * 128, DMA_BUF = 2 * DMA_TILE, DMA_BYTES = 3 * DMA_BUF;
+  // fp32 at head_dim 128 with both position terms: K, V and the two bias scratches together exceed a
+  // CU's 160 KB, so V takes K's place in LDS once the tile's scores are done (kv_alias).
+  static constexpr bool kv_alias(bool c2p, bool p2c) {
+    return K_BYTES + V_BYTES + (c2p ? C2P_BYTES : 0) + (p2c ? P2C_BYTES : 0) > 160 * 1024;
+  }
   static constexpr int lds_bytes(bool c2p, bool p2c) {
-    return K_BYTES + V_BYTES + (c2p ? C2P_BYTES : 0) + (p2c ? P2C_BYTES : 0);
+    return K_BYTES + (kv_alias(c2p, p2c) ? 0 : V_BYTES) + (c2p ? C2P_BYTES : 0) + (p2c ? P2C_BYTES : 0);
   }
   static constexpr int lds_bytes_mode(int mode, bool c2p, bool p2c) {
     if (DMA_OK && (mode == 1 || (mode == 0 && !c2p && !p2c))) return DMA_BYTES;
@@ -307,9 +312,11 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
   constexpr bool FAR_ONLY = MODE == kFarOnly, RING = MODE == kNearRing;
   static_assert(!RING || (!FP8 && QT::SZ == 2 && (C2P || P2C)), "the ring mode is for the position terms of the 16-bit types");
   extern __shared__ __attribute__((aligned(16))) char smem[];
+  constexpr bool KV_ALIAS = C::kv_alias(C2P, P2C);
+  static_assert(!KV_ALIAS || MODE == kFused, "only the fused mode shares one buffer between K and V");
   char* Ks = smem;
-  char* Vs = Ks + C::K_BYTES;
-  ST* c2pS = (ST*)(Vs + C::V_BYTES);
+  char* Vs = KV_ALIAS ? Ks : Ks + C::K_BYTES;
+  ST* c2pS = (ST*)(Ks + C::K_BYTES + (KV_ALIAS ? 0 : C::V_BYTES));
   ST* p2cS = (ST*)((char*)c2pS + (C2P ? C::C2P_BYTES : 0));
   char* EK = (char*)p2cS + (P2C ? C::P2C_BYTES : 0);
   char* EQ = EK + (C2P ? C::RING_BYTES : 0);
@@ -489,6 +496,7 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
     }
   }
   auto dma_issue = [&](int tile, int bufoff) __attribute__((always_inline)) {
+    static_assert(kDmaLoadsPerTile == 2 * 2, "two 8-row groups of K and of V per wave and tile");
     const char* kt = kb + (uint64_t)(uint32_t)(tile * FDB_BN) * k_rsb;
     const char* vt = vb + (uint64_t)(uint32_t)(tile * FDB_BN) * v_rsb;
     const int last = Lb - 1 - tile * FDB_BN;
@@ -520,7 +528,7 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
         dma_cur = 2 * C::DMA_BUF;  // stage() steps to buffer 0
       } else {
         tile_load<D * QT::SZ>(kreg, kb, k_rsb, first * FDB_BN, Lb, tid);
-        tile_load<D * VT::SZ>(vreg, vb, v_rsb, first * FDB_BN, Lb, tid);
+        tile_load<D * VT::SZ>(vreg, vb, v_rsb, first * FDB_BN, Lb, tid);  // kv_alias: stays in registers until stage_v
       }
     }
   }
@@ -528,7 +536,7 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
   auto stage = [&](int t) __attribute__((always_inline)) {
     if constexpr (DMA) {
       const int nt = next_tile(t);
-      if (nt < t_end) wait_vmcnt<4>(); else wait_vmcnt<0>();  // this wave's part of tile t has landed (tile nt's may still fly)
+      if (nt < t_end) wait_vmcnt<kDmaLoadsPerTile>(); else wait_vmcnt<0>();  // this wave's part of tile t has landed (tile nt's may still fly)
       __syncthreads();  // ... and everyone's; every wave is done with the tile before
       dma_cur = dma_cur == 2 * C::DMA_BUF ? 0 : dma_cur + C::DMA_BUF;
       if (nt < t_end) {
@@ -543,13 +551,23 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
     } else {
       __syncthreads();  // every wave is done with the previous tile and its bias scratch
       tile_store<D * QT::SZ, C::K_RS>(Ks, kreg, tid);
-      tile_store<D * VT::SZ, C::V_RS>(Vs, vreg, tid);
+      if constexpr (!KV_ALIAS) tile_store<D * VT::SZ, C::V_RS>(Vs, vreg, tid);
       __syncthreads();
       const int nt = next_tile(t);
       if (nt < t_end) {  // next tile's global loads fly during this tile's math
         tile_load<D * QT::SZ>(kreg, kb, k_rsb, nt * FDB_BN, Lb, tid);
-        tile_load<D * VT::SZ>(vreg, vb, v_rsb, nt * FDB_BN, Lb, tid);
+        if constexpr (!KV_ALIAS) tile_load<D * VT::SZ>(vreg, vb, v_rsb, nt * FDB_BN, Lb, tid);
       }
+    }
+  };
+  // K and V in one buffer: once every wave has its scores of tile t, V replaces K.
+  auto stage_v = [&](int t) __attribute__((always_inline)) {
+    if constexpr (KV_ALIAS) {
+      __syncthreads();
+      tile_store<D * VT::SZ, C::V_RS>(Vs, vreg, tid);
+      __syncthreads();
+      const int nt = next_tile(t);
+      if (nt < t_end) tile_load<D * VT::SZ>(vreg, vb, v_rsb, nt * FDB_BN, Lb, tid);
     }
   };
   auto vload = [&](int c, int d) __attribute__((always_inline)) {
@@ -596,13 +614,19 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
     for (int t = t0; t < t1; ++t) {
       stage(t);
       f32x16 sacc[2];
-      if constexpr (PRE) {
+      if constexpr (PRE && !KV_ALIAS) {
         qk(sacc, qfar, negm);
         auto requery = [&](f32x16 (&sx)[2]) __attribute__((always_inline)) { qk(sx, qfar, negm); };
         softmax_pv_pre2<VT, D, MASK>(sacc, o_acc, m_run, l_run, a_far, negm, vload, requery, lane, t * FDB_BN, i, Lb,
                                      MASK && p.causal != 0);
+      } else if constexpr (PRE) {  // K is gone once V is staged: no second pass over the scores
+        qk(sacc, qfar, negm);
+        stage_v(t);
+        softmax_pv_pre<VT, D, MASK>(sacc, o_acc, m_run, l_run, a_far, negm, vload, lane, t * FDB_BN, i, Lb,
+                                    MASK && p.causal != 0);
       } else {
         qk(sacc, qf, zero16);
+        stage_v(t);
         softmax_pv<VT, D, MASK>(sacc, o_acc, m_run, l_run, x_scale, a_far, vload, lane, t * FDB_BN, i, Lb,
                                 MASK && p.causal != 0);
       }
@@ -932,6 +956,7 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
             if constexpr (P2C) sacc[jb][v] += (float)pbase[cj * kP2cStride - cj];
           }
       }
+      stage_v(t);
       softmax_pv<VT, D, MASK>(sacc, o_acc, m_run, l_run, x_scale, 0.f, vload, lane, j0, i, Lb,
                               MASK && p.causal != 0);
     }
@@ -1007,7 +1032,8 @@ int launch_one(const FdbKParams& p, int grid_x, hipStream_t stream) {
   auto kern = fdb_attn_kernel<QT, VT, D, FP8, C2P, P2C, MODE>;
   constexpr int lds = C::lds_bytes_mode(MODE, C2P, P2C);
   static_assert(lds <= 160 * 1024, "LDS budget");
-  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+  static std::atomic<uint64_t> lds_set{0};
+  hipError_t e = fdb_set_lds_once((const void*)kern, lds, lds_set);
   if (e != hipSuccess) return (int)e;
   const unsigned parts = MODE == kFarOnly && p.far_parts > 1 ? (unsigned)p.far_parts : 1u;
   hipLaunchKernelGGL(kern, dim3((unsigned)grid_x * p.H, parts, 1), dim3(kThreads), lds, stream, p);
@@ -1057,7 +1083,8 @@ int fdb_launch_attn(const FdbKParams& p, int dtype, int head_dim, int grid_x, in
       switch (head_dim) {
         case 32: return launch_pos<F32Tr, F32Tr, 32, false>(p, grid_x, mode, stream);
         case 64: return launch_pos<F32Tr, F32Tr, 64, false>(p, grid_x, mode, stream);
-        default: return FDB_ERR_UNSUPPORTED;
+        case 128: return launch_pos<F32Tr, F32Tr, 128, false>(p, grid_x, mode, stream);
+        default: return FDB_ERR_HEAD_DIM;
       }
     case FDB_FP8_E4M3: FDB_DISPATCH_D(Fp8Tr, Bf16Tr, true)
     default: return FDB_ERR_DTYPE;

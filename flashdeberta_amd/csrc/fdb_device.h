@@ -293,10 +293,13 @@ __device__ __forceinline__ void block_map(int n, int nx, int heads, int tiles_pe
 // that the compiler keeps no account of it: the kernel waits for these loads itself, with
 // wait_vmcnt, and only for the tile it is about to read.  Loads complete in issue order, so the
 // compiler's own vmcnt waits, which do not count them, can only wait longer than needed.  M0 is
-// written without being declared (it is a reserved register): nothing else in these kernels uses it.
+// a reserved register that cannot be named as a clobber: the block saves it, sets it, uses it and puts
+// the old value back, so whatever the compiler itself keeps in M0 survives the block.
 __device__ __forceinline__ void dma16(const void* g, uint32_t lds_base) {
   const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(base) : "memory");
+  uint32_t keep;
+  asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0"
+               : "=&s"(keep) : "v"(g), "s"(base) : "memory");
 }
 // The same with the address split into a base that is the same in every lane (it travels in scalar
 // registers) and this lane's 32-bit byte offset from it.
@@ -305,7 +308,9 @@ __device__ __forceinline__ void dma16s(const void* base, uint32_t lane_off, uint
   const uint64_t b64 = (uint64_t)(uintptr_t)base;
   const uint32_t blo = __builtin_amdgcn_readfirstlane((uint32_t)b64), bhi = __builtin_amdgcn_readfirstlane((uint32_t)(b64 >> 32));
   const uint64_t sb = ((uint64_t)bhi << 32) | blo;
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(sb), "s"(lb) : "memory");
+  uint32_t keep;
+  asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\ts_mov_b32 m0, %0"
+               : "=&s"(keep) : "v"(lane_off), "s"(sb), "s"(lb) : "memory");
 }
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
@@ -313,6 +318,10 @@ __device__ __forceinline__ void wait_vmcnt() {
   if constexpr (N == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   if constexpr (N == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
 }
+
+// Number of direct loads (dma16 / dma16s) a wave issues per K/V tile of the far-only staging: the waits
+// of that staging name this count, so the two are tied together here.
+constexpr int kDmaLoadsPerTile = 4;
 
 // Orders this wave's earlier LDS accesses before its later ones (the LDS unit executes one wave's
 // operations in order; this only stops the compiler from moving them across).

@@ -62,6 +62,22 @@ __device__ __forceinline__ float* far_part_lse(const FdbKParams& p, int part, in
 }
 #endif
 
+#if defined(__HIPCC__)
+// hipFuncSetAttribute(MaxDynamicSharedMemorySize) once per kernel instantiation and device instead of
+// once per launch.  `done` is a per-instantiation bit mask over device ordinals (a racing first call
+// merely sets the attribute twice).
+#include <atomic>
+inline hipError_t fdb_set_lds_once(const void* kern, int lds_bytes, std::atomic<uint64_t>& done) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+  const uint64_t bit = 1ull << dev;
+  if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+  const hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+  if (e == hipSuccess) done.fetch_or(bit, std::memory_order_release);
+  return e;
+}
+#endif
+
 // Most workgroups per query tile a far-only launch is split into.
 #define FDB_MAX_FAR_PARTS 4
 

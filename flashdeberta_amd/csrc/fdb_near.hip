@@ -518,7 +518,8 @@ int launch_near_one(const FdbKParams& p, int grid_x, hipStream_t stream) {
   auto kern = fdb_near_kernel<QT, QT, C2P, P2C>;
   constexpr int lds = NCfg::lds_bytes(C2P, P2C);
   static_assert(lds <= 80 * 1024, "two workgroups per CU");
-  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+  static std::atomic<uint64_t> lds_set{0};
+  hipError_t e = fdb_set_lds_once((const void*)kern, lds, lds_set);
   if (e != hipSuccess) return (int)e;
   hipLaunchKernelGGL(kern, dim3((unsigned)grid_x * p.H, p.near_parts > 1 ? (unsigned)p.near_parts : 1u, 1), dim3(kNThreads),
                      lds, stream, p);

@@ -24,25 +24,32 @@ from . import ops
 from .padding import key_padding_mask, seq_bounds
 
 
+def _stamp(t):
+    """What a remembered value depends on besides the tensor object: its in-place version counter, and the
+    storage, dtype and device behind it (`p.data = x`, `module.to(dtype)` and `.half()` swap those under
+    an unchanged object and version)."""
+    return (t._version, t.data_ptr(), t.dtype, t.device)
+
+
 class _Memo:
-    """One remembered value, valid while the tensors it was computed from are the same objects and
-    have not been written in place (their version counters are unchanged) and `extra` compares equal.
-    The tensors are held weakly."""
+    """One remembered value, valid while the tensors it was computed from are the same objects, have not
+    been written in place, still sit in the same storage with the same dtype on the same device, and
+    `extra` compares equal.  The tensors are held weakly."""
 
     def __init__(self):
-        self._refs, self._versions, self._extra, self._value = (), (), None, None
+        self._refs, self._stamps, self._extra, self._value = (), (), None, None
 
     def get(self, tensors, extra=None):
         if len(self._refs) != len(tensors) or extra != self._extra:
             return None
-        for ref, ver, t in zip(self._refs, self._versions, tensors):
-            if ref() is not t or t._version != ver:
+        for ref, stamp, t in zip(self._refs, self._stamps, tensors):
+            if ref() is not t or _stamp(t) != stamp:
                 return None
         return self._value
 
     def put(self, tensors, value, extra=None):
         self._refs = tuple(weakref.ref(t) for t in tensors)
-        self._versions = tuple(t._version for t in tensors)
+        self._stamps = tuple(_stamp(t) for t in tensors)
         self._extra, self._value = extra, value
         return value
 
@@ -50,16 +57,15 @@ class _Memo:
         return (_Memo, ())
 
 
-_MASK_MEMO = _Memo()
-
-
 def _seq_bounds_of(attention_mask):
-    """(seq_start, seq_len) of a mask; every layer of an encoder receives the same mask object, so
-    the two reductions run once per forward instead of once per layer."""
-    hit = _MASK_MEMO.get((attention_mask,))
-    if hit is None:
-        hit = _MASK_MEMO.put((attention_mask,), seq_bounds(key_padding_mask(attention_mask)))
-    return hit
+    """(seq_start, seq_len, holes) of a mask; every layer of an encoder receives the same mask object, so
+    the reductions run once per forward instead of once per layer.  The result rides on the mask tensor
+    itself (no state outside it) and is dropped when the mask is written in place or re-seated."""
+    hit = attention_mask.__dict__.get("_fdb_bounds")
+    if hit is None or hit[0] != _stamp(attention_mask):
+        hit = (_stamp(attention_mask), seq_bounds(key_padding_mask(attention_mask)))
+        attention_mask._fdb_bounds = hit
+    return hit[1]
 
 
 class FlashDisentangledSelfAttention(DisentangledSelfAttention):
@@ -142,6 +148,9 @@ class FlashDisentangledSelfAttention(DisentangledSelfAttention):
         materialised, so `output_attentions` yields None like the reference (model.py:252)."""
         if self.training and torch.is_grad_enabled() and hidden_states.requires_grad:
             raise RuntimeError("FlashDisentangledSelfAttention is forward-only; use the eager implementation to train")
+        # Outside training the forward still runs with autograd recording (the reference's test calls the
+        # module without no_grad); the fused op then sits in the graph as a node whose backward raises, as the
+        # reference's packed op does (flash_attention_varlen.py:480-483), instead of cutting the graph silently.
         if query_states is None:
             query_states = hidden_states
         B, L, _ = hidden_states.shape
@@ -159,8 +168,11 @@ class FlashDisentangledSelfAttention(DisentangledSelfAttention):
         seq_start = seq_len = None
         out = None
         if attention_mask is not None:
-            seq_start, seq_len = _seq_bounds_of(attention_mask)
-            out = torch.zeros((B, L, H, D), dtype=v.dtype, device=v.device)  # padded rows stay zero
+            seq_start, seq_len, holes = _seq_bounds_of(attention_mask)
+            # Padded rows stay zero.  The kernels take the real tokens of a row as one contiguous run; a row
+            # whose mask has a hole inside that run gets no tokens (seq_len 0) and NaN in every position, so
+            # the unsupported mask cannot pass for a result (the eager module honours arbitrary masks).
+            out = torch.where(holes.view(B, 1, 1, 1), float("nan"), 0.0).to(v.dtype).expand(B, L, H, D).contiguous()
 
         kw = {}
         if self.fp8_qk:
@@ -175,7 +187,7 @@ class FlashDisentangledSelfAttention(DisentangledSelfAttention):
                 pos_query, kw["pos_query_scale"] = ops.quantize_e4m3_per_head(pos_query.transpose(0, 1))
                 pos_query = pos_query.transpose(0, 1)
 
-        ctx = ops.disentangled_attention_fwd(
+        ctx = ops.disentangled_attention_forward_only(
             q, k, v, pos_key, pos_query, sm_scale=sm_scale,
             position_buckets=self.position_buckets if self.relative_attention else 0,
             max_relative_positions=self.max_relative_positions if self.relative_attention else 0,

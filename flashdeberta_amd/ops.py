@@ -223,6 +223,28 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
     return (out, lse) if return_lse else out
 
 
+class _ForwardOnly(torch.autograd.Function):
+    """The fused forward as an autograd node whose backward raises: a graph that runs through the op fails
+    loudly at .backward() instead of silently dropping the gradients of everything before it (the
+    reference's packed op does the same, flash_attention_varlen.py:480-483)."""
+
+    @staticmethod
+    def forward(ctx, kwargs, q, k, v, pos_key, pos_query):
+        return disentangled_attention_fwd(q, k, v, pos_key, pos_query, **kwargs)
+
+    @staticmethod
+    def backward(ctx, *grads):
+        raise RuntimeError("the fused disentangled attention is forward-only: no backward is implemented; "
+                           "use the eager implementation where gradients are needed")
+
+
+def disentangled_attention_forward_only(q, k, v, pos_key=None, pos_query=None, **kwargs):
+    """disentangled_attention_fwd (single output, no return_lse) for callers that may run under autograd."""
+    if torch.is_grad_enabled() and any(x is not None and x.requires_grad for x in (q, k, v, pos_key, pos_query)):
+        return _ForwardOnly.apply(kwargs, q, k, v, pos_key, pos_query)
+    return disentangled_attention_fwd(q, k, v, pos_key, pos_query, **kwargs)
+
+
 def flash_attention_with_disentangled(q, k, v, k_pos, q_pos, causal=False, sm_scale=None,
                                       position_buckets=0, max_relative_distance=0):
     """Same call shape as the reference op (flash_attention.py:1088-1091): q, k, v [B, H, L, D],

@@ -26,12 +26,26 @@ def key_padding_mask(attention_mask):
 
 
 def seq_bounds(mask2d):
-    """[B, L] bool -> (seq_start int32 [B], seq_len int32 [B]) on the mask's device, no host sync.
-    The real tokens of a row are assumed contiguous (left or right padding)."""
+    """[B, L] bool -> (seq_start int32 [B], seq_len int32 [B], holes bool [B]) on the mask's device, no
+    host sync.  The kernels take the real tokens of a row as one contiguous run (left or right padding).
+    A row whose ones are not contiguous is flagged in `holes` and given seq_len 0, so that nothing is
+    computed from a mask the kernels cannot honour."""
     m = mask2d.to(torch.int32)
-    seq_len = m.sum(dim=-1, dtype=torch.int32)
-    seq_start = torch.argmax(m, dim=-1).to(torch.int32)  # first 1; 0 for an all-padding row
-    return seq_start, seq_len
+    L = m.shape[-1]
+    count = m.sum(dim=-1, dtype=torch.int32)
+    first = torch.argmax(m, dim=-1).to(torch.int32)  # first 1; 0 for an all-padding row
+    last = (L - 1 - torch.argmax(m.flip(-1), dim=-1)).to(torch.int32)
+    holes = (count > 0) & (last - first + 1 != count)
+    return first, torch.where(holes, torch.zeros_like(count), count), holes
+
+
+def assert_contiguous_mask(attention_mask):
+    """Raise ValueError if any row of the mask has masked tokens between real ones (one host sync);
+    for callers that prefer an error to the NaN rows the module writes for such a mask."""
+    _, _, holes = seq_bounds(key_padding_mask(attention_mask))
+    if bool(holes.any()):
+        raise ValueError("attention_mask rows %s have masked tokens between real ones; the fused attention takes "
+                         "the real tokens of a row as one contiguous run" % holes.nonzero().flatten().tolist())
 
 
 def get_unpad_data(mask2d):

@@ -104,7 +104,7 @@ def test_argument_validation_codes():
     a = _good_args(); a.att_span = 0; assert chk(a) == -6
     a = _good_args(); a.dtype = _lib.FDB_FP8_E4M3; assert chk(a) == -7   # no scales
     a = _good_args(); a.cu_seqlens = 0x4000; assert chk(a) == -8          # no work-list
-    a = _good_args(); a.dtype = _lib.FDB_F32; a.head_dim = 128; assert chk(a) == -10
+    a = _good_args(); a.dtype = _lib.FDB_F32; a.head_dim = 128; assert chk(a) == 0       # every dtype at every head_dim
     a = _good_args(); a.pos_key = a.pos_query = None; a.delta_lut = None; a.att_span = 0; assert chk(a) == 0
     assert lib.fdb_attn_check(None) == -1
     # launching with bad arguments returns the same code without touching the GPU
@@ -257,6 +257,18 @@ def test_module_projection_memos():
         pk2, pq2 = att._pos_layers(rel)
         assert pq2 is not pq and torch.allclose(pq2, att.query_proj(rel).view(64, 2, 64).transpose(0, 1))
         assert att._pos_layers(rel.clone())[0] is not pk2      # another tensor object
+        # a parameter re-seated through .data (EMA / loader style weight swaps): same object, same version
+        att.key_proj.weight.data = torch.randn_like(att.key_proj.weight)
+        for got, ref in zip(att._qkv(x, x), separate()):
+            assert torch.allclose(got, ref, atol=1e-6)
+        assert torch.allclose(att._pos_layers(rel)[0], att.key_proj(rel).view(64, 2, 64).transpose(0, 1))
+        # a cast of the whole module after a forward: the remembered tensors follow the new dtype
+        att.to(torch.bfloat16)
+        assert att._fused_qkv()[0].dtype == torch.bfloat16
+        assert att._pos_layers(rel.to(torch.bfloat16))[0].dtype == torch.bfloat16
+        att.to(torch.float32)
+        for got, ref in zip(att._qkv(x, x), separate()):
+            assert torch.allclose(got, ref, atol=1e-6)
     att.train()
     assert att._pos_layers(rel)[0] is not att._pos_layers(rel)[0]
 
@@ -288,11 +300,12 @@ def test_module_projection_memos():
 
     # mask bounds: once per mask object and version
     m = torch.tensor([[1, 1, 1, 0, 0], [0, 0, 1, 1, 1]])
-    s0, n0 = _seq_bounds_of(m)
-    assert _seq_bounds_of(m)[0] is s0 and s0.tolist() == [0, 2] and n0.tolist() == [3, 3]
+    s0, n0, h0 = _seq_bounds_of(m)
+    assert _seq_bounds_of(m)[0] is s0 and s0.tolist() == [0, 2] and n0.tolist() == [3, 3] and not h0.any()
     m[0, 3] = 1
-    s1, n1 = _seq_bounds_of(m)
+    s1, n1, _ = _seq_bounds_of(m)
     assert s1 is not s0 and n1.tolist() == [4, 3]
+    assert _seq_bounds_of(m.clone())[0] is not s1  # the result rides on the mask object: nothing global
 
 
 def test_padding_helpers():
@@ -301,11 +314,21 @@ def test_padding_helpers():
     m = torch.tensor([[1, 1, 1, 0, 0], [0, 0, 1, 1, 1], [1, 1, 1, 1, 1]])
     ext = m[:, None, None, :] * m[:, None, :, None]
     assert torch.equal(key_padding_mask(ext), m.bool()) and torch.equal(key_padding_mask(m), m.bool())
-    s, n = seq_bounds(m.bool())
-    assert s.tolist() == [0, 2, 0] and n.tolist() == [3, 3, 5]
+    s, n, holes = seq_bounds(m.bool())
+    assert s.tolist() == [0, 2, 0] and n.tolist() == [3, 3, 5] and holes.tolist() == [False, False, False]
+    # masked tokens between real ones: flagged, and the row gets no tokens
+    mh = torch.tensor([[1, 1, 0, 1, 1], [0, 1, 1, 1, 0], [0, 0, 0, 0, 0], [1, 0, 0, 0, 1]]).bool()
+    s, n, holes = seq_bounds(mh)
+    assert holes.tolist() == [True, False, False, True] and n.tolist() == [0, 3, 0, 0] and s.tolist()[1] == 1
+    from flashdeberta_amd.padding import assert_contiguous_mask
+    assert_contiguous_mask(m)
+    with pytest.raises(ValueError, match="rows \\[0, 3\\]"):
+        assert_contiguous_mask(mh)
     idx, cu, mx = get_unpad_data(m.bool())
+    # literal values: flattened positions of the ones of the three rows, their running counts, the longest row
+    assert idx.tolist() == [0, 1, 2, 7, 8, 9, 10, 11, 12, 13, 14] and cu.tolist() == [0, 3, 6, 11] and int(mx) == 5
     ref_idx, ref_cu, ref_mx = O.unpad_data(m.numpy())
-    assert idx.tolist() == ref_idx.tolist() and cu.tolist() == ref_cu.tolist() and int(mx) == ref_mx
+    assert ref_idx.tolist() == [0, 1, 2, 7, 8, 9, 10, 11, 12, 13, 14] and ref_cu.tolist() == [0, 3, 6, 11] and ref_mx == 5
     x = torch.arange(15.0).view(3, 5, 1)
     assert torch.equal(pad_input(unpad_input(x, idx), idx, 3, 5), x * m[:, :, None])
 
