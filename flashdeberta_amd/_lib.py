@@ -12,7 +12,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libfdb_hip.so")
 
 FDB_F32, FDB_BF16, FDB_F16, FDB_FP8_E4M3 = 0, 1, 2, 3
-FDB_VERSION = 3  # of include/fdb.h as mirrored below
+FDB_NOALLOC_SCRATCH_BYTES = 32 * 1024 * 1024
+FDB_VERSION = 4  # of include/fdb.h as mirrored below
 
 
 class FdbAttnArgs(ctypes.Structure):
@@ -32,7 +33,7 @@ class FdbAttnArgs(ctypes.Structure):
 
 
 EXPORTS = (
-    "fdb_version", "fdb_attn_args_size", "fdb_strerror", "fdb_attn_check", "fdb_attn_fwd", "fdb_attn_workspace_bytes",
+    "fdb_version", "fdb_attn_args_size", "fdb_strerror", "fdb_attn_check", "fdb_attn_fwd", "fdb_attn_fwd_noalloc", "fdb_attn_workspace_bytes",
     "fdb_worklist_ints",
     "fdb_worklist_max_tiles", "fdb_tile_rows", "fdb_build_worklist", "fdb_delta_lut_radius", "fdb_delta_lut",
     "fdb_quant_e4m3_per_head", "fdb_dequant_e4m3_per_head",
@@ -60,6 +61,8 @@ def _load():
     lib.fdb_attn_check.argtypes = [ctypes.POINTER(FdbAttnArgs)]
     lib.fdb_attn_fwd.restype = ctypes.c_int
     lib.fdb_attn_fwd.argtypes = [ctypes.POINTER(FdbAttnArgs), vp]
+    lib.fdb_attn_fwd_noalloc.restype = ctypes.c_int
+    lib.fdb_attn_fwd_noalloc.argtypes = [ctypes.POINTER(FdbAttnArgs), vp]
     lib.fdb_attn_workspace_bytes.restype = i64
     lib.fdb_attn_workspace_bytes.argtypes = [ctypes.POINTER(FdbAttnArgs)]
     lib.fdb_worklist_ints.restype = i64

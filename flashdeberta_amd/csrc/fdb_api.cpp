@@ -6,7 +6,7 @@
 
 #include <atomic>
 
-#include <hip/hip_runtime_api.h>
+#include <hip/hip_runtime.h>
 
 #include "../../include/fdb.h"
 #include "fdb_kernels.h"
@@ -151,6 +151,56 @@ int64_t far_part_bytes(const fdb_attn_args* a) {
 
 }  // namespace
 
+// ---- the entry point that allocates nothing ---------------------------------------------------------
+// Its scratch lives in the library's own device image: one copy per GPU, held until the process ends.
+// The name below is a host-side handle only; the device address is asked for once per device
+// (hipGetSymbolAddress) and that pointer is what kernels receive.
+static __device__ __align__(256) unsigned char fdb_noalloc_scratch[FDB_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+
+std::atomic<unsigned char*> g_scratch_ptr[64];
+
+// Device address of this GPU's copy of the scratch array (nullptr + error code on failure).
+int scratch_base(unsigned char** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= 64) return FDB_ERR_SCRATCH;
+  unsigned char* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    void* sym = nullptr;
+    e = hipGetSymbolAddress(&sym, HIP_SYMBOL(fdb_noalloc_scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!sym) return FDB_ERR_SCRATCH;
+    p = (unsigned char*)sym;
+    g_scratch_ptr[dev].store(p, std::memory_order_release);  // a racing first call stores the same address
+  }
+  *out = p;
+  return FDB_OK;
+}
+
+int64_t align256(int64_t n) { return (n + 255) & ~(int64_t)255; }
+
+// What fdb_attn_fwd_noalloc validates before it launches: the argument block as fdb_attn_fwd sees it,
+// and that the hand-over buffers fit the scratch.
+int check_noalloc(const fdb_attn_args* a) {
+  if (!a) return FDB_ERR_NULL;
+  fdb_attn_args b = *a;
+  int32_t dummy_wl = 0;
+  if (b.cu_seqlens && !b.worklist) b.worklist = &dummy_wl;  // supplied from the scratch by the call itself
+  b.workspace = nullptr;
+  b.workspace_bytes = 0;
+  const int rc = fdb_attn_check(&b);
+  if (rc != FDB_OK) return rc;
+  int64_t need = 0;
+  if (!b.lse && (b.pos_key || b.pos_query) && fdb_near_supported(b.dtype, b.head_dim)) need += align256(lse_rows(&b) * b.heads * 4);
+  if (b.cu_seqlens) need += align256(fdb_worklist_ints(b.total_tokens, b.batch) * 4);
+  return need > FDB_NOALLOC_SCRATCH_BYTES ? FDB_ERR_SCRATCH : FDB_OK;
+}
+
+}  // namespace
+
 extern "C" {
 
 int fdb_version(void) { return FDB_VERSION; }
@@ -170,6 +220,7 @@ const char* fdb_strerror(int code) {
     case FDB_ERR_WORKLIST: return "cu_seqlens given without a work-list buffer";
     case FDB_ERR_LUT_ARGS: return "invalid position_buckets/max_position/radius/out for the delta table";
     case FDB_ERR_UNSUPPORTED: return "dtype/head_dim combination not built";
+    case FDB_ERR_SCRATCH: return "fdb_attn_fwd_noalloc: the call needs more than FDB_NOALLOC_SCRATCH_BYTES of built-in scratch";
     default: break;
   }
   if (code > 0) return hipGetErrorString((hipError_t)code);
@@ -294,6 +345,35 @@ int fdb_attn_fwd(const fdb_attn_args* a, void* stream) {
     return fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, FDB_MODE_NEAR_RING, stream);
   }
   return fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, FDB_MODE_FUSED, stream);
+}
+
+int fdb_attn_fwd_noalloc(const fdb_attn_args* a, void* stream) {
+  const int rc = check_noalloc(a);
+  if (rc != FDB_OK) return rc;
+  fdb_attn_args b = *a;
+  unsigned char* base = nullptr;
+  const int rs = scratch_base(&base);
+  if (rs != FDB_OK) return rs;
+  // [log-sum-exp hand-over][work-list][partial results], each part 256-byte aligned
+  int64_t off = 0;
+  const bool has_pos = b.pos_key || b.pos_query;
+  if (!b.lse && has_pos && fdb_near_supported(b.dtype, b.head_dim)) {
+    b.lse = (float*)(base + off);
+    off += align256(lse_rows(&b) * b.heads * 4);
+  }
+  if (b.cu_seqlens) {
+    b.worklist = (int32_t*)(base + off);
+    off += align256(fdb_worklist_ints(b.total_tokens, b.batch) * 4);
+  }
+  if (off > FDB_NOALLOC_SCRATCH_BYTES) return FDB_ERR_SCRATCH;
+  // what is left holds as many partial results as fit: the call shares less with a smaller remainder
+  b.workspace = base + off;
+  b.workspace_bytes = FDB_NOALLOC_SCRATCH_BYTES - off;
+  if (b.cu_seqlens) {
+    const int rw = fdb_launch_worklist(b.cu_seqlens, b.batch, b.worklist, fdb_worklist_max_tiles(b.total_tokens, b.batch), stream);
+    if (rw != 0) return rw;
+  }
+  return fdb_attn_fwd(&b, stream);
 }
 
 int fdb_build_worklist(const int32_t* cu_seqlens, int32_t batch, int32_t total_tokens, int32_t* worklist,

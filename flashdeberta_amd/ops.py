@@ -80,7 +80,8 @@ def _pos_arg(x, H, D, span, name):
 def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seqlens=None, max_seqlen=None,
                                sm_scale=None, position_buckets=0, max_relative_positions=0, causal=False,
                                return_lse=False, seq_start=None, seq_len=None, q_scale=None, k_scale=None, pos_key_scale=None,
-                               pos_query_scale=None, out=None, single_kernel=False, far_splits=0, near_splits=0, workspace=None):
+                               pos_query_scale=None, out=None, single_kernel=False, far_splits=0, near_splits=0, workspace=None,
+                               no_alloc=False):
     """Fused forward.  Layouts (strides are free except a unit stride on D):
          fixed length : q, k, v  [B, L, H, D]   -> out [B, L, H, D] (contiguous: a free view of [B, L, H*D])
          packed varlen: q, k, v  [T, H, D] + cu_seqlens int32 [B+1] (+ max_seqlen upper bound) -> out [T, H, D]
@@ -97,6 +98,10 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
        workspace: a uint8 GPU tensor for the partial results of such shared launches, to reuse one buffer across
        calls; by default one of the size the library asks for is allocated per call.  A smaller one is fine: the
        library then shares less.
+       no_alloc=True goes through fdb_attn_fwd_noalloc: the log-sum-exp hand-over, the work-list of a packed
+       call and the partial results come from the scratch built into the library (one per GPU; calls on one
+       GPU must not overlap), so with `out` given nothing is allocated on the way; the fp8 expansion and
+       single_kernel are not available there.
     """
     if not q.is_cuda:
         raise RuntimeError("disentangled_attention_fwd runs on the GPU only; got device %s" % q.device)
@@ -124,7 +129,7 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
         if q_scale is None or k_scale is None or (pos_key is not None and pos_key_scale is None) or (
                 pos_query is not None and pos_query_scale is None):
             raise ValueError("fp8 path: q_scale, k_scale and a scale for each position tensor are required")
-        if D <= 64 and not single_kernel:
+        if D <= 64 and not single_kernel and not no_alloc:
             # At head_dim <= 64 a key tile is bound by its soft-max and LDS work, not by the MFMA rate, and the
             # 16-bit kernels (direct-to-LDS staging, far / near pair of launches) are about three times faster
             # than the fp8-MFMA kernel: FP8 operands are expanded to bf16 (scale applied, one rounding to eight
@@ -165,7 +170,9 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
         raise ValueError("out must have q's shape, v's dtype and a unit stride on D")
     # the log-sum-exp buffer is also the hand-over between the far-tile and near-tile launches, so it is
     # always provided when a position term is present (T*H floats)
-    want_lse = return_lse or ((pos_key is not None or pos_query is not None) and not single_kernel)
+    if no_alloc and (single_kernel or workspace is not None):
+        raise ValueError("no_alloc excludes single_kernel and a caller-owned workspace")
+    want_lse = return_lse or ((pos_key is not None or pos_query is not None) and not single_kernel and not no_alloc)
     lse = torch.empty((T, H), dtype=torch.float32, device=q.device) if want_lse else None
     a.q, a.k, a.v, a.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
     a.pos_key, a.pos_query = (_ptr(pos_key) or ctypes.c_void_p()).value, (_ptr(pos_query) or ctypes.c_void_p()).value
@@ -175,10 +182,12 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
             setattr(a, n + "_stride_b", 0)
             setattr(a, n + "_stride_t", x.stride(0))
             setattr(a, n + "_stride_h", x.stride(1))
-        wl = torch.empty(int(lib.fdb_worklist_ints(T, B)), dtype=torch.int32, device=q.device)
-        keep.append(wl)
-        check(lib.fdb_build_worklist(_ptr(cu_seqlens), B, T, _ptr(wl), _stream_ptr(q.device)), "fdb_build_worklist")
-        a.cu_seqlens, a.worklist = cu_seqlens.data_ptr(), wl.data_ptr()
+        a.cu_seqlens = cu_seqlens.data_ptr()
+        if not no_alloc:
+            wl = torch.empty(int(lib.fdb_worklist_ints(T, B)), dtype=torch.int32, device=q.device)
+            keep.append(wl)
+            check(lib.fdb_build_worklist(_ptr(cu_seqlens), B, T, _ptr(wl), _stream_ptr(q.device)), "fdb_build_worklist")
+            a.worklist = wl.data_ptr()
     else:
         for n, x in (("q", q), ("k", k), ("v", v), ("o", out)):
             setattr(a, n + "_stride_b", x.stride(0))
@@ -208,6 +217,9 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
     a.dtype, a.causal, a.sm_scale, a.far_splits = dt, int(bool(causal)), float(sm_scale), int(far_splits)
     a.near_splits = int(near_splits)
     with torch.cuda.device(q.device):
+        if no_alloc:
+            check(lib.fdb_attn_fwd_noalloc(ctypes.byref(a), _stream_ptr(q.device)), "fdb_attn_fwd_noalloc")
+            return (out, lse) if return_lse else out
         if workspace is not None:
             if workspace.dtype != torch.uint8 or not workspace.is_cuda or not workspace.is_contiguous():
                 raise ValueError("workspace must be a contiguous uint8 GPU tensor")

@@ -35,7 +35,7 @@ extern "C" {
 #endif
 
 /* bumped whenever fdb_attn_args or the meaning of an entry point changes: a binding checks it next to the struct size */
-#define FDB_VERSION 3
+#define FDB_VERSION 4
 
 /* element types of q/k/pos_key/pos_query (v and out: see fdb_attn_args.dtype) */
 enum fdb_dtype {
@@ -57,7 +57,8 @@ enum fdb_status {
   FDB_ERR_SCALE = -7,       /* fp8 dtype without the needed scale vectors                  */
   FDB_ERR_WORKLIST = -8,    /* cu_seqlens given without a work-list buffer                 */
   FDB_ERR_LUT_ARGS = -9,    /* fdb_delta_lut: bad bucket/max_position/radius/out           */
-  FDB_ERR_UNSUPPORTED = -10 /* combination not built                                       */
+  FDB_ERR_UNSUPPORTED = -10, /* combination not built                                      */
+  FDB_ERR_SCRATCH = -11     /* fdb_attn_fwd_noalloc: hand-over buffers exceed the built-in scratch */
 };
 
 /*
@@ -128,6 +129,23 @@ int fdb_attn_check(const fdb_attn_args* a);
 
 /* Enqueue the fused forward on `stream` (a hipStream_t). */
 int fdb_attn_fwd(const fdb_attn_args* a, void* stream);
+
+/*
+ * fdb_attn_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The caller passes the inputs
+ * and `out` only; what fdb_attn_fwd takes from caller-owned buffers besides them -- the log-sum-exp
+ * hand-over between its two launches (used when `lse` is NULL; a non-NULL `lse` is filled as usual), the
+ * packed layout's work-list (built here, `worklist` is ignored) and the workspace of partial results
+ * (`workspace` is ignored) -- comes from FDB_NOALLOC_SCRATCH_BYTES of device memory inside the library's
+ * own image, one copy per GPU, held until the process ends.  The call allocates and frees nothing.
+ * Limit: hand-over plus work-list, rows * heads * 4 + fdb_worklist_ints(...) * 4 bytes (each rounded up to
+ * 256), must fit the scratch, else FDB_ERR_SCRATCH and nothing is launched; partial results use what is
+ * left and the call shares less when that is small (same result up to rounding).  Nothing in the scratch
+ * has to start at zero (every word read was written earlier in the same call).  All calls on one GPU
+ * share its scratch: calls that overlap in time on one GPU (two streams, two threads) race; serialise them.
+ */
+#define FDB_NOALLOC_SCRATCH_BYTES (32 * 1024 * 1024)
+int fdb_attn_fwd_noalloc(const fdb_attn_args* a, void* stream);
 
 /*
  * Bytes of workspace the call would use (0: none), for the device that is current.  A launch whose

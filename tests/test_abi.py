@@ -33,7 +33,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_struct_mirror_and_version():
     assert lib.fdb_attn_args_size() == ctypes.sizeof(FdbAttnArgs)
-    assert lib.fdb_version() == _lib.FDB_VERSION == 3
+    assert lib.fdb_version() == _lib.FDB_VERSION == 4
     assert lib.fdb_tile_rows() == 128
 
 
@@ -331,6 +331,27 @@ def test_padding_helpers():
     assert ref_idx.tolist() == [0, 1, 2, 7, 8, 9, 10, 11, 12, 13, 14] and ref_cu.tolist() == [0, 3, 6, 11] and ref_mx == 5
     x = torch.arange(15.0).view(3, 5, 1)
     assert torch.equal(pad_input(unpad_input(x, idx), idx, 3, 5), x * m[:, :, None])
+
+
+def test_no_alloc_entry_point_refuses_what_does_not_fit():
+    # hand-over of rows * heads * 4 bytes: 8 x 65536 rows x 32 heads = 64 MiB > the 32 MiB scratch; host-side
+    # refusal, nothing is launched (the pointers are never dereferenced)
+    a = _lib.FdbAttnArgs()
+    a.q = a.k = a.v = a.out = a.pos_key = a.pos_query = a.delta_lut = 0x10000
+    B, L, H, D = 8, 65536, 32, 64
+    for n in ("q", "k", "v", "o"):
+        setattr(a, n + "_stride_b", L * H * D)
+        setattr(a, n + "_stride_t", H * D)
+        setattr(a, n + "_stride_h", D)
+    a.pk_stride_h = a.pq_stride_h = D
+    a.pk_stride_r = a.pq_stride_r = H * D
+    a.batch, a.heads, a.head_dim, a.max_seqlen, a.total_tokens = B, H, D, L, B * L
+    a.att_span, a.lut_radius, a.dtype, a.sm_scale = 256, 512, _lib.FDB_BF16, 0.07
+    assert lib.fdb_attn_check(ctypes.byref(a)) == 0
+    rc = lib.fdb_attn_fwd_noalloc(ctypes.byref(a), None)
+    assert rc == -11 and "scratch" in _lib.strerror(rc)
+    with pytest.raises(ValueError, match="scratch"):
+        _lib.check(rc, "fdb_attn_fwd_noalloc")
 
 
 def test_bench_contract_without_a_gpu():
