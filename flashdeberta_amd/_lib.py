@@ -28,7 +28,7 @@ class FdbAttnArgs(ctypes.Structure):
         + [(n, ctypes.c_int32) for n in (
             "batch", "heads", "head_dim", "max_seqlen", "total_tokens", "att_span", "lut_radius", "dtype", "causal", "far_splits",
             "near_splits")]
-        + [("sm_scale", ctypes.c_float)]
+        + [("sm_scale", ctypes.c_float), ("launch_mask", ctypes.c_int32)]
     )
 
 

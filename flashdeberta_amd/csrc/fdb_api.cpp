@@ -251,7 +251,7 @@ int fdb_attn_check(const fdb_attn_args* a) {
   if (a->batch < 1 || a->heads < 1 || a->heads > 65535 || a->max_seqlen < 1 || a->total_tokens < 1)
     return FDB_ERR_SHAPE;
   if (a->far_splits < 0 || a->far_splits > FDB_MAX_FAR_SPLITS || a->near_splits < 0 ||
-      a->near_splits > FDB_MAX_FAR_SPLITS || a->workspace_bytes < 0)
+      a->near_splits > FDB_MAX_FAR_SPLITS || a->workspace_bytes < 0 || a->launch_mask < 0 || a->launch_mask > 2)
     return FDB_ERR_SHAPE;
   if (a->workspace && !aligned16(a->workspace)) return FDB_ERR_ALIGN;
   if (!a->cu_seqlens && (int64_t)a->batch * a->max_seqlen != a->total_tokens) return FDB_ERR_SHAPE;
@@ -331,10 +331,11 @@ int fdb_attn_fwd(const fdb_attn_args* a, void* stream) {
     p.ws_slots = p.far_parts - 1 + (p.near_parts > 1 ? p.near_parts : 0);
     p.ws = (char*)a->workspace;
     p.ws_rows = lse_rows(a);
-    if (need_far) {
+    if (need_far && a->launch_mask != 2) {
       const int rc_far = fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, FDB_MODE_FAR_ONLY, stream);
       if (rc_far != 0) return rc_far;
     }
+    if (a->launch_mask == 1) return FDB_OK;
     p.far_done = need_far ? 1 : 0;
     // head_dim 64: the near kernel (32-key steps, two workgroups per CU); head_dim 32: the fused kernel's ring mode
     if (fdb_near32_supported(a->dtype, a->head_dim)) {

@@ -81,7 +81,7 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
                                sm_scale=None, position_buckets=0, max_relative_positions=0, causal=False,
                                return_lse=False, seq_start=None, seq_len=None, q_scale=None, k_scale=None, pos_key_scale=None,
                                pos_query_scale=None, out=None, single_kernel=False, far_splits=0, near_splits=0, workspace=None,
-                               no_alloc=False):
+                               no_alloc=False, _launch_mask=0):
     """Fused forward.  Layouts (strides are free except a unit stride on D):
          fixed length : q, k, v  [B, L, H, D]   -> out [B, L, H, D] (contiguous: a free view of [B, L, H*D])
          packed varlen: q, k, v  [T, H, D] + cu_seqlens int32 [B+1] (+ max_seqlen upper bound) -> out [T, H, D]
@@ -216,6 +216,7 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
     a.batch, a.heads, a.head_dim, a.max_seqlen, a.total_tokens = B, H, D, L, T
     a.dtype, a.causal, a.sm_scale, a.far_splits = dt, int(bool(causal)), float(sm_scale), int(far_splits)
     a.near_splits = int(near_splits)
+    a.launch_mask = int(_launch_mask)  # measurement only: 1 = far launch alone, 2 = near launch alone
     with torch.cuda.device(q.device):
         if no_alloc:
             check(lib.fdb_attn_fwd_noalloc(ctypes.byref(a), _stream_ptr(q.device)), "fdb_attn_fwd_noalloc")

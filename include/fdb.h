@@ -115,6 +115,8 @@ typedef struct fdb_attn_args {
   int32_t far_splits;      /* 0: the library decides; 1 .. FDB_MAX_FAR_SPLITS: workgroups that share the far keys of a query tile */
   int32_t near_splits;     /* the same for the near keys (those whose bucketed relative position varies)                  */
   float sm_scale;
+  int32_t launch_mask;     /* 0: the whole call.  Measurement only (the output of such a call is not a result): 1 = only the
+                              launch over the far keys, 2 = only the launch over the near keys (and its merge kernel)       */
 } fdb_attn_args;
 
 #define FDB_MAX_FAR_SPLITS 4

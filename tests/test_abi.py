@@ -370,7 +370,14 @@ def test_bench_contract_without_a_gpu():
     assert abs(bench.flops([L] * B, H, D) / 1e9 - 463.86) < 0.01
     assert bench.flops([512], 12, 64, pos=False) == 12 * 4 * 512 * 512 * 64
     rec = bench.cpu_baseline(2, 64, 256)
-    assert rec["kind"] == "port" and rec["cores"] >= 1 and rec["value"] > 0 and rec["unit"] == "TFLOP/s"
-    assert "sample" in rec and ("eager_module" not in rec or "value" in rec["eager_module"] or "error" in rec["eager_module"])
+    # headline = the reference's eager class (transformers is installed here), the numpy port beside it
+    assert rec["kind"] == "reference" and rec["cores"] >= 1 and rec["value"] > 0 and rec["unit"] == "TFLOP/s"
+    assert "DisentangledSelfAttention" in rec["sample"]
+    assert rec["port"]["kind"] == "port" and rec["port"]["value"] > 0 and rec["port"]["cores"] >= 1
+    # tile census at L = 4096: 64 key tiles per query tile, 16.75 of them near on average
+    far, near = bench.tile_census([4096])
+    assert far + near == 32 * 64 and near == 536
+    tv, src = bench.measured_traffic("v3base_L4096_B8_bf16", with_source=True)
+    assert (tv is None) == (src is None)
     t = bench.measured_traffic("v3base_L4096_B8_bf16")
     assert t is None or t > 2e8
