@@ -148,7 +148,7 @@ __device__ __forceinline__ void softmax_pv(f32x16 (&sacc)[2], f32x16 (&o_acc)[D 
 #pragma unroll
     for (int e = 0; e < 8; ++e) pv[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[c >> 1][8 * (c & 1) + e], x_scale, off));
     const vfrag pf = VT::from_f32(pv);
-    l_run = VT::sum8(pf, l_run);  // the row sum is taken over the probabilities as the MFMA sees them
+    l_run = sum8(pv, l_run);
 #pragma unroll
     for (int d = 0; d < D / 32; ++d) {
       const vfrag vf = vload(c, d);
@@ -208,7 +208,7 @@ __device__ __forceinline__ void softmax_pv_pre(f32x16 (&sacc)[2], f32x16 (&o_acc
 #pragma unroll
     for (int e = 0; e < 8; ++e) pv[e] = __builtin_amdgcn_exp2f(sacc[c >> 1][8 * (c & 1) + e]);
     const vfrag pf = VT::from_f32(pv);
-    l_run = VT::sum8(pf, l_run);
+    l_run = sum8(pv, l_run);
 #pragma unroll
     for (int d = 0; d < D / 32; ++d) {
       const vfrag vf = vload(c, d);
@@ -250,7 +250,7 @@ __device__ __forceinline__ void softmax_pv_pre2(f32x16 (&sacc)[2], f32x16 (&o_ac
 #pragma unroll
       for (int e = 0; e < 8; ++e) pv[e] = __builtin_amdgcn_exp2f(sacc[c >> 1][8 * (c & 1) + e]);
       pf[c] = VT::from_f32(pv);
-      l_tile = VT::sum8(pf[c], l_tile);
+      l_tile = sum8(pv, l_tile);
     }
   };
   const bool first = m_run == -INFINITY;

@@ -41,13 +41,6 @@ struct Bf16Tr {
   }
   static __device__ __forceinline__ f32x8 to_f32(frag x) { return __builtin_convertvector(x, f32x8); }
   static __device__ __forceinline__ frag from_f32(f32x8 x) { return __builtin_convertvector(x, frag); }
-  // sum of the 8 elements (as rounded to the operand type) accumulated onto acc
-  static __device__ __forceinline__ float sum8(frag x, float acc) {
-    const bf16x2 one = {(__bf16)1.0f, (__bf16)1.0f};
-#pragma unroll
-    for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_fdot2_f32_bf16(bf16x2{x[2 * e], x[2 * e + 1]}, one, acc, false);
-    return acc;
-  }
   static __device__ __forceinline__ void store4(char* p, float a, float b, float c, float d) {
     f32x4 x = {a, b, c, d};
     *(bf16x4*)p = __builtin_convertvector(x, bf16x4);
@@ -62,6 +55,10 @@ struct Bf16Tr {
     return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pair), bf16x2{(__bf16)-0.0f, (__bf16)1.0f}, acc, false);
   }
   static __device__ __forceinline__ f32x4 load4(const char* p) { return __builtin_convertvector(*(const bf16x4*)p, f32x4); }
+  // four fp32 values rounded to the type, and one 16-bit pattern of the type back as fp32
+  using scratch4 = bf16x4;
+  static __device__ __forceinline__ scratch4 pack4(f32x4 x) { return __builtin_convertvector(x, bf16x4); }
+  static __device__ __forceinline__ float scratch_to_f32(uint16_t b) { return __builtin_bit_cast(float, (uint32_t)b << 16); }
 };
 
 struct F16Tr {
@@ -75,12 +72,6 @@ struct F16Tr {
   }
   static __device__ __forceinline__ f32x8 to_f32(frag x) { return __builtin_convertvector(x, f32x8); }
   static __device__ __forceinline__ frag from_f32(f32x8 x) { return __builtin_convertvector(x, frag); }
-  static __device__ __forceinline__ float sum8(frag x, float acc) {
-    const f16x2 one = {(_Float16)1.0f, (_Float16)1.0f};
-#pragma unroll
-    for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_fdot2(f16x2{x[2 * e], x[2 * e + 1]}, one, acc, false);
-    return acc;
-  }
   static __device__ __forceinline__ void store4(char* p, float a, float b, float c, float d) {
     f32x4 x = {a, b, c, d};
     *(f16x4*)p = __builtin_convertvector(x, f16x4);
@@ -92,6 +83,9 @@ struct F16Tr {
     return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, pair), f16x2{(_Float16)-0.0f, (_Float16)1.0f}, acc, false);
   }
   static __device__ __forceinline__ f32x4 load4(const char* p) { return __builtin_convertvector(*(const f16x4*)p, f32x4); }
+  using scratch4 = f16x4;
+  static __device__ __forceinline__ scratch4 pack4(f32x4 x) { return __builtin_convertvector(x, f16x4); }
+  static __device__ __forceinline__ float scratch_to_f32(uint16_t b) { return (float)__builtin_bit_cast(_Float16, b); }
 };
 
 struct F32Tr {
@@ -108,11 +102,6 @@ struct F32Tr {
   }
   static __device__ __forceinline__ f32x8 to_f32(frag x) { return x; }
   static __device__ __forceinline__ frag from_f32(f32x8 x) { return x; }
-  static __device__ __forceinline__ float sum8(frag x, float acc) {
-#pragma unroll
-    for (int e = 0; e < 8; ++e) acc += x[e];
-    return acc;
-  }
   static __device__ __forceinline__ void store4(char* p, float a, float b, float c, float d) {
     *(f32x4*)p = f32x4{a, b, c, d};
   }
@@ -135,6 +124,13 @@ struct Fp8Tr {  // OCP e4m3, operands of the three score products only
   static __device__ __forceinline__ float add_lo(float acc, uint32_t) { return acc; }               // unused
   static __device__ __forceinline__ float add_hi(float acc, uint32_t) { return acc; }
 };
+
+// Row-sum contribution of eight probabilities, in fp32 and before they are rounded for the MFMA: plain
+// adds.  (A 16-bit dot product per pair would halve the instruction count, but the dot instructions do not
+// run beside MFMAs of other waves, and a key tile is short of exactly that overlap: 2.5 % of the far launch.)
+__device__ __forceinline__ float sum8(const f32x8& x, float acc) {
+  return acc + (((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7])));
+}
 
 // V^T operand of a K=16 step: lane (d = l%32, g = l/32) needs V[j(g,e)][d] for
 // j(g,e) = 16*c + 8*(e/4) + 4*g + e%4 -- the key rows whose probabilities sit in this lane
@@ -312,11 +308,16 @@ __device__ __forceinline__ void dma16s(const void* base, uint32_t lane_off, uint
   asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\ts_mov_b32 m0, %0"
                : "=&s"(keep) : "v"(lane_off), "s"(sb), "s"(lb) : "memory");
 }
+// Wait until at most N vector-memory loads of this wave are outstanding (loads complete in issue
+// order).  Issued through the builtin rather than asm, so that the compiler's own count of its
+// outstanding loads takes the wait into account and it does not wait a second time for a value
+// these waits have already covered.  Encoding (gfx9): vmcnt in bits 3:0 (and 15:14), expcnt 6:4 and
+// lgkmcnt 11:8 left at their maxima (no wait).
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
-  static_assert(N == 0 || N == 4, "counts used by the kernels");
-  if constexpr (N == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  if constexpr (N == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+  static_assert(N >= 0 && N < 16, "counts used by the kernels");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | N);
+  asm volatile("" ::: "memory");
 }
 
 // Number of direct loads (dma16 / dma16s) a wave issues per K/V tile of the far-only staging: the waits

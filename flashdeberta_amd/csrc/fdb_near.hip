@@ -19,15 +19,18 @@
 //   (i, j) wants index r = i - j.  C goes through a per-wave fp32 LDS scratch and comes back as the
 //   initial value of the content product's accumulator; P is computed with the keys as MFMA rows, so
 //   its skew is a permutation of lanes within a register (ds_bpermute) and needs no scratch.
-// LDS: K 4 KB + V 4 KB + rings 40 KB + scratch 18.5 KB = 66.5 KB.
+// LDS: K 2 x 4 KB + V 2 x 4 KB + rings 2 x 24 KB + scratch 11 KB = 75 KB.
 //
-// Staging rides inside the step, between its two barriers B1 (top: K, the ring rows and V's buffer
-// are ready / free) and B2 (every wave has its operands of the step out of LDS):
-//   after B1: V(s) registers -> LDS (read by the soft-max at the end of the step), V(s+1) global -> registers;
-//   after B2: K(s+1) and batch k+5 registers -> LDS, then K(s+2), the rows of batch k+6 and the table
-//             values of batch k+7 global -> registers.
+// Staging goes global -> LDS directly (global_load_lds_dwordx4: no staging registers, no LDS write
+// instructions of the waves' own) and runs one step ahead: right after the one barrier of step s (every
+// wave is done with step s-1) a wave issues its share of K(s+1) and V(s+1) into the buffers step s does not
+// read and of the 32 rows per table that step s+1 reads for the first time into the ring's sixth batch;
+// it waits for these loads at the top of step s+1, before that step's barrier, behind which everybody's
+// have landed.  The loads have a whole step to arrive.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <utility>
 
 #include "fdb_device.h"
 #include "fdb_kernels.h"
@@ -39,24 +42,35 @@ namespace {
 
 constexpr int kNThreads = 256;
 constexpr int kStep = 32;        // keys per step
-constexpr int kRingRows = 160;   // 5 batches of 32 relative positions
-constexpr int kScrW = 36;        // fp32 words between the rows of a wave's bias scratch (rows overlap, see below)
-constexpr int kScrWords = 32 * kScrW + 32;  // row 31 reaches column 63
+constexpr int kRingBatches = 6;  // 5 batches of 32 relative positions in use by a step + the one being filled for the next
+constexpr int kRingRows = 32 * kRingBatches;
+constexpr int kScrW = 44;        // 16-bit elements between the rows of a wave's bias scratch: 36 in use; rows 8-byte aligned, and
+                                 // 22 words apart, so that the 32 rows of a write land in 64 different banks
+constexpr int kScrElems = 32 * kScrW;
 constexpr int kRowBytes = 128;   // head_dim 64, 16-bit
 
 struct NCfg {
   static constexpr int K_BYTES = kStep * kRowBytes;  // K and V rows are swizzled like the ring rows
   static constexpr int V_BYTES = kStep * kRowBytes;
   static constexpr int RING_BYTES = kRingRows * kRowBytes;
-  static constexpr int SCR_BYTES = 4 * kScrWords * 4;
+  static constexpr int SCR_BYTES = 4 * kScrElems * 2;
   static constexpr int lds_bytes(bool c2p, bool p2c) {
-    return K_BYTES + V_BYTES + (c2p ? RING_BYTES + SCR_BYTES : 0) + (p2c ? RING_BYTES : 0);
+    return 2 * K_BYTES + 2 * V_BYTES + (c2p ? RING_BYTES + SCR_BYTES : 0) + (p2c ? RING_BYTES : 0);
   }
 };
 
 // f(row) of the ring swizzle: slot (row, s) holds chunk s ^ f(row), f = 4*bit1(row) | bits3:2(row);
 // sixteen consecutive rows put one chunk in sixteen different bank groups.
 __device__ __forceinline__ int ring_f(int row) { return 4 * ((row >> 1) & 1) | ((row >> 2) & 3); }
+
+// px[v] = xs[v] of the lane (ROT0 - c(v)) places further up in this lane's half-wave (mod 32), c(v) = 8*(v/4) + 3 - v%4:
+// ds_swizzle in rotate mode, the amount in the instruction's offset field (0xC000 | amount << 5).
+template <int ROT0, int... V>
+__device__ __forceinline__ void rotate16(const float (&xs)[16], float (&px)[16], std::integer_sequence<int, V...>) {
+  ((px[V] = __builtin_bit_cast(
+        float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, xs[V]), 0xC000 | ((ROT0 - (8 * (V >> 2) + 3 - (V & 3))) << 5)))),
+   ...);
+}
 
 template <class QT, class VT, bool C2P, bool P2C>
 __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams p) {
@@ -65,9 +79,9 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
   using vfrag = typename VT::frag;
   static_assert(QT::SZ == 2 && VT::SZ == 2, "16-bit element types only");
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  char* Ks = smem;                      // [32][128]
-  char* Vs = Ks + NCfg::K_BYTES;        // [32][128]
-  char* EK = Vs + NCfg::V_BYTES;        // [160][128] rows K_r[delta(r)], slot = (r_hi0 - r) mod 160
+  char* Ks = smem;                      // [2][32][128]: step k reads buffer k & 1
+  char* Vs = Ks + 2 * NCfg::K_BYTES;    // [2][32][128], likewise
+  char* EK = Vs + 2 * NCfg::V_BYTES;    // [192][128] rows K_r[delta(r)], slot = (r_hi0 - r) mod 192
   char* EQ = EK + (C2P ? NCfg::RING_BYTES : 0);
   char* scr_raw = EQ + (P2C ? NCfg::RING_BYTES : 0);  // C's scratch (absent without the c2p term)
 
@@ -76,7 +90,7 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
   const int lane = tid & 63, li = lane & 31, g = lane >> 5;
   int xq, h;
   block_map((int)blockIdx.x, p.grid_x, p.H, p.tiles_per_seq, p.cu == nullptr, kMiddleFirst, xq, h);
-  float* scr = (float*)scr_raw + wave * kScrWords;
+  uint16_t* scr = (uint16_t*)scr_raw + wave * kScrElems;
 
   int b, m0, tok0, Lb;
   int64_t qo, ko, vo, oo;
@@ -134,23 +148,26 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
   const int n_full = p.causal ? 0 : max(0, min(n_steps, Lb / kStep - s0));  // steps k < n_full need no mask
 
   // relative positions of the workgroup at step k = s - s0: r in [r_hi0 - 32k - 158, r_hi0 - 32k];
-  // u = r_hi0 - r counts downwards from the first step's largest r; ring slot = u mod 160; batch = u / 32.
+  // u = r_hi0 - r counts downwards from the first step's largest r; ring slot = u mod 192; batch = u / 32.
   const int r_hi0 = m0 + FDB_BM - 1 - s0 * kStep;
 
   // ---- staging: one 16-byte chunk per thread of K, of V and of one batch of each ring ----------------
+  // A direct load fills 1 KB = 8 rows per wave, lane l the 16-byte slot l: thread tid owns slot scc of
+  // row srow of the 32-row tile, and since slot (row, s) holds chunk s ^ f(row), it fetches that chunk.
   const int srow = tid >> 3, scc = tid & 7;
-  const int ring_wr = srow * kRowBytes + ((scc ^ ring_f(srow)) * 16);  // within a batch's segment
-  u32x4 kreg = {0, 0, 0, 0}, vreg = {0, 0, 0, 0}, ekreg = {0, 0, 0, 0}, eqreg = {0, 0, 0, 0};
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(LDS_AS char*)smem;
+  const uint32_t wave_kb = (uint32_t)wave * 1024u;                  // this wave's 1 KB of a 32-row tile
+  const uint32_t chunk_off = (uint32_t)((scc ^ ring_f(srow)) * 16);
   int dnext = 0;
-  auto k_load = [&](int s) __attribute__((always_inline)) {
+  auto k_dma = [&](int s, int buf) __attribute__((always_inline)) {
     // LDS row srow holds key srow ^ 3 of the step (see the scratch reads below); rows past the end
     // re-read the last one, their scores are masked
     const int row = min(s * kStep + (srow ^ 3), Lb - 1);
-    kreg = *(const u32x4*)(kb + (uint64_t)(uint32_t)row * k_rsb + scc * 16);
+    dma16(kb + (uint64_t)(uint32_t)row * k_rsb + chunk_off, lds0 + buf * NCfg::K_BYTES + wave_kb);
   };
-  auto v_load = [&](int s) __attribute__((always_inline)) {
+  auto v_dma = [&](int s, int buf) __attribute__((always_inline)) {
     const int row = min(s * kStep + srow, Lb - 1);
-    vreg = *(const u32x4*)(vb + (uint64_t)(uint32_t)row * v_rsb + scc * 16);
+    dma16(vb + (uint64_t)(uint32_t)row * v_rsb + chunk_off, lds0 + 2 * NCfg::K_BYTES + buf * NCfg::V_BYTES + wave_kb);
   };
   auto batch_delta = [&](int batch) __attribute__((always_inline)) {  // table row of this thread's ring row
     const int r = r_hi0 - (batch * 32 + srow);
@@ -158,14 +175,11 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
     // has to wait for the load before the next step uses it
     return (int)((const uint16_t*)p.lut)[max(-p.R, min(p.R, r)) + p.R];
   };
-  auto batch_load = [&](int delta) __attribute__((always_inline)) {
-    if constexpr (C2P) ekreg = *(const u32x4*)(pkb + (int64_t)delta * p.pk_sr * 2 + scc * 16);
-    if constexpr (P2C) eqreg = *(const u32x4*)(pqb + (int64_t)delta * p.pq_sr * 2 + scc * 16);
-  };
-  auto batch_store = [&](int batch) __attribute__((always_inline)) {
-    const int seg = (batch % 5) * (32 * kRowBytes);
-    if constexpr (C2P) *(u32x4*)(EK + seg + ring_wr) = ekreg;
-    if constexpr (P2C) *(u32x4*)(EQ + seg + ring_wr) = eqreg;
+  const uint32_t ek_lds = lds0 + (uint32_t)(EK - smem) + wave_kb, eq_lds = lds0 + (uint32_t)(EQ - smem) + wave_kb;
+  auto batch_dma = [&](int delta, int batch) __attribute__((always_inline)) {
+    const uint32_t seg = (uint32_t)(batch % kRingBatches) * (32 * kRowBytes);
+    if constexpr (C2P) dma16(pkb + (int64_t)delta * p.pk_sr * 2 + chunk_off, ek_lds + seg);
+    if constexpr (P2C) dma16(pqb + (int64_t)delta * p.pq_sr * 2 + chunk_off, eq_lds + seg);
   };
 
   f32x16 o_acc[DBLKS];
@@ -175,34 +189,6 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
     for (int v = 0; v < 16; ++v) o_acc[d][v] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
 
-  // ---- prologue: step 0's K and ring batches 0..4 to LDS; V(0), K(1), batch 5 in the registers --------
-  // All table values first, then all rows: the loads of one kind are in flight together instead of five
-  // dependent round trips one after the other.
-  if (n_steps > 0) {
-    int d0[7];
-#pragma unroll
-    for (int bt = 0; bt < 7; ++bt) d0[bt] = batch_delta(bt);
-    k_load(s0);
-    u32x4 ek0[5], eq0[5];
-#pragma unroll
-    for (int bt = 0; bt < 5; ++bt) {
-      batch_load(d0[bt]);
-      ek0[bt] = ekreg;
-      eq0[bt] = eqreg;
-    }
-    *(u32x4*)(Ks + ring_wr) = kreg;
-#pragma unroll
-    for (int bt = 0; bt < 5; ++bt) {
-      ekreg = ek0[bt];
-      eqreg = eq0[bt];
-      batch_store(bt);
-    }
-    v_load(s0);
-    k_load(s0 + 1);
-    batch_load(d0[5]);
-    dnext = d0[6];
-  }
-
   // ---- per-lane constants ------------------------------------------------------------------------------
   // A row (block bk, lane li) of the wave's sub-tile at step k: r = iw0 - 32s - 31 + 32bk + li, i.e.
   // u = 158 + 32k - 32*(wave + bk) - li; its slot keeps the low five bits of 158 - li for ever.
@@ -210,7 +196,7 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
   uint32_t rlx[KS];  // chunk 2s + g of the row sits in slot (2s) ^ g ^ f
 #pragma unroll
   for (int s = 0; s < KS; ++s) rlx[s] = ((g ^ fr) * 16) ^ (32 * s);
-  int slot0 = (158 - li + 32 * ((5 - wave) % 5)) % kRingRows;  // block 0 at step 0 (u = 158 - li - 32*wave, mod 160)
+  int slot0 = 158 - li - 32 * wave;  // block 0 at step 0: u = 158 - li - 32*wave >= 31
   uint32_t klx[KS], vlx[4];  // K fragment rows li; V^T operand (c, d-block db, half h): row 16c + 8h + 4*(grp/2) + s16/4,
                              // 8-byte unit 8db + 4*(grp%2) + s16%4, i.e. chunk ^ f = lane part ^ (4db) ^ (2h)
   {
@@ -223,27 +209,22 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
       vlx[x] = vlane ^ (64 * (x >> 1) ^ 32 * (x & 1));
     }
   }
-  // scratch (fp32, so no conversion and no sub-word extraction): C[i = li][rr] with rr = r - r_lo in
-  // 0..63; element (jj = 8q + 4g + e, i = li) reads C[li][li + 31 - jj].  Only a band of 32 columns of
-  // each row is ever read (rr in [li, li + 31]), so the rows are laid 36 words apart and overlap: the
-  // bands (plus the three columns a four-column group may stick out on either side) stay disjoint, and
-  // a lane does not write the groups of its row that lie wholly outside the band.
+  // scratch: C[i = li][rr] with rr = r - r_lo in 0..63; element (jj, i = li) wants C[li][li + 31 - jj], i.e. only the
+  // band rr in [li, li + 31] of row li is ever read.  Of the two columns rr = c and c + 32 (the same accumulator
+  // register of block 0 and of block 1) a lane therefore needs exactly one, c if c >= li: it picks that one
+  // (the lanes that pick block 0 are a constant of the register: a scalar mask), rounds to the 16-bit type and
+  // writes 32 columns, position rr mod 32, as four 8-byte groups instead of 64 columns in fp32 -- LDS writes are
+  // what a step pays most for.  Positions 32..35 repeat 0..3, so that a run of four positions never wraps.
   // K's rows sit in LDS with the low two bits of the row index inverted, so MFMA row m = 8q + 4g + e of
   // the content product is key jj = 8q + 4g + 3 - e: the four C elements a lane adds to consecutive
-  // accumulator registers then lie at ascending addresses and can be read in pairs straight into the
-  // accumulator's registers.
-  float* c_wrp = scr + li * kScrW + 4 * g;  // row = this lane's MFMA column; group (bk, q4) at + 32 bk + 8 q4
-  bool c_wr[2][4];
+  // accumulator registers are the run of positions that starts at (li + 28 - 8q - 4g) mod 32.
+  uint16_t* c_wrp = scr + li * kScrW + 4 * g;  // row = this lane's MFMA column; group q4 at + 8 q4
+  // (read through volatile pointers: four neighbouring 16-bit reads must stay four instructions -- fused into
+  // one 8-byte read at an address aligned to two bytes only, they would be served lane by lane)
+  LDS_AS const volatile uint16_t* c_rd[4];
 #pragma unroll
-  for (int q4 = 0; q4 < 4; ++q4) {
-    const int m = 8 * q4 + 4 * g;  // first column of the group within its block
-    c_wr[0][q4] = m + 3 >= li;
-    c_wr[1][q4] = m + 1 <= li;
-  }
-  LDS_AS const float* c_rd = (LDS_AS const float*)(scr + (kScrW + 1) * li + 4 - 4 * g);   // register 4q + e at + 8 (3 - q) + e
-  asm volatile("" : "+v"(c_rd));  // opaque base: the reads keep small immediate offsets
-  // P's lane permutation: register v (key jj = 4g + c) of lane (g, li) comes from lane (g, (li + 31 - jj) mod 32)
-  const int p_nj = li + 4 * g, p_src = 4 * (li + 31 - 4 * g), p_half = 128 * g;
+  for (int q = 0; q < 4; ++q)
+    c_rd[q] = (LDS_AS const volatile uint16_t*)(scr + li * kScrW + ((li + 28 - 8 * q - 4 * g) & 31));
 
   // Block 1 of a step holds the rows that were block 0 of the step before, and a step reads only its
   // new block 0 from the rings.  C[r][i] does not depend on the keys, so C's block 1 IS the block 0 the
@@ -259,7 +240,22 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
       if constexpr (P2C) aq[buf][x] = QT::load(EQ + slot * kRowBytes + rlx[x]);
     }
   };
+  // ---- prologue: step 0's K and ring batches 0..4 on their way to LDS -------------------------------------
+  // All table values first, then all rows: the loads of one kind are in flight together.
   if (n_steps > 0) {
+    int d0[6];
+#pragma unroll
+    for (int bt = 0; bt < 6; ++bt) d0[bt] = batch_delta(bt);
+    // (taken here: the compiler, which does not count the direct loads, would otherwise wait for each
+    // value at its use, behind all the direct loads issued before it)
+#pragma unroll
+    for (int bt = 0; bt < 6; ++bt) asm volatile("" : "+v"(d0[bt]));
+    k_dma(s0, 0);
+    v_dma(s0, 0);
+#pragma unroll
+    for (int bt = 0; bt < 5; ++bt) batch_dma(d0[bt], bt);
+    dnext = d0[5];
+    wait_vmcnt<0>();
     __syncthreads();  // the prologue's ring rows
     ring_read(1, slot0 >= 32 ? slot0 - 32 : slot0 + (kRingRows - 32));  // block 1 of step 0
     if constexpr (C2P) {
@@ -279,16 +275,26 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
     constexpr int PAR = decltype(par_tag)::value;  // buffer of this step's block 0
     const int s = s0 + k;
     const int j0 = s * kStep;
-    __syncthreads();  // B1
+    // This wave's direct loads of the step before -- K, V and the new ring batch of this step -- have landed;
+    // behind the barrier everyone's have, and every wave is done with the buffers the loads below overwrite.
+    wait_vmcnt<0>();
+    // The table value fetched a step ago is among the loads just waited for; taking it here keeps the compiler,
+    // which does not count the direct loads, from waiting for it further down, behind this step's direct loads.
+    asm volatile("" : "+v"(dnext));
+    __syncthreads();
+    // ---- staging for the next step, straight into LDS ----------------------------------------------------------
+    // It runs unconditionally, past the last step too (row and table indices are clamped, and nobody reads
+    // what the last steps fetch), so every step issues the same loads and the one wait above covers them.
+    k_dma(s + 1, PAR ^ 1);
+    v_dma(s + 1, PAR ^ 1);
+    batch_dma(dnext, k + 5);
+    __builtin_amdgcn_sched_barrier(0);  // the table load stays behind the direct loads
+    dnext = batch_delta(k + 6);         // used a step from now
     // ---- operands of the step out of LDS ------------------------------------------------------------------
     qfrag kf[KS];
 #pragma unroll
-    for (int x = 0; x < KS; ++x) kf[x] = QT::load(Ks + klx[x]);
+    for (int x = 0; x < KS; ++x) kf[x] = QT::load(Ks + PAR * NCfg::K_BYTES + klx[x]);
     ring_read(PAR, slot0);
-    // V of this step to LDS, V of the next one on its way
-    *(u32x4*)(Vs + ring_wr) = vreg;
-    __builtin_amdgcn_sched_barrier(0);
-    v_load(s + 1);
     // ---- the five products -------------------------------------------------------------------------------
     // C, C to the scratch and its skewed diagonal back as the initial value of the content product's
     // accumulator; P runs while those reads are in flight (the scheduling fence keeps it behind them).
@@ -303,16 +309,22 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
       for (int x = 0; x < KS; ++x) ckeep[PAR] = QT::mma(ac[x], qf[x], x == 0 ? zero : ckeep[PAR]);
       const f32x16(&cacc)[2] = ckeep;  // block bk of this step sits in ckeep[PAR ^ bk]
 #pragma unroll
-      for (int bk = 0; bk < 2; ++bk)
+      for (int q4 = 0; q4 < 4; ++q4) {  // C[i = li][(32*bk) + 8*q4 + 4*g + 0..3], block 0 where that column is >= li
+        f32x4 pick;
 #pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4)  // C[i = li][32*bk + 8*q4 + 4*g + 0..3]
-          if (__builtin_expect(c_wr[bk][q4], 1))
-            *(f32x4*)(c_wrp + 32 * bk + 8 * q4) =
-                f32x4{cacc[PAR ^ bk][4 * q4], cacc[PAR ^ bk][4 * q4 + 1], cacc[PAR ^ bk][4 * q4 + 2],
-                      cacc[PAR ^ bk][4 * q4 + 3]};
+        for (int e = 0; e < 4; ++e) {
+          const int c0 = 8 * q4 + e, c1 = c0 + 4;  // the column in the lanes g = 0 / g = 1
+          const uint64_t mask = ((2ull << c0) - 1ull) | ((c1 >= 31 ? 0xffffffffull : (2ull << c1) - 1ull) << 32);
+          pick[e] = __builtin_amdgcn_inverse_ballot_w64(mask) ? cacc[PAR][4 * q4 + e] : cacc[PAR ^ 1][4 * q4 + e];
+        }
+        const typename QT::scratch4 packed = QT::pack4(pick);
+        *(typename QT::scratch4*)(c_wrp + 8 * q4) = packed;
+        if (q4 == 0) *(typename QT::scratch4*)(c_wrp + 32) = packed;
+      }
       wave_lds_fence();
 #pragma unroll
-      for (int v = 0; v < 16; ++v) sacc[v] = c_rd[8 * (3 - (v >> 2)) + (v & 3)];
+      for (int v = 0; v < 16; ++v)
+        sacc[v] = QT::scratch_to_f32(c_rd[v >> 2][v & 3]);
       wave_lds_fence();
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -332,28 +344,24 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
     for (int x = 0; x < KS; ++x) sacc = QT::mma(kf[x], qf[x], sacc);
     float px[16];
     if constexpr (P2C) {
-      int nj = p_nj, src = p_src;
-      asm volatile("" : "+v"(nj), "+v"(src));  // per-register masks and addresses are made here, not kept
+      // Source lane (g, n) of register v (key jj = 4g + c) is read by lane (g, (n - rot) mod 32), which wants
+      // block 1 from it if n + jj < 31 and block 0 otherwise: which lanes pick block 1 is a constant of the
+      // register, so the select takes its mask from a scalar pair.  The move itself is a rotation of each
+      // half-wave by a constant, rot = 31 - jj: ds_swizzle in rotate mode (offset 0xC000 | rot << 5), no
+      // address registers; the halves differ by 4 in jj, so each half runs its own sixteen under its
+      // half of the execution mask.
+      float xs[16];
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int c = 8 * (v >> 2) + 3 - (v & 3);  // jj - 4g
-        const float x = (nj + c < 31) ? pacc[1][v] : pacc[0][v];
-        const int addr = ((src - 4 * c) & 124) | p_half;
-        px[v] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(addr, __builtin_bit_cast(int, x)));
+        const uint64_t mask = (uint64_t)((1u << (31 - c)) - 1u) | ((uint64_t)(c < 27 ? (1u << (27 - c)) - 1u : 0u) << 32);
+        xs[v] = __builtin_amdgcn_inverse_ballot_w64(mask) ? pacc[1][v] : pacc[0][v];
       }
+      if (g == 0)
+        rotate16<31>(xs, px, std::make_integer_sequence<int, 16>{});
+      else
+        rotate16<27>(xs, px, std::make_integer_sequence<int, 16>{});
     }
-    // ---- B2: nobody reads K or the ring of this step from LDS any more --------------------------------------
-    __syncthreads();
-    // The staging runs unconditionally, past the last step too (row and table indices are clamped, and
-    // nobody reads what the last steps store): with a fixed sequence of loads the compiler waits at each
-    // use for exactly the loads that are older, instead of for every outstanding one.
-    *(u32x4*)(Ks + ring_wr) = kreg;
-    batch_store(k + 5);
-    __builtin_amdgcn_sched_barrier(0);  // the loads below reuse the registers just stored
-    const int dnew = batch_delta(k + 7);  // first: whatever consumes it waits for this load alone
-    batch_load(dnext);                    // its table value was loaded a step ago
-    k_load(s + 2);
-    dnext = dnew;
     if constexpr (P2C) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) sacc[v] += px[v];
@@ -381,7 +389,7 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
         for (int e = 0; e < 8; ++e)  // the V^T operand takes the keys in ascending order
           pv[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[8 * c + (e ^ 3)], x_scale, off));
         pf[c] = VT::from_f32(pv);
-        l_blk = VT::sum8(pf[c], l_blk);
+        l_blk = sum8(pv, l_blk);
       }
     };
     bool slow = __any(m_run == -INFINITY);
@@ -411,8 +419,8 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
     for (int c = 0; c < 2; ++c)
 #pragma unroll
       for (int d = 0; d < DBLKS; ++d) {
-        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(Vs + vlx[2 * d] + 2048 * c));
-        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(Vs + vlx[2 * d + 1] + 2048 * c + 1024));
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(Vs + PAR * NCfg::V_BYTES + vlx[2 * d] + 2048 * c));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(Vs + PAR * NCfg::V_BYTES + vlx[2 * d + 1] + 2048 * c + 1024));
         const vfrag vf = __builtin_bit_cast(vfrag, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
         o_acc[d] = VT::mma(vf, pf[c], o_acc[d]);
       }
@@ -442,6 +450,7 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
     }
     if (k < n_steps) step(std::true_type{}, T0{}, k);
   }
+  wait_vmcnt<0>();  // the last step's direct loads: none may still be writing LDS when the workgroup ends
 
   // ---- epilogue: merge with the far tiles' partial result, normalise, store ------------------------------
   const float l_tot = wave_half_sum(l_run);
