@@ -1,4 +1,4 @@
-"""CPU oracle for the DeBERTa-v2/v3 disentangled-attention forward.  TEST INFRASTRUCTURE ONLY.
+"""CPU oracle for the DeBERTa-v2/v3 disentangled attention (forward and backward).  TEST INFRASTRUCTURE ONLY.
 
 This file is the checker, never the product: only tests/, __graft_entry__.smoke() and the
 cpu_baseline leg of bench.py may import it.  The shipped path (flashdeberta_amd) never does and
@@ -17,6 +17,9 @@ Pinning (what fixes each function besides re-reading it; the tests are in tests/
   disentangled_attention : content-only case == torch scaled_dot_product_attention; a triple-loop
         fp64 brute force on tiny inputs; row/column-constant bias invariants; golden fixtures.
   module_forward         : golden fixtures (hidden states -> context) from the third-party class.
+  disentangled_attention_backward : central finite differences of disentangled_attention on tiny inputs
+        (every operand, both position terms, masked and causal); the golden gradient fixtures, which
+        autograd wrote through the third-party class (hidden states, relative embeddings, every weight).
   quantize_e4m3_per_head : torch.float8_e4m3fn round trip (library routine).
   fp8 attention          : no reference counterpart exists; "parity unpinned" beyond the
         de-quantised-input restatement and the bound against the unquantised result.
@@ -122,6 +125,62 @@ def disentangled_attention(q, k, v, pos_key=None, pos_query=None, position_bucke
             out[b, h] = p @ v[b, h]
             lse[b, h] = l
     return (out, lse) if return_lse else out
+
+
+def disentangled_attention_backward(q, k, v, dout, pos_key=None, pos_query=None, position_buckets=-1,
+                                    max_relative_positions=-1, mask=None, causal=False, dtype=np.float64):
+    """Gradients of sum(disentangled_attention(...) * dout) with respect to q, k, v [B, H, L, D] and
+    pos_key, pos_query [H, 2S, D]: the chain rule through the eager graph (HF:236-271 for scores,
+    soft-max and PV; HF:315-324 and HF:327-343 for the two gathers, whose adjoint is a scatter-add
+    into the [L, 2S] position scores).  The reference's counterpart are its three backward kernels
+    (REF: src/flashdeberta/ops/flash_attention.py:62-141, 581-941), which leave the gradient of the
+    [B, H, L, 2S] bias tensors to autograd; here the chain is carried through to K_r / Q_r.
+    Rows of `dout` that belong to padded queries must be zero (the module never produces them)."""
+    q, k, v, dout = [np.asarray(x, dtype=dtype) for x in (q, k, v, dout)]
+    B, H, L, D = q.shape
+    scale_factor = 1 + (pos_key is not None) + (pos_query is not None)
+    scale = dtype(math.sqrt(D * scale_factor))
+    span = att_span_of(position_buckets, max_relative_positions)
+    if pos_key is not None or pos_query is not None:
+        rel = build_relative_position(L, L, position_buckets, max_relative_positions)
+        c2p_pos = np.clip(rel + span, 0, 2 * span - 1)
+        p2c_pos = np.clip(-rel + span, 0, 2 * span - 1)
+    dq, dk, dv = np.zeros_like(q), np.zeros_like(k), np.zeros_like(v)
+    dpk = None if pos_key is None else np.zeros(np.asarray(pos_key).shape, dtype=dtype)
+    dpq = None if pos_query is None else np.zeros(np.asarray(pos_query).shape, dtype=dtype)
+    neg = np.finfo(dtype).min
+    rows = np.arange(L)[:, None]
+    for b in range(B):
+        for h in range(H):
+            s = q[b, h] @ (k[b, h].T / scale)
+            if pos_key is not None:
+                pk = np.asarray(pos_key[h], dtype=dtype)
+                s = s + np.take_along_axis(q[b, h] @ pk.T, c2p_pos, axis=-1) / scale
+            if pos_query is not None:
+                pq = np.asarray(pos_query[h], dtype=dtype)
+                s = s + np.take_along_axis(k[b, h] @ pq.T, p2c_pos, axis=-1).T / scale
+            if mask is not None:
+                s = np.where(np.asarray(mask[b], dtype=bool)[None, :], s, neg)
+            if causal:
+                s = np.where(np.tril(np.ones((L, L), dtype=bool)), s, neg)
+            p, _ = _softmax_lastdim(s)
+            do = dout[b, h]
+            dv[b, h] = p.T @ do
+            dp = do @ v[b, h].T
+            ds = p * (dp - (p * dp).sum(axis=-1, keepdims=True)) / scale  # w.r.t. the raw score sums
+            dq[b, h] = ds @ k[b, h]
+            dk[b, h] = ds.T @ q[b, h]
+            if pos_key is not None:
+                g = np.zeros((L, 2 * span), dtype=dtype)  # d(q K_r^T)[i, delta]
+                np.add.at(g, (rows, c2p_pos), ds)
+                dq[b, h] += g @ pk[:2 * span]
+                dpk[h, :2 * span] += g.T @ q[b, h]
+            if pos_query is not None:
+                g = np.zeros((L, 2 * span), dtype=dtype)  # d(k Q_r^T)[j, delta]: element (i, j) read [j, p2c_pos[j, i]]
+                np.add.at(g, (rows, p2c_pos), ds.T)
+                dk[b, h] += g @ pq[:2 * span]
+                dpq[h, :2 * span] += g.T @ k[b, h]
+    return dq, dk, dv, dpk, dpq
 
 
 def disentangled_attention_varlen(q, k, v, cu_seqlens, pos_key=None, pos_query=None, position_buckets=-1,

@@ -5,7 +5,8 @@ The eager side of the reference's switch is transformers' DisentangledSelfAttent
 (transformers 5.15.0), built from a plain config object the way the reference's own test does
 (tests/attention.py:6-18,52).  This script runs that class on CPU in fp32 with seeded inputs and
 stores inputs, weights and outputs, plus the relative-position ids of
-transformers' build_relative_position.  Run from the repo root:  python tests/golden/make_golden.py
+transformers' build_relative_position, and for the g_* cases the gradients torch.autograd computes
+through the class for a seeded upstream gradient (hidden states, relative embeddings, every weight).  Run from the repo root:  python tests/golden/make_golden.py
 """
 import os
 
@@ -41,7 +42,45 @@ CASES = {
 }
 
 
+GRAD_CASES = {
+    # name: (B, L, hidden, heads, buckets, max_rel, pos_att_type, share_att_key, lengths or None)
+    "g_L48_b8_share": (2, 48, 64, 2, 8, 16, ["c2p", "p2c"], True, None),
+    "g_L150_b32_masked": (2, 150, 128, 2, 32, 64, ["c2p", "p2c"], False, [150, 101]),
+    "g_L40_b8_c2p": (1, 40, 64, 2, 8, 16, ["c2p"], False, None),
+}
+
+
+def grad_cases():
+    for idx, (name, (B, L, hid, H, pb, mr, pat, share, lens)) in enumerate(GRAD_CASES.items()):
+        torch.manual_seed(2000 + idx)
+        mod = DisentangledSelfAttention(Cfg(hid, H, pb, mr, pat, share)).eval()
+        with torch.no_grad():
+            for p in mod.parameters():
+                p.normal_(0.0, 0.2)
+        hidden = torch.randn(B, L, hid, requires_grad=True)
+        rel = torch.randn(2 * pb, hid, requires_grad=True)
+        mask2d = torch.ones(B, L)
+        if lens is not None:
+            for b, n in enumerate(lens):
+                mask2d[b, n:] = 0
+        ext = mask2d.unsqueeze(1).unsqueeze(2)
+        ext = ext * ext.squeeze(-2).unsqueeze(-1)
+        out = mod(hidden, ext, rel_embeddings=rel)[0]
+        gout = torch.randn_like(out) * mask2d[:, :, None]  # nothing flows back from padded rows
+        (out * gout).sum().backward()
+        data = {"hidden": hidden.detach().numpy(), "rel_embeddings": rel.detach().numpy(),
+                "mask": mask2d.numpy().astype(np.uint8), "out": out.detach().numpy(), "gout": gout.numpy(),
+                "g.hidden": hidden.grad.numpy(), "g.rel_embeddings": rel.grad.numpy(),
+                "meta": np.array([B, L, hid, H, pb, mr, int("c2p" in pat), int("p2c" in pat), int(share)], dtype=np.int64)}
+        for k, v in mod.named_parameters():
+            data["w." + k] = v.detach().numpy()
+            data["g.w." + k] = (v.grad if v.grad is not None else torch.zeros_like(v)).numpy()
+        np.savez_compressed(os.path.join(HERE, name + ".npz"), **data)
+        print(name, out.shape, float(hidden.grad.abs().max()))
+
+
 def main():
+    grad_cases()
     for idx, (name, (B, L, hid, H, pb, mr, pat, share, lens, scale)) in enumerate(CASES.items()):
         torch.manual_seed(1000 + idx)
         cfg = Cfg(hid, H, pb, mr, pat, share)

@@ -148,6 +148,90 @@ def test_module_forward_matches_golden(path):
     assert err < 2e-4 * max(1.0, np.abs(ref).max()), err  # the stored vectors are fp32 eager outputs
 
 
+# ---- backward -----------------------------------------------------------------------------------
+@pytest.mark.parametrize("kw", [{}, {"masked": True}, {"causal": True}], ids=["plain", "masked", "causal"])
+@pytest.mark.parametrize("terms", [(True, True), (True, False), (False, True), (False, False)], ids=["c2p+p2c", "c2p", "p2c", "content"])
+def test_backward_matches_finite_differences(kw, terms):
+    """Central differences of the forward oracle, entry by entry, against the analytic gradients (every operand)."""
+    rng = np.random.default_rng(50)
+    B, H, L, D, pb, mr = 1, 2, 21, 8, 4, 8  # radius 8: linear zone, log zone and both saturated ends inside 21 tokens
+    q, k, v, do = [rng.standard_normal((B, H, L, D)) for _ in range(4)]
+    pk = rng.standard_normal((H, 2 * pb, D)) if terms[0] else None
+    pq = rng.standard_normal((H, 2 * pb, D)) if terms[1] else None
+    fkw = {}
+    if kw.get("masked"):
+        fkw["mask"] = np.arange(L)[None, :] < 17
+        do[:, :, 17:] = 0
+    if kw.get("causal"):
+        fkw["causal"] = True
+    grads = O.disentangled_attention_backward(q, k, v, do, pk, pq, pb, mr, **fkw)
+    f = lambda: (O.disentangled_attention(q, k, v, pk, pq, pb, mr, **fkw) * do).sum()
+    for x, g in zip((q, k, v, pk, pq), grads):
+        if x is None:
+            assert g is None
+            continue
+        for _ in range(25):
+            idx = tuple(rng.integers(0, n) for n in x.shape)
+            old, e = x[idx], 1e-5
+            x[idx] = old + e
+            fp = f()
+            x[idx] = old - e
+            fm = f()
+            x[idx] = old
+            assert abs((fp - fm) / (2 * e) - g[idx]) < 1e-7, (idx, (fp - fm) / (2 * e), g[idx])
+
+
+class _OracleAttention(torch.autograd.Function):
+    """The numpy oracle (forward and backward) as an autograd node, so that torch carries the chain through
+    the projections around it."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, pk, pq, pb, mr, mask):
+        n = lambda x: None if x is None else x.detach().numpy().astype(np.float64)
+        ctx.save_for_backward(q, k, v, *(x for x in (pk, pq) if x is not None))
+        ctx.cfg = (pk is not None, pq is not None, pb, mr, mask)
+        return torch.from_numpy(O.disentangled_attention(n(q), n(k), n(v), n(pk), n(pq), pb, mr, mask=mask))
+
+    @staticmethod
+    def backward(ctx, dout):
+        has_pk, has_pq, pb, mr, mask = ctx.cfg
+        saved = [x.numpy().astype(np.float64) for x in ctx.saved_tensors]
+        q, k, v = saved[:3]
+        pk = saved[3] if has_pk else None
+        pq = saved[3 + has_pk] if has_pq else None
+        g = O.disentangled_attention_backward(q, k, v, dout.numpy(), pk, pq, pb, mr, mask=mask)
+        t = lambda x: None if x is None else torch.from_numpy(x)
+        return t(g[0]), t(g[1]), t(g[2]), t(g[3]), t(g[4]), None, None, None
+
+
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "g_*.npz"))))
+def test_backward_matches_golden_gradients(path):
+    """Gradients torch.autograd wrote through the third-party eager class (hidden states, relative embeddings,
+    every weight) against the oracle's backward, with torch carrying the chain through the projections."""
+    g = np.load(path)
+    B, L, hid, H, pb, mr, c2p, p2c, share = g["meta"].tolist()
+    D = hid // H
+    W = {k[2:]: torch.tensor(g[k], dtype=torch.float64, requires_grad=True) for k in g.files if k.startswith("w.")}
+    hidden = torch.tensor(g["hidden"], dtype=torch.float64, requires_grad=True)
+    rel = torch.tensor(g["rel_embeddings"], dtype=torch.float64, requires_grad=True)
+    lin = lambda x, n: torch.nn.functional.linear(x, W[n + ".weight"], W.get(n + ".bias"))
+    heads = lambda x: x.view(*x.shape[:-1], H, D).transpose(-2, -3)  # [..., L, H*D] -> [..., H, L, D]
+    q, k, v = heads(lin(hidden, "query_proj")), heads(lin(hidden, "key_proj")), heads(lin(hidden, "value_proj"))
+    pk = heads(lin(rel, "key_proj" if share else "pos_key_proj")) if c2p else None
+    pq = heads(lin(rel, "query_proj" if share else "pos_query_proj")) if p2c else None
+    mask = g["mask"].astype(bool)
+    out = _OracleAttention.apply(q, k, v, pk, pq, pb, mr, None if mask.all() else mask)
+    out = out.transpose(1, 2).reshape(B, L, hid)
+    assert np.abs(np.where(mask[:, :, None], out.detach().numpy() - g["out"], 0)).max() < 2e-4 * max(1.0, np.abs(g["out"]).max())
+    (out * torch.from_numpy(g["gout"].astype(np.float64))).sum().backward()
+    got = {"hidden": hidden.grad, "rel_embeddings": rel.grad, **{"w." + n: t.grad for n, t in W.items()}}
+    for name, t in got.items():
+        ref = g["g." + name]
+        val = np.zeros_like(ref) if t is None else t.numpy()
+        err = np.abs(val - ref).max()
+        assert err < 2e-4 * max(1.0, np.abs(ref).max()), (name, err, np.abs(ref).max())  # fp32 autograd vs fp64
+
+
 # ---- fp8 ---------------------------------------------------------------------------------------
 def test_e4m3_round_matches_torch():
     x = np.concatenate([_rand(20000, 30, 100.0), _rand(20000, 31, 1.0), _rand(20000, 32, 0.01),
