@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(_HERE, "libfdb_hip.so")
 
 FDB_F32, FDB_BF16, FDB_F16, FDB_FP8_E4M3 = 0, 1, 2, 3
 FDB_NOALLOC_SCRATCH_BYTES = 32 * 1024 * 1024
-FDB_VERSION = 4  # of include/fdb.h as mirrored below
+FDB_VERSION = 5  # of include/fdb.h as mirrored below
 
 
 class FdbAttnArgs(ctypes.Structure):
@@ -32,8 +32,19 @@ class FdbAttnArgs(ctypes.Structure):
     )
 
 
+class FdbAttnBwdArgs(ctypes.Structure):
+    _fields_ = (
+        [(n, ctypes.c_void_p) for n in (
+            "q", "k", "v", "dout", "dq", "dk", "dv", "lse", "delta", "c2p_bias", "p2c_bias", "d_c2p_bias", "d_p2c_bias",
+            "seq_start", "seq_len", "delta_lut")]
+        + [(n + s, ctypes.c_int64) for n in ("q", "k", "v", "do", "dq", "dk", "dv") for s in ("_stride_b", "_stride_t", "_stride_h")]
+        + [(n, ctypes.c_int32) for n in ("batch", "heads", "head_dim", "seqlen", "att_span", "lut_radius", "dtype", "causal")]
+        + [("sm_scale", ctypes.c_float)]
+    )
+
+
 EXPORTS = (
-    "fdb_version", "fdb_attn_args_size", "fdb_strerror", "fdb_attn_check", "fdb_attn_fwd", "fdb_attn_fwd_noalloc", "fdb_attn_workspace_bytes",
+    "fdb_version", "fdb_attn_args_size", "fdb_strerror", "fdb_attn_check", "fdb_attn_fwd", "fdb_attn_fwd_noalloc", "fdb_attn_bwd", "fdb_attn_bwd_args_size", "fdb_attn_workspace_bytes",
     "fdb_worklist_ints",
     "fdb_worklist_max_tiles", "fdb_tile_rows", "fdb_build_worklist", "fdb_delta_lut_radius", "fdb_delta_lut",
     "fdb_quant_e4m3_per_head", "fdb_dequant_e4m3_per_head",
@@ -63,6 +74,12 @@ def _load():
     lib.fdb_attn_fwd.argtypes = [ctypes.POINTER(FdbAttnArgs), vp]
     lib.fdb_attn_fwd_noalloc.restype = ctypes.c_int
     lib.fdb_attn_fwd_noalloc.argtypes = [ctypes.POINTER(FdbAttnArgs), vp]
+    lib.fdb_attn_bwd_args_size.restype = ctypes.c_size_t
+    if lib.fdb_attn_bwd_args_size() != ctypes.sizeof(FdbAttnBwdArgs):
+        raise ImportError("flashdeberta_amd: %s was built from a different include/fdb.h (backward struct size %d, binding %d); "
+                          "rebuild it" % (LIB_PATH, lib.fdb_attn_bwd_args_size(), ctypes.sizeof(FdbAttnBwdArgs)))
+    lib.fdb_attn_bwd.restype = ctypes.c_int
+    lib.fdb_attn_bwd.argtypes = [ctypes.POINTER(FdbAttnBwdArgs), vp]
     lib.fdb_attn_workspace_bytes.restype = i64
     lib.fdb_attn_workspace_bytes.argtypes = [ctypes.POINTER(FdbAttnArgs)]
     lib.fdb_worklist_ints.restype = i64

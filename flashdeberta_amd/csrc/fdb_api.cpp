@@ -377,6 +377,50 @@ int fdb_attn_fwd_noalloc(const fdb_attn_args* a, void* stream) {
   return fdb_attn_fwd(&b, stream);
 }
 
+size_t fdb_attn_bwd_args_size(void) { return sizeof(fdb_attn_bwd_args); }
+
+int fdb_attn_bwd(const fdb_attn_bwd_args* a, void* stream) {
+  if (!a) return FDB_ERR_NULL;
+  if (!a->q || !a->k || !a->v || !a->dout || !a->dq || !a->dk || !a->dv || !a->lse || !a->delta) return FDB_ERR_NULL;
+  if (a->dtype != FDB_F32 && a->dtype != FDB_BF16 && a->dtype != FDB_F16) return FDB_ERR_DTYPE;
+  if (a->head_dim != 32 && a->head_dim != 64 && a->head_dim != 128) return FDB_ERR_HEAD_DIM;
+  if (a->batch < 1 || a->heads < 1 || a->heads > 65535 || a->batch > 65535 || a->seqlen < 1) return FDB_ERR_SHAPE;
+  const bool has_pos = a->c2p_bias || a->p2c_bias;
+  if ((a->c2p_bias && !a->d_c2p_bias) || (a->p2c_bias && !a->d_p2c_bias)) return FDB_ERR_NULL;
+  if (has_pos && (a->att_span < 1 || a->lut_radius < 1 || !a->delta_lut)) return FDB_ERR_SPAN;
+  const int sz = qk_elem_size(a->dtype);
+  const void* ptrs[] = {a->q, a->k, a->v, a->dout, a->dq, a->dk, a->dv};
+  for (const void* ptr : ptrs)
+    if (!aligned16(ptr)) return FDB_ERR_ALIGN;
+  const int64_t strides[] = {a->q_stride_b, a->q_stride_t, a->q_stride_h, a->k_stride_b, a->k_stride_t, a->k_stride_h,
+                             a->v_stride_b, a->v_stride_t, a->v_stride_h, a->do_stride_b, a->do_stride_t, a->do_stride_h,
+                             a->dq_stride_b, a->dq_stride_t, a->dq_stride_h, a->dk_stride_b, a->dk_stride_t, a->dk_stride_h,
+                             a->dv_stride_b, a->dv_stride_t, a->dv_stride_h};
+  for (int64_t st : strides)
+    if ((st * sz) % 16 != 0) return FDB_ERR_ALIGN;
+  FdbBwdParams p;
+  memset(&p, 0, sizeof(p));
+  p.q = (const char*)a->q; p.k = (const char*)a->k; p.v = (const char*)a->v; p.dout = (const char*)a->dout;
+  p.dq = (char*)a->dq; p.dk = (char*)a->dk; p.dv = (char*)a->dv;
+  p.lse = a->lse; p.delta = a->delta;
+  p.c2p = a->c2p_bias; p.p2c = a->p2c_bias; p.d_c2p = a->d_c2p_bias; p.d_p2c = a->d_p2c_bias;
+  p.seq_start = a->seq_start; p.seq_len = a->seq_len; p.lut = a->delta_lut;
+  p.q_sb = a->q_stride_b; p.q_st = a->q_stride_t; p.q_sh = a->q_stride_h;
+  p.k_sb = a->k_stride_b; p.k_st = a->k_stride_t; p.k_sh = a->k_stride_h;
+  p.v_sb = a->v_stride_b; p.v_st = a->v_stride_t; p.v_sh = a->v_stride_h;
+  p.g_sb = a->do_stride_b; p.g_st = a->do_stride_t; p.g_sh = a->do_stride_h;
+  p.dq_sb = a->dq_stride_b; p.dq_st = a->dq_stride_t; p.dq_sh = a->dq_stride_h;
+  p.dk_sb = a->dk_stride_b; p.dk_st = a->dk_stride_t; p.dk_sh = a->dk_stride_h;
+  p.dv_sb = a->dv_stride_b; p.dv_st = a->dv_stride_t; p.dv_sh = a->dv_stride_h;
+  p.B = a->batch; p.H = a->heads; p.L = a->seqlen;
+  p.S = has_pos ? a->att_span : 0;
+  p.R = has_pos ? a->lut_radius : 1;
+  p.causal = a->causal ? 1 : 0;
+  p.sm_scale = a->sm_scale;
+  p.scale_log2 = a->sm_scale * 1.4426950408889634f;
+  return fdb_launch_bwd(p, a->dtype, a->head_dim, stream);
+}
+
 int fdb_build_worklist(const int32_t* cu_seqlens, int32_t batch, int32_t total_tokens, int32_t* worklist,
                        void* stream) {
   if (!cu_seqlens || !worklist) return FDB_ERR_NULL;

@@ -45,6 +45,41 @@ struct FdbKParams {
   float scale_log2; // sm_scale * log2(e)
 };
 
+// Backward launch (fdb_bwd.hip): fixed layout only.  Position scores and their gradients are fp32
+// [B, L, H, 2S] (token-major like lse); lse / delta are fp32 [B*L, H].
+struct FdbBwdParams {
+  const char* q;
+  const char* k;
+  const char* v;
+  const char* dout;
+  char* dq;
+  char* dk;
+  char* dv;
+  const float* lse;
+  const float* delta;   // sum_d dO * O per row
+  const float* c2p;     // q_i . K_r[delta] or NULL
+  const float* p2c;     // k_j . Q_r[delta] or NULL
+  float* d_c2p;         // zero-initialised by the caller; scatter-added
+  float* d_p2c;
+  const int32_t* seq_start;
+  const int32_t* seq_len;
+  const int16_t* lut;
+  int64_t q_sb, q_st, q_sh;
+  int64_t k_sb, k_st, k_sh;
+  int64_t v_sb, v_st, v_sh;
+  int64_t g_sb, g_st, g_sh;     // dout
+  int64_t dq_sb, dq_st, dq_sh;
+  int64_t dk_sb, dk_st, dk_sh;
+  int64_t dv_sb, dv_st, dv_sh;
+  int32_t B, H, L;
+  int32_t S;        // att_span
+  int32_t R;        // table radius
+  int32_t causal;
+  float scale_log2; // sm_scale * log2(e)
+  float sm_scale;
+};
+int fdb_launch_bwd(const FdbBwdParams& p, int dtype, int head_dim, void* stream);
+
 // Workspace slot `slot`: its output rows and its log-sum-exps (row_bytes = head_dim * element size).
 #if defined(__HIPCC__)
 __device__ __forceinline__ char* ws_slot_out(const FdbKParams& p, int slot, int row_bytes) {

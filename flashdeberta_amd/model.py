@@ -5,8 +5,9 @@ Counterparts in the reference (src/flashdeberta/model.py):
   DEBERTA_SELF_ATTENTION_CLASSES   :254-257  {"eager", "flash_attention_2"}
   FlashDebertaV2Model              :394-496  here a thin subclass of transformers' DebertaV2Model
 The eager entry is transformers' own DisentangledSelfAttention, exactly as in the reference.
-Forward / inference only (the reference's varlen path has no backward either,
-src/flashdeberta/ops/flash_attention_varlen.py:480-483).
+Differentiable like the reference's fixed-length op (padded batches included: they stay in the fixed layout
+here); attention-probability dropout is not applied (nor is it on the reference's flash path: only the dropout
+on the relative embeddings remains, model.py:159-160).
 """
 import math
 import weakref
@@ -103,7 +104,9 @@ class FlashDisentangledSelfAttention(DisentangledSelfAttention):
         """q, k, v as [B, L, H, D] views (reference model.py:147-149)."""
         B, L, _ = hidden_states.shape
         H, D = self.num_attention_heads, self.attention_head_size
-        fused = None if (self.training or query_states is not hidden_states) else self._fused_qkv()
+        # the concatenated weights are a copy made outside autograd: only where nothing is being recorded
+        recording = torch.is_grad_enabled() and (hidden_states.requires_grad or self.query_proj.weight.requires_grad)
+        fused = None if (self.training or recording or query_states is not hidden_states) else self._fused_qkv()
         if fused is not None:
             qkv = F.linear(hidden_states, fused[0], fused[1]).view(B, L, 3, H, D)
             return qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
@@ -122,7 +125,8 @@ class FlashDisentangledSelfAttention(DisentangledSelfAttention):
         if "p2c" in self.pos_att_type:
             qproj = self.query_proj if self.share_att_key else self.pos_query_proj
         key = None
-        if not self.training:
+        recording = torch.is_grad_enabled() and (rel_embeddings.requires_grad or self.query_proj.weight.requires_grad)
+        if not self.training and not recording:  # a remembered K_r / Q_r must not carry an autograd graph
             key = (rel_embeddings,) + tuple(p for m in (kproj, qproj) if m is not None for p in (m.weight, m.bias)
                                             if p is not None)
             hit = self._pos_memo.get(key, tuple(self.pos_att_type))
@@ -146,11 +150,8 @@ class FlashDisentangledSelfAttention(DisentangledSelfAttention):
         """-> (context [B, L, H*D], None).  `relative_pos` is ignored: the bucketed relative
         position is an integer table inside the kernel.  Attention probabilities are never
         materialised, so `output_attentions` yields None like the reference (model.py:252)."""
-        if self.training and torch.is_grad_enabled() and hidden_states.requires_grad:
-            raise RuntimeError("FlashDisentangledSelfAttention is forward-only; use the eager implementation to train")
-        # Outside training the forward still runs with autograd recording (the reference's test calls the
-        # module without no_grad); the fused op then sits in the graph as a node whose backward raises, as the
-        # reference's packed op does (flash_attention_varlen.py:480-483), instead of cutting the graph silently.
+        # Under autograd the fused op is one node: differentiable in fp32 / bf16 / fp16 (the reference's
+        # FlashAttentionDisentangled, flash_attention.py:1032-1086); with FP8 operands its backward raises.
         if query_states is None:
             query_states = hidden_states
         B, L, _ = hidden_states.shape
@@ -187,7 +188,7 @@ class FlashDisentangledSelfAttention(DisentangledSelfAttention):
                 pos_query, kw["pos_query_scale"] = ops.quantize_e4m3_per_head(pos_query.transpose(0, 1))
                 pos_query = pos_query.transpose(0, 1)
 
-        ctx = ops.disentangled_attention_forward_only(
+        ctx = ops.disentangled_attention(
             q, k, v, pos_key, pos_query, sm_scale=sm_scale,
             position_buckets=self.position_buckets if self.relative_attention else 0,
             max_relative_positions=self.max_relative_positions if self.relative_attention else 0,

@@ -236,10 +236,101 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
     return (out, lse) if return_lse else out
 
 
+def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=None, *, sm_scale=None, position_buckets=0,
+                               max_relative_positions=0, causal=False, seq_start=None, seq_len=None):
+    """Backward of the fixed layout: q, k, v, out, dout [B, L, H, D], lse [B*L, H] as the forward returns it,
+    pos_key = K_r / pos_query = Q_r [H, 2S, D] or None  ->  (dq, dk, dv, d pos_key, d pos_query).
+    Counterpart of FlashAttentionDisentangled.backward (reference flash_attention.py:1066-1086), which hands
+    flash_attn_v2_bwd_dise the position-score tensors and gets their gradients back; as there, those tensors
+    are two GEMMs around the kernel (here fp32 [B, L, H, 2S]) and the chain through K_r / Q_r and back into
+    q / k is four more."""
+    B, L, H, D = q.shape
+    if q.dtype not in _DTYPES:
+        raise ValueError("unsupported dtype %s" % q.dtype)
+    span = att_span(position_buckets, max_relative_positions)
+    pos_key = _pos_arg(pos_key, H, D, span, "pos_key")
+    pos_query = _pos_arg(pos_query, H, D, span, "pos_query")
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(D * (1 + (pos_key is not None) + (pos_query is not None)))
+    q, k, v, dout = [x if x.stride(-1) == 1 else x.contiguous() for x in (q, k, v, dout)]
+    a = _lib.FdbAttnBwdArgs()
+    f32 = torch.float32
+    c2p = p2c = d_c2p = d_p2c = None
+    if pos_key is not None or pos_query is not None:
+        lut, radius = delta_lut_device(position_buckets, max_relative_positions, q.device)
+        a.delta_lut, a.lut_radius, a.att_span = lut.data_ptr(), radius, span
+    if pos_key is not None:
+        pk32 = pos_key[:, :2 * span].to(f32)
+        c2p = torch.einsum("blhd,hsd->blhs", q.to(f32), pk32).contiguous()
+        d_c2p = torch.zeros_like(c2p)
+        a.c2p_bias, a.d_c2p_bias = c2p.data_ptr(), d_c2p.data_ptr()
+    if pos_query is not None:
+        pq32 = pos_query[:, :2 * span].to(f32)
+        p2c = torch.einsum("blhd,hsd->blhs", k.to(f32), pq32).contiguous()
+        d_p2c = torch.zeros_like(p2c)
+        a.p2c_bias, a.d_p2c_bias = p2c.data_ptr(), d_p2c.data_ptr()
+    delta = (dout.to(f32) * out.to(f32)).sum(dim=-1).contiguous()  # [B, L, H]
+    lse = lse.contiguous()
+    padded = seq_start is not None or seq_len is not None
+    alloc = torch.zeros if padded else torch.empty
+    dq, dk, dv = [alloc((B, L, H, D), dtype=q.dtype, device=q.device) for _ in range(3)]
+    a.q, a.k, a.v, a.dout = q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr()
+    a.dq, a.dk, a.dv, a.lse, a.delta = dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), lse.data_ptr(), delta.data_ptr()
+    for n, x in (("q", q), ("k", k), ("v", v), ("do", dout), ("dq", dq), ("dk", dk), ("dv", dv)):
+        setattr(a, n + "_stride_b", x.stride(0))
+        setattr(a, n + "_stride_t", x.stride(1))
+        setattr(a, n + "_stride_h", x.stride(2))
+    keep = []
+    for n, x in (("seq_start", seq_start), ("seq_len", seq_len)):
+        if x is not None:
+            x = x.contiguous()
+            keep.append(x)
+            setattr(a, n, x.data_ptr())
+    a.batch, a.heads, a.head_dim, a.seqlen = B, H, D, L
+    a.dtype, a.causal, a.sm_scale = _DTYPES[q.dtype], int(bool(causal)), float(sm_scale)
+    with torch.cuda.device(q.device):
+        check(lib.fdb_attn_bwd(ctypes.byref(a), _stream_ptr(q.device)), "fdb_attn_bwd")
+    dpk = dpq = None
+    if pos_key is not None:  # score = q . K_r[delta]: both factors get their share
+        dq = (dq.to(f32) + torch.einsum("blhs,hsd->blhd", d_c2p, pk32)).to(q.dtype)
+        dpk = torch.zeros(pos_key.shape, dtype=f32, device=q.device)
+        dpk[:, :2 * span] = torch.einsum("blhs,blhd->hsd", d_c2p, q.to(f32))
+        dpk = dpk.to(pos_key.dtype)
+    if pos_query is not None:
+        dk = (dk.to(f32) + torch.einsum("blhs,hsd->blhd", d_p2c, pq32)).to(k.dtype)
+        dpq = torch.zeros(pos_query.shape, dtype=f32, device=q.device)
+        dpq[:, :2 * span] = torch.einsum("blhs,blhd->hsd", d_p2c, k.to(f32))
+        dpq = dpq.to(pos_query.dtype)
+    return dq, dk, dv, dpk, dpq
+
+
+class _DisentangledAttention(torch.autograd.Function):
+    """Fused forward + the backward above as one autograd node (fixed layout).  Counterpart of the reference's
+    FlashAttentionDisentangled (flash_attention.py:1032-1086)."""
+
+    @staticmethod
+    def forward(ctx, kwargs, q, k, v, pos_key, pos_query):
+        out, lse = disentangled_attention_fwd(q, k, v, pos_key, pos_query, return_lse=True, **kwargs)
+        ctx.save_for_backward(q, k, v, out, lse, *(x for x in (pos_key, pos_query) if x is not None))
+        ctx.cfg = (kwargs, pos_key is not None, pos_query is not None)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        kwargs, has_pk, has_pq = ctx.cfg
+        q, k, v, out, lse = ctx.saved_tensors[:5]
+        pk = ctx.saved_tensors[5] if has_pk else None
+        pq = ctx.saved_tensors[5 + has_pk] if has_pq else None
+        kw = {n: kwargs[n] for n in ("sm_scale", "position_buckets", "max_relative_positions", "causal", "seq_start", "seq_len")
+              if n in kwargs}
+        dq, dk, dv, dpk, dpq = disentangled_attention_bwd(q, k, v, out, lse, dout, pk, pq, **kw)
+        return None, dq, dk, dv, dpk, dpq
+
+
 class _ForwardOnly(torch.autograd.Function):
-    """The fused forward as an autograd node whose backward raises: a graph that runs through the op fails
-    loudly at .backward() instead of silently dropping the gradients of everything before it (the
-    reference's packed op does the same, flash_attention_varlen.py:480-483)."""
+    """The fused forward as an autograd node whose backward raises: a graph that runs through a variant
+    without a backward fails loudly at .backward() instead of silently dropping the gradients of everything
+    before it (the reference's packed op does the same, flash_attention_varlen.py:480-483)."""
 
     @staticmethod
     def forward(ctx, kwargs, q, k, v, pos_key, pos_query):
@@ -247,15 +338,25 @@ class _ForwardOnly(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, *grads):
-        raise RuntimeError("the fused disentangled attention is forward-only: no backward is implemented; "
-                           "use the eager implementation where gradients are needed")
+        raise RuntimeError("this variant of the fused disentangled attention is forward-only (packed layout and FP8 "
+                           "operands have no backward); use the fixed layout or the eager implementation")
 
 
-def disentangled_attention_forward_only(q, k, v, pos_key=None, pos_query=None, **kwargs):
-    """disentangled_attention_fwd (single output, no return_lse) for callers that may run under autograd."""
+_BWD_KW = {"sm_scale", "position_buckets", "max_relative_positions", "causal", "seq_start", "seq_len", "out", "far_splits",
+           "near_splits", "workspace"}
+
+
+def disentangled_attention(q, k, v, pos_key=None, pos_query=None, **kwargs):
+    """disentangled_attention_fwd (single output) for callers that may run under autograd: with gradients
+    required, the fixed layout in fp32 / bf16 / fp16 is differentiable (dq, dk, dv, d pos_key, d pos_query);
+    the packed layout and FP8 operands become a node whose backward raises."""
     if torch.is_grad_enabled() and any(x is not None and x.requires_grad for x in (q, k, v, pos_key, pos_query)):
-        return _ForwardOnly.apply(kwargs, q, k, v, pos_key, pos_query)
+        differentiable = q.dim() == 4 and q.dtype in _DTYPES and set(kwargs) <= _BWD_KW
+        return (_DisentangledAttention if differentiable else _ForwardOnly).apply(kwargs, q, k, v, pos_key, pos_query)
     return disentangled_attention_fwd(q, k, v, pos_key, pos_query, **kwargs)
+
+
+disentangled_attention_forward_only = disentangled_attention  # earlier name
 
 
 def flash_attention_with_disentangled(q, k, v, k_pos, q_pos, causal=False, sm_scale=None,

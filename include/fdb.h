@@ -22,6 +22,8 @@
  *                             (flash_attention.py:236-254, flash_attention_varlen.py:174-186), i.e.
  *                             make_log_bucket_position of transformers' modeling_deberta_v2.py:56-69
  *                             followed by clamp(. + S, 0, 2S-1) (:318, :336); host-side, integers out.
+ *   fdb_attn_bwd           <- flash_attn_v2_bwd_dise (flash_attention.py:942-1030) with _bwd_preprocess,
+ *                             _bwd_kv_dise_kernel and _bwd_q_dise_kernel (:62-141, :581-941).
  *   fdb_quant_e4m3_per_head, fdb_dequant_e4m3_per_head   no reference counterpart (FP8 Q/K variant).
  */
 #ifndef FDB_H_
@@ -35,7 +37,7 @@ extern "C" {
 #endif
 
 /* bumped whenever fdb_attn_args or the meaning of an entry point changes: a binding checks it next to the struct size */
-#define FDB_VERSION 4
+#define FDB_VERSION 5
 
 /* element types of q/k/pos_key/pos_query (v and out: see fdb_attn_args.dtype) */
 enum fdb_dtype {
@@ -148,6 +150,57 @@ int fdb_attn_fwd(const fdb_attn_args* a, void* stream);
  */
 #define FDB_NOALLOC_SCRATCH_BYTES (32 * 1024 * 1024)
 int fdb_attn_fwd_noalloc(const fdb_attn_args* a, void* stream);
+
+/*
+ * Backward, fixed layout (optionally with seq_start / seq_len).  Replaces flash_attn_v2_bwd_dise and the three
+ * kernels it launches (src/flashdeberta/ops/flash_attention.py:942-1030, :62-141, :581-941), called from
+ * FlashAttentionDisentangled.backward (:1066-1086).  Same division of labour as there: the position scores come
+ * in as tensors, c2p_bias[b,l,h,delta] = q . K_r[delta] and p2c_bias[b,l,h,delta] = k . Q_r[delta] (fp32,
+ * [B, L, H, 2S] contiguous; the reference: [B,H,L,2S] in the input dtype), and the gradients with respect to them
+ * leave in d_c2p_bias / d_p2c_bias (same shape, fp32, ZEROED BY THE CALLER: they are scatter-added); the chain
+ * through K_r / Q_r and into q / k is the caller's GEMMs.  dq, dk, dv hold only the content part,
+ *   dq_i = sum_j dS_ij k_j,  dk_j = sum_i dS_ij q_i,  dv_j = sum_i P_ij dO_i,  dS = P (dO V^T - delta) sm_scale,
+ * with P recomputed from lse (the forward's log-sum-exp, [B*L, H]) and delta[row] = sum_d dO * O ([B*L, H] fp32).
+ * Rows outside [seq_start, seq_start + seq_len) are not written.  q, k, v, dout, dq, dk, dv: element type of
+ * `dtype` (fp32 / bf16 / fp16), layout and strides as in fdb_attn_args.
+ */
+typedef struct fdb_attn_bwd_args {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* dout;
+  void* dq;
+  void* dk;
+  void* dv;
+  const float* lse;
+  const float* delta;
+  const float* c2p_bias;   /* or NULL: no content->position term */
+  const float* p2c_bias;   /* or NULL: no position->content term */
+  float* d_c2p_bias;       /* required with c2p_bias */
+  float* d_p2c_bias;       /* required with p2c_bias */
+  const int32_t* seq_start;
+  const int32_t* seq_len;
+  const int16_t* delta_lut;
+  int64_t q_stride_b, q_stride_t, q_stride_h;
+  int64_t k_stride_b, k_stride_t, k_stride_h;
+  int64_t v_stride_b, v_stride_t, v_stride_h;
+  int64_t do_stride_b, do_stride_t, do_stride_h;
+  int64_t dq_stride_b, dq_stride_t, dq_stride_h;
+  int64_t dk_stride_b, dk_stride_t, dk_stride_h;
+  int64_t dv_stride_b, dv_stride_t, dv_stride_h;
+  int32_t batch;
+  int32_t heads;
+  int32_t head_dim;
+  int32_t seqlen;
+  int32_t att_span;
+  int32_t lut_radius;
+  int32_t dtype;           /* FDB_F32, FDB_BF16 or FDB_F16 */
+  int32_t causal;
+  float sm_scale;
+} fdb_attn_bwd_args;
+
+size_t fdb_attn_bwd_args_size(void);
+int fdb_attn_bwd(const fdb_attn_bwd_args* a, void* stream);
 
 /*
  * Bytes of workspace the call would use (0: none), for the device that is current.  A launch whose

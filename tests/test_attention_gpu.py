@@ -880,8 +880,8 @@ def test_packed_call_with_an_underestimated_max_seqlen():
 
 def test_module_mask_with_holes_and_backward():
     """A mask row with masked tokens between real ones cannot be honoured by the kernels: the module marks
-    the whole row NaN (the other rows are computed as usual).  Under autograd the fused op is a node whose
-    backward raises."""
+    the whole row NaN (the other rows are computed as usual).  With FP8 operands the fused op is, under autograd,
+    a node whose backward raises."""
     from flashdeberta_amd import FlashDisentangledSelfAttention
 
     class Cfg:
@@ -902,12 +902,120 @@ def test_module_mask_with_holes_and_backward():
     holed[2, 7] = 0
     out = att(x, holed, rel_embeddings=rel)[0]
     assert torch.isnan(out[2]).all() and torch.equal(out[:2], good[:2]) and not torch.isnan(good).any()
-    # eval mode, autograd recording: the forward runs, the backward raises instead of returning nothing
+    # FP8 operands have no backward: under autograd the forward runs, the backward raises instead of returning nothing
+    att8 = FlashDisentangledSelfAttention(Cfg(), fp8_qk=True).eval().cuda().to(torch.bfloat16)
+    att8.load_state_dict(att.state_dict())
     xg = x.clone().requires_grad_(True)
-    y = att(xg, mask, rel_embeddings=rel)[0]
-    assert torch.equal(y.detach(), good)
+    y = att8(xg, mask, rel_embeddings=rel)[0]
     with pytest.raises(RuntimeError, match="forward-only"):
         y.float().sum().backward()
+
+
+# ---- backward ------------------------------------------------------------------------------------------------
+BWD_CASES = [
+    # B, L, H, D, buckets, max_rel, c2p, p2c, causal, lengths (None: full)
+    (1, 40, 2, 64, 8, 16, True, True, False, None),       # radius 16: every zone inside one tile
+    (2, 200, 2, 64, 32, 64, True, True, False, None),     # ragged tail, far steps on both sides
+    (2, 333, 2, 64, 32, 64, True, True, False, [333, 150]),  # padded batch (seq_len), ragged
+    (1, 300, 2, 64, 32, 64, True, False, False, None),
+    (1, 300, 2, 64, 32, 64, False, True, False, None),
+    (1, 260, 1, 64, 32, 64, False, False, False, None),   # content only
+    (2, 200, 2, 64, 32, 64, True, True, True, None),      # causal
+    (1, 700, 1, 64, 256, 512, True, True, False, None),   # v3 buckets: linear + log zone + saturation
+    (1, 150, 2, 32, 32, 64, True, True, False, None),
+    (1, 150, 2, 128, 32, 64, True, True, False, None),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("case", BWD_CASES, ids=lambda c: "B%dL%dH%dD%d_b%d_m%d_%d%d_c%d_%s" % (c[:9] + ("pad" if c[9] else "full",)))
+def test_backward_matches_oracle(case, dtype):
+    """dq, dk, dv, dK_r, dQ_r of the HIP backward (through the autograd node) against the oracle's chain rule on
+    the same seeded inputs; bound relative to each gradient's largest entry."""
+    B, L, H, D, pb, mr, c2p, p2c, causal, lens = case
+    q, k, v, pk, pq = _inputs(B, L, H, D, pb, mr, dtype, 3000 + L, 1.0, c2p, p2c)
+    g = torch.Generator().manual_seed(3001 + L)
+    dout = torch.randn(B, L, H, D, generator=g).to(dtype)
+    mask = None
+    kw = dict(position_buckets=pb, max_relative_positions=mr, causal=causal)
+    if lens is not None:
+        mask = np.arange(L)[None, :] < np.array(lens)[:, None]
+        dout = dout * torch.from_numpy(mask)[:, :, None, None].to(dtype)
+        kw["seq_len"] = torch.tensor(lens, dtype=torch.int32, device="cuda")
+        kw["out"] = torch.zeros(B, L, H, D, dtype=dtype, device="cuda")
+    t = lambda x: _np(x).transpose(0, 2, 1, 3)
+    ref = O.disentangled_attention_backward(t(q), t(k), t(v), t(dout), _np(pk), _np(pq), pb, mr, mask=mask, causal=causal)
+    leaves = [None if x is None else x.cuda().requires_grad_(True) for x in (q, k, v, pk, pq)]
+    out = ops.disentangled_attention(*leaves, **kw)
+    out.backward(dout.cuda())
+    tol = 2e-4 if dtype == torch.float32 else 3e-2
+    names = ("dq", "dk", "dv", "dK_r", "dQ_r")
+    for n, leaf, r in zip(names, leaves, ref):
+        if leaf is None:
+            continue
+        got = leaf.grad.float().cpu().numpy()
+        r = r.transpose(0, 2, 1, 3) if r.ndim == 4 else r
+        if mask is not None and r.ndim == 4:
+            r = r * mask[:, :, None, None]
+        err = np.abs(got - r).max()
+        assert not np.isnan(got).any() and err <= tol * max(np.abs(r).max(), 1e-3), "%s: err %.3e, ref max %.3e" % (n, err, np.abs(r).max())
+
+
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "g_*.npz"))), ids=os.path.basename)
+def test_module_backward_matches_golden_gradients(path):
+    """The drop-in module under autograd against the gradients torch.autograd wrote through the eager class:
+    hidden states, relative embeddings and every weight (fp32)."""
+    g = np.load(path)
+    mod = _module_from_golden(g).cuda()  # eval mode (the fixture's config has dropout on the relative embeddings), autograd recording
+    hidden = torch.from_numpy(g["hidden"]).cuda().requires_grad_(True)
+    rel = torch.from_numpy(g["rel_embeddings"]).cuda().requires_grad_(True)
+    mask = torch.from_numpy(g["mask"]).cuda()
+    out = mod(hidden, None if bool(mask.all()) else mask, rel_embeddings=rel)[0]
+    valid = g["mask"].astype(bool)[:, :, None]
+    assert np.abs(np.where(valid, out.detach().cpu().numpy() - g["out"], 0)).max() < 2e-4 * max(1.0, np.abs(g["out"]).max())
+    (out * torch.from_numpy(g["gout"]).cuda()).sum().backward()
+    got = {"hidden": hidden.grad, "rel_embeddings": rel.grad}
+    got.update({"w." + n: prm.grad for n, prm in mod.named_parameters()})
+    for name, t in got.items():
+        ref = g["g." + name]
+        val = np.zeros_like(ref) if t is None else t.cpu().numpy()
+        err = np.abs(val - ref).max()
+        assert err < 5e-4 * max(1.0, np.abs(ref).max()), (name, err, np.abs(ref).max())
+
+
+def test_module_backward_matches_live_eager_bf16():
+    """bf16 training step of the drop-in module against the eager class in fp32 on the host: same weights, same
+    inputs, gradients of the hidden states and of every weight."""
+    from transformers.models.deberta_v2.modeling_deberta_v2 import DisentangledSelfAttention
+
+    from flashdeberta_amd import FlashDisentangledSelfAttention
+
+    class Cfg:
+        hidden_size, num_attention_heads = 256, 4
+        attention_probs_dropout_prob = hidden_dropout_prob = 0.0
+        pos_att_type = ["c2p", "p2c"]
+        relative_attention, position_buckets, max_relative_positions = True, 256, 512
+        max_position_embeddings, share_att_key = 512, True
+
+    torch.manual_seed(8)
+    eager = DisentangledSelfAttention(Cfg()).train()
+    flash = FlashDisentangledSelfAttention(Cfg()).train()
+    flash.load_state_dict(eager.state_dict())
+    flash = flash.cuda().to(torch.bfloat16)
+    B, L = 2, 700
+    hidden = torch.randn(B, L, 256)
+    rel = torch.randn(512, 256)
+    gout = torch.randn(B, L, 256)
+    h0 = hidden.clone().requires_grad_(True)
+    (eager(h0, torch.ones(B, 1, L, L), rel_embeddings=rel)[0] * gout).sum().backward()
+    h1 = hidden.cuda().to(torch.bfloat16).requires_grad_(True)
+    (flash(h1, None, rel_embeddings=rel.cuda().to(torch.bfloat16))[0] * gout.cuda().to(torch.bfloat16)).sum().backward()
+    pairs = [("hidden", h0.grad, h1.grad)] + [(n, p0.grad, p1.grad) for (n, p0), (_, p1) in
+                                                zip(eager.named_parameters(), flash.named_parameters())]
+    for name, a, b in pairs:
+        ref = a.numpy()
+        err = np.abs(b.float().cpu().numpy() - ref).max()
+        assert err <= 4e-2 * np.abs(ref).max(), (name, err, np.abs(ref).max())
 
 
 def test_bad_arguments_raise():
