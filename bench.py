@@ -190,6 +190,9 @@ def main():
     ap.add_argument("--workload", default="v3base_L4096_B8_bf16", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-settle", action="store_true", help="skip the untimed settle phase before the warm-up")
+    ap.add_argument("--backward", action="store_true",
+                    help="time forward + backward through the autograd node instead (fixed-layout 16-bit / fp32 workloads); "
+                         "priced at 3.5 x the forward's algorithmic FLOPs (two products forward, five backward)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="also run one device-to-device copy of this many MiB (a kernel of known HBM traffic "
                          "against which rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled)")
@@ -206,6 +209,16 @@ def main():
     B, L, H, D, dt, kind = WORKLOADS[args.workload]
     tensors, kw, out, lens = make_inputs(args.workload, device)
     step = lambda: ops.disentangled_attention_fwd(*tensors, out=out, **kw)
+    if args.backward:
+        if kind != "fixed" or dt == "fp8":
+            sys.exit("bench.py --backward: the backward exists for the fixed layout in fp32 / bf16 / fp16")
+        leaves = [t.detach().clone().requires_grad_(True) for t in tensors]
+        dout = torch.randn_like(out) * 0.02
+
+        def step():
+            for t in leaves:
+                t.grad = None
+            ops.disentangled_attention(*leaves, **kw).backward(dout)
     if args.copy_calibration:
         src = torch.empty(args.copy_calibration << 20, dtype=torch.uint8, device=device)
         dst = torch.empty_like(src)
@@ -243,7 +256,7 @@ def main():
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
     kern_ms = ev0.elapsed_time(ev1) / args.steps
-    fl = flops(lens, H, D)
+    fl = flops(lens, H, D) * (3.5 if args.backward else 1.0)
     tokens = sum(lens)
     # e4m3 operands at head_dim <= 64 are expanded to bf16 inside the step (ops.disentangled_attention_fwd) and
     # contracted on the bf16 MFMA path: the arithmetic type, and the peak it is priced against, are bf16
@@ -253,7 +266,7 @@ def main():
     # the two launches of a step timed one at a time (same stream, HIP events), priced with the FLOPs of the
     # tiles each walks: content products of its tiles; the position products belong to the near launch
     kernels = None
-    if dt != "fp32" and D == 64:
+    if dt != "fp32" and D == 64 and not args.backward:
         far_t, near_t = tile_census(lens)
         split = {}
         for name, mask in (("far", 1), ("near", 2)):
@@ -275,7 +288,7 @@ def main():
         kernels = split
     traffic, traffic_source = measured_traffic(args.workload, with_source=True)
     rec = {
-        "metric": "disentangled_attn_fwd_tflops", "value": round(fl / (wall_ms * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
+        "metric": "disentangled_attn_fwd_bwd_tflops" if args.backward else "disentangled_attn_fwd_tflops", "value": round(fl / (wall_ms * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 4),
         "settle_ms": round(settle_ms, 1),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": arith, "data": "synthetic",

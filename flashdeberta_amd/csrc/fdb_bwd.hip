@@ -125,7 +125,12 @@ __global__ __launch_bounds__(kBwdThreads) void fdb_bwd_kernel(const FdbBwdParams
   const int S2 = 2 * p.S;
   const float* cbx = C2P && kDQ ? p.c2p + tok_x * S2 : nullptr;     // this lane's row of the lane-side position scores
   const float* pbx = P2C && !kDQ ? p.p2c + tok_x * S2 : nullptr;
-  float* gx = kDQ ? (C2P ? p.d_c2p + tok_x * S2 : nullptr) : (P2C ? p.d_p2c + tok_x * S2 : nullptr);  // ... and of its gradient
+  // Score gradients.  A far step (one table row for the block) adds the lane side's: one row sum per lane.  A near
+  // step adds the loop side's: register v is one row of that tensor and the 32 lanes of a half-wave fall on
+  // neighbouring table rows, so an atomic instruction touches a few cache lines instead of 64.  The other half of
+  // each tensor comes from the other role's launch, which classifies the same 32 x 32 blocks the same way.
+  float* gx = kDQ ? (C2P ? p.d_c2p + tok_x * S2 : nullptr) : (P2C ? p.d_p2c + tok_x * S2 : nullptr);
+  float* gy = kDQ ? (P2C ? p.d_p2c : nullptr) : (C2P ? p.d_c2p : nullptr);
 
   f32x16 acc1[DBLKS], acc2[DBLKS];  // dQ^T (dQ role) / dK^T and dV^T (dK/dV role)
 #pragma unroll
@@ -192,34 +197,43 @@ __global__ __launch_bounds__(kBwdThreads) void fdb_bwd_kernel(const FdbBwdParams
     const bool far = (C2P || P2C) && (r_min >= p.R || r_max <= -p.R);  // one table row for the whole block
     const int d_far = far ? delta_of(r_min) : 0;
     float lane_bias = 0.f;
-    if (far && x_ok) {
+    if (far) {
       if (C2P && kDQ) lane_bias = cbx[d_far];
       if (P2C && !kDQ) lane_bias = pbx[d_far];
     }
-    float ds[16], pr[16], g_sum = 0.f;
+    // Every position score of the step is requested before the first one is used: the loads are unconditional
+    // (rows past the end read the last valid row, lanes past the end read row 0) and only their use is masked,
+    // so that sixteen elements cost one round trip to memory, not sixteen.
+    float ds[16], pr[16], g_sum = 0.f, bias[16];
+    int dl[16];
+    bool ok[16];
+    int64_t goff[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int yr = y0 + 8 * (v >> 2) + 4 * g + (v & 3);
+      const int i = kDQ ? xr : yr, j = kDQ ? yr : xr;
+      ok[v] = x_ok && yr < Lb && (!p.causal || j <= i);
+      dl[v] = far ? d_far : ((C2P || P2C) ? delta_of(i - j) : 0);
+      const int64_t tok_y = ((int64_t)b * p.L + tok0 + min(yr, Lb - 1)) * p.H + h;
+      float bv = 0.f;
+      if (C2P) bv += kDQ ? (far ? lane_bias : cbx[dl[v]]) : p.c2p[tok_y * S2 + dl[v]];
+      if (P2C) bv += kDQ ? p.p2c[tok_y * S2 + dl[v]] : (far ? lane_bias : pbx[dl[v]]);
+      bias[v] = bv;
+      goff[v] = tok_y * S2 + dl[v];
+    }
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
       const int yl = 8 * (v >> 2) + 4 * g + (v & 3);
-      const int yr = y0 + yl;
-      const int i = kDQ ? xr : yr, j = kDQ ? yr : xr;
-      const bool ok = x_ok && yr < Lb && (!p.causal || j <= i);
-      const int dl = far ? d_far : ((C2P || P2C) ? delta_of(i - j) : 0);
-      float s = sacc[v];
-      if (ok) {
-        const int64_t tok_y = ((int64_t)b * p.L + tok0 + yr) * p.H + h;
-        if (C2P) s += kDQ ? (far ? lane_bias : cbx[dl]) : p.c2p[tok_y * S2 + dl];
-        if (P2C) s += kDQ ? p.p2c[tok_y * S2 + dl] : (far ? lane_bias : pbx[dl]);
-      }
       const float lse_i = kDQ ? lse_x : lse_s[yl], del_i = kDQ ? del_x : del_s[yl];
-      const float pv = ok ? __builtin_amdgcn_exp2f(__builtin_fmaf(s, c_log2, -lse_i)) : 0.f;
-      const float dsv = pv * (dpacc[v] - del_i) * c_sm;
+      const float pv = ok[v] ? __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[v] + bias[v], c_log2, -lse_i)) : 0.f;
       pr[v] = pv;
-      ds[v] = dsv;
-      if (gx != nullptr && ok) {
-        if (far) g_sum += dsv;
-        else unsafeAtomicAdd(gx + dl, dsv);
-      }
-      // the other side's score gradient: the other role's launch adds it
+      ds[v] = pv * (dpacc[v] - del_i) * c_sm;
+      g_sum += ds[v];
+    }
+    if (gy != nullptr && !far) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        if (ok[v]) unsafeAtomicAdd(gy + goff[v], ds[v]);
     }
     if (gx != nullptr && far) {
       g_sum = wave_half_sum(g_sum);
