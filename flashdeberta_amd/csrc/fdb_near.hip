@@ -243,15 +243,15 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
   // ---- prologue: step 0's K and ring batches 0..4 on their way to LDS -------------------------------------
   // All table values first, then all rows: the loads of one kind are in flight together.
   if (n_steps > 0) {
+    k_dma(s0, 0);  // K and V need no table value: on their way while the table is read
+    v_dma(s0, 0);
     int d0[6];
 #pragma unroll
     for (int bt = 0; bt < 6; ++bt) d0[bt] = batch_delta(bt);
-    // (taken here: the compiler, which does not count the direct loads, would otherwise wait for each
-    // value at its use, behind all the direct loads issued before it)
+    // (taken here, all at once: the compiler, which does not count the direct loads, would otherwise wait for
+    // each value at its use, behind all the direct loads issued before it)
 #pragma unroll
     for (int bt = 0; bt < 6; ++bt) asm volatile("" : "+v"(d0[bt]));
-    k_dma(s0, 0);
-    v_dma(s0, 0);
 #pragma unroll
     for (int bt = 0; bt < 5; ++bt) batch_dma(d0[bt], bt);
     dnext = d0[5];

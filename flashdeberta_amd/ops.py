@@ -142,7 +142,7 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
                 cu_seqlens=cu_seqlens, max_seqlen=max_seqlen, sm_scale=sm_scale, position_buckets=position_buckets,
                 max_relative_positions=max_relative_positions, causal=causal, return_lse=return_lse,
                 seq_start=seq_start, seq_len=seq_len, out=out, far_splits=far_splits, near_splits=near_splits,
-                workspace=workspace)
+                workspace=workspace, _launch_mask=_launch_mask)
         dt = _lib.FDB_FP8_E4M3
     else:
         if q.dtype not in _DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
