@@ -59,12 +59,15 @@ class _Memo:
 
 
 def _seq_bounds_of(attention_mask):
-    """(seq_start, seq_len, holes) of a mask; every layer of an encoder receives the same mask object, so
+    """(seq_start, seq_len, fill) of a mask; every layer of an encoder receives the same mask object, so
     the reductions run once per forward instead of once per layer.  The result rides on the mask tensor
     itself (no state outside it) and is dropped when the mask is written in place or re-seated."""
     hit = attention_mask.__dict__.get("_fdb_bounds")
     if hit is None or hit[0] != _stamp(attention_mask):
-        hit = (_stamp(attention_mask), seq_bounds(key_padding_mask(attention_mask)))
+        start, length, holes = seq_bounds(key_padding_mask(attention_mask))
+        # what the rows of the output start from: zero, or NaN for a row whose mask the kernels cannot honour
+        fill = torch.where(holes, float("nan"), 0.0).view(-1, 1, 1, 1)
+        hit = (_stamp(attention_mask), (start, length, fill))
         attention_mask._fdb_bounds = hit
     return hit[1]
 
@@ -169,11 +172,12 @@ class FlashDisentangledSelfAttention(DisentangledSelfAttention):
         seq_start = seq_len = None
         out = None
         if attention_mask is not None:
-            seq_start, seq_len, holes = _seq_bounds_of(attention_mask)
+            seq_start, seq_len, fill = _seq_bounds_of(attention_mask)
             # Padded rows stay zero.  The kernels take the real tokens of a row as one contiguous run; a row
             # whose mask has a hole inside that run gets no tokens (seq_len 0) and NaN in every position, so
             # the unsupported mask cannot pass for a result (the eager module honours arbitrary masks).
-            out = torch.where(holes.view(B, 1, 1, 1), float("nan"), 0.0).to(v.dtype).expand(B, L, H, D).contiguous()
+            out = torch.empty((B, L, H, D), dtype=v.dtype, device=v.device)
+            out.copy_(fill.expand(B, L, H, D))  # one fill kernel per layer
 
         kw = {}
         if self.fp8_qk:

@@ -300,8 +300,8 @@ def test_module_projection_memos():
 
     # mask bounds: once per mask object and version
     m = torch.tensor([[1, 1, 1, 0, 0], [0, 0, 1, 1, 1]])
-    s0, n0, h0 = _seq_bounds_of(m)
-    assert _seq_bounds_of(m)[0] is s0 and s0.tolist() == [0, 2] and n0.tolist() == [3, 3] and not h0.any()
+    s0, n0, f0 = _seq_bounds_of(m)
+    assert _seq_bounds_of(m)[0] is s0 and s0.tolist() == [0, 2] and n0.tolist() == [3, 3] and f0.flatten().tolist() == [0.0, 0.0]
     m[0, 3] = 1
     s1, n1, _ = _seq_bounds_of(m)
     assert s1 is not s0 and n1.tolist() == [4, 3]
