@@ -11,14 +11,14 @@
 // every eight to nine cycles, and nothing else hides that but a second wave.  Two workgroups share
 // a CU when each stays under 80 KB, which the rings allow only with 32-key steps:
 //   workgroup = 4 waves x 32 query rows, one step = 32 keys;
-//   a step sees 159 relative positions (5 batches of 32), and since the rows of the next step are
-//   stored after every wave has finished reading the ring in the current one, the rings hold
-//   exactly 5 batches = 160 rows of 128 bytes, unpadded and XOR-swizzled;
+//   a step sees 159 relative positions (5 batches of 32); the rings hold a sixth batch, the one being
+//   filled for the next step: 192 rows of 128 bytes, unpadded and XOR-swizzled;
 //   a wave's 32 x 32 sub-tile sees 63 relative positions, so both position products are 2 MFMA
 //   blocks, private to the wave: C[i][r] = q_i . E_K[r] and P[j][r] = k_j . E_Q[r], of which element
-//   (i, j) wants index r = i - j.  C goes through a per-wave fp32 LDS scratch and comes back as the
-//   initial value of the content product's accumulator; P is computed with the keys as MFMA rows, so
-//   its skew is a permutation of lanes within a register (ds_bpermute) and needs no scratch.
+//   (i, j) wants index r = i - j.  C goes through a per-wave 16-bit LDS scratch (only the one of its
+//   two blocks a lane needs, picked before the write) and comes back as the initial value of the
+//   content product's accumulator; P is computed with the keys as MFMA rows, so its skew is a rotation
+//   of the lanes of a half-wave by a constant of the register (ds_swizzle) and needs no scratch.
 // LDS: K 2 x 4 KB + V 2 x 4 KB + rings 2 x 24 KB + scratch 11 KB = 75 KB.
 //
 // Staging goes global -> LDS directly (global_load_lds_dwordx4: no staging registers, no LDS write
