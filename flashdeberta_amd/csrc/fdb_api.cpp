@@ -388,6 +388,8 @@ int fdb_attn_bwd(const fdb_attn_bwd_args* a, void* stream) {
   const bool has_pos = a->c2p_bias || a->p2c_bias;
   if ((a->c2p_bias && !a->d_c2p_bias) || (a->p2c_bias && !a->d_p2c_bias)) return FDB_ERR_NULL;
   if (has_pos && (a->att_span < 1 || a->lut_radius < 1 || !a->delta_lut)) return FDB_ERR_SPAN;
+  // the kernels address a sequence's rows of the position-score tensors with 32-bit element offsets
+  if (has_pos && (int64_t)a->seqlen * a->heads * 2 * a->att_span > 0x7fffffffll) return FDB_ERR_SHAPE;
   const int sz = qk_elem_size(a->dtype);
   const void* ptrs[] = {a->q, a->k, a->v, a->dout, a->dq, a->dk, a->dv};
   for (const void* ptr : ptrs)

@@ -14,10 +14,15 @@
 //   S' = Y1 X1^T (+ gathered position scores), P' = exp2(S' * c log2e - lse_i log2e), dP' = Y2 X2^T,
 //   dS' = P' (dP' - Delta_i) c, and the outputs contract over the loop rows, which sit in the accumulator
 //   registers: out^T += Y^T dS' (or P'), with Y^T read transposed from LDS -- the layout trick of the forward.
+// Score gradients without atomics.  Each role owns the tensor of its lane side (dQ role: d c2p, a row per query;
+// dK/dV role: d p2c, a row per key).  The table row delta(i - j) is monotone in the loop row with steps of 0 or 1, so
+// the entries a lane row can still receive form a window of at most 33 neighbours that slides one way as the loop
+// advances: a 64-entry ring per row in LDS takes the adds (ds_add_f32), and the entries the window has left behind
+// are stored once, row by row with the lanes on neighbouring entries, and cleared.  The tensors arrive zeroed;
+// entries no element maps to are never written.  Results do not depend on the order workgroups run in.
 // A step whose relative positions all lie beyond the table radius has one table row: its position scores are
-// one load per row and its score gradients leave as one row sum per lane instead of one atomic per element.
+// one load per row and its score gradients enter the ring as one row sum per lane.
 #include <hip/hip_runtime.h>
-#include <hip/amd_detail/amd_hip_unsafe_atomics.h>
 #include <stdint.h>
 
 #include <atomic>
@@ -32,7 +37,11 @@ namespace {
 
 constexpr int kBwdThreads = 256;
 constexpr int kBwdStep = 32;    // loop-side rows per step
-constexpr int kLutLds = 4096;   // table entries kept in LDS (larger tables are read from global memory)
+constexpr int kRing = 64;       // score-gradient entries kept per lane-side row (the live window is at most 33 wide)
+// Row stride of the ring in floats.  The lanes of a half-wave hit entry (delta0 -+ lane) of row `lane` (dQ role: +,
+// dK/dV role: -): with stride 65 resp. 67 that is bank 2 * lane, no two lanes alike.
+constexpr int ring_stride(bool dq) { return dq ? kRing + 1 : kRing + 3; }
+constexpr int kRingStrideMax = kRing + 3;
 
 template <class QT, int D>
 struct BCfg {
@@ -40,7 +49,9 @@ struct BCfg {
   static constexpr int RS = D * QT::SZ + 16;                 // LDS row stride of a staged tile
   static constexpr int TILE = kBwdStep * RS;
   static constexpr int CHUNKS = (kBwdStep * D * QT::SZ / 16 + kBwdThreads - 1) / kBwdThreads;  // 16-byte chunks per thread
-  static constexpr int lds_bytes() { return 2 * TILE + 2 * kBwdStep * 4 + kLutLds * 2; }
+  // two tile buffers, loop-row statistics, ring windows, far-step scores; the table follows
+  static constexpr int fixed_lds_bytes() { return 4 * TILE + 4 * kBwdStep * 4 + FDB_BM * kRingStrideMax * 4 + FDB_BM * 4; }
+  static int lds_bytes(int radius) { return fixed_lds_bytes() + (((2 * radius + 1) * 2 + 15) & ~15); }
 };
 
 // [32 x D] tile: global -> registers -> LDS.  Rows past the end re-read the last valid row; their scores are masked.
@@ -66,17 +77,18 @@ __device__ __forceinline__ void btile_store(char* lds, const u32x4 (&reg)[NCH], 
 }
 
 template <class QT, int D, int ROLE, bool C2P, bool P2C>
-__global__ __launch_bounds__(kBwdThreads) void fdb_bwd_kernel(const FdbBwdParams p) {
+__global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_bwd_kernel(const FdbBwdParams p) {
   using C = BCfg<QT, D>;
   using frag = typename QT::frag;
   constexpr int KS = C::KS, DBLKS = C::DBLKS;
   constexpr bool kDQ = ROLE == 0;
+  constexpr int kRingStride = ring_stride(kDQ);
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  char* Y1s = smem;                                   // K (dQ role) / Q (dK/dV role)
-  char* Y2s = Y1s + C::TILE;                          // V / dO
-  float* lse_s = (float*)(Y2s + C::TILE);             // dK/dV role: log-sum-exp (base 2) and Delta of the 32 loop rows
-  float* del_s = lse_s + kBwdStep;
-  int16_t* lut_s = (int16_t*)(del_s + kBwdStep);
+  char* Ys = smem;                                    // two buffers of [K | V] (dQ role) / [Q | dO] (dK/dV role)
+  float* stat_s = (float*)(Ys + 4 * C::TILE);         // dK/dV role: per buffer, log-sum-exp (base 2) and Delta of the 32 loop rows
+  float* ring_s = stat_s + 4 * kBwdStep;              // [128 lane-side rows][kRingStride] score-gradient windows
+  float* vec_s = ring_s + FDB_BM * kRingStrideMax;      // [4 waves][32] loop-side position scores of a far step
+  LDS_AS int16_t* lut_s = (LDS_AS int16_t*)(vec_s + FDB_BM);  // the whole table (the launcher sizes the allocation for it)
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -86,10 +98,8 @@ __global__ __launch_bounds__(kBwdThreads) void fdb_bwd_kernel(const FdbBwdParams
   const int tok0 = p.seq_start ? min(max(p.seq_start[b], 0), p.L) : 0;
   const int Lb = p.seq_len ? min(max(p.seq_len[b], 0), p.L - tok0) : p.L;
   if (m0 >= Lb) return;
-  const int n_lut = 2 * p.R + 1;
-  const bool lut_in_lds = n_lut <= kLutLds;
-  if (lut_in_lds && (C2P || P2C))
-    for (int x = tid; x < n_lut; x += kBwdThreads) lut_s[x] = p.lut[x];
+  if (C2P || P2C)
+    for (int x = tid; x < 2 * p.R + 1; x += kBwdThreads) lut_s[x] = p.lut[x];
 
   auto base = [&](const char* ptr, int64_t sb, int64_t st, int64_t sh) {
     return ptr + (b * sb + (int64_t)tok0 * st + (int64_t)h * sh) * QT::SZ;
@@ -123,14 +133,22 @@ __global__ __launch_bounds__(kBwdThreads) void fdb_bwd_kernel(const FdbBwdParams
     del_x = p.delta[tok_x];
   }
   const int S2 = 2 * p.S;
-  const float* cbx = C2P && kDQ ? p.c2p + tok_x * S2 : nullptr;     // this lane's row of the lane-side position scores
-  const float* pbx = P2C && !kDQ ? p.p2c + tok_x * S2 : nullptr;
-  // Score gradients.  A far step (one table row for the block) adds the lane side's: one row sum per lane.  A near
-  // step adds the loop side's: register v is one row of that tensor and the 32 lanes of a half-wave fall on
-  // neighbouring table rows, so an atomic instruction touches a few cache lines instead of 64.  The other half of
-  // each tensor comes from the other role's launch, which classifies the same 32 x 32 blocks the same way.
-  float* gx = kDQ ? (C2P ? p.d_c2p + tok_x * S2 : nullptr) : (P2C ? p.d_p2c + tok_x * S2 : nullptr);
-  float* gy = kDQ ? (P2C ? p.d_p2c : nullptr) : (C2P ? p.d_c2p : nullptr);
+  // Position-score tensors are addressed as one base per (batch row, head) plus 32-bit element offsets
+  // (token * H * 2S + table row; the launcher checks that L * H * 2S fits).
+  const int64_t seq_base = (((int64_t)b * p.L + tok0) * p.H + h) * S2;
+  const uint32_t row_elems = (uint32_t)p.H * (uint32_t)S2;           // elements between neighbouring tokens
+  const uint32_t x_off = (uint32_t)(x_ok ? xr : 0) * row_elems;      // this lane's row
+  // Score gradients of the lane side's tensor: ring rows of this wave in LDS, rows of this wave in the tensor.
+  constexpr bool kGrad = kDQ ? C2P : P2C;
+  float* ring_w = ring_s + wave * 32 * kRingStride;
+  float* ring_x = ring_w + li * kRingStride;
+  float* vec_w = vec_s + wave * 32;
+  float* gw = nullptr;
+  if (kGrad) {
+    gw = (kDQ ? p.d_c2p : p.d_p2c) + seq_base;
+    for (int e = lane; e < 32 * kRingStride; e += 64) ring_w[e] = 0.f;
+  }
+  constexpr int kDir = kDQ ? -1 : 1;        // the way the window moves as the loop row grows
 
   f32x16 acc1[DBLKS], acc2[DBLKS];  // dQ^T (dQ role) / dK^T and dV^T (dK/dV role)
 #pragma unroll
@@ -144,9 +162,18 @@ __global__ __launch_bounds__(kBwdThreads) void fdb_bwd_kernel(const FdbBwdParams
     if (kDQ) y_hi = min(Lb, m0 + FDB_BM);  // keys j <= i
     else y_lo = (m0 / kBwdStep) * kBwdStep;  // queries i >= j
   }
+  const float c_log2 = p.scale_log2, c_sm = p.sm_scale;
+  auto delta_of = [&](int r) __attribute__((always_inline)) -> int {
+    const int x = max(-p.R, min(p.R, r)) + p.R;
+    return (int)lut_s[x];
+  };
+  // The two tiles of a step sit in one of two LDS buffers: the tiles of step t + 1 are on their way to registers
+  // while step t computes and go to the other buffer at its end, so a step has one barrier.
   u32x4 y1reg[C::CHUNKS], y2reg[C::CHUNKS];
   float st_reg[2] = {0.f, 0.f};
-  auto stats_load = [&](int r0) __attribute__((always_inline)) {
+  auto tiles_load = [&](int r0) __attribute__((always_inline)) {
+    btile_load<QT, D>(y1reg, y1b, y1_rsb, r0, Lb, tid);
+    btile_load<QT, D>(y2reg, y2b, y2_rsb, r0, Lb, tid);
     if (!kDQ && tid < kBwdStep) {
       const int row = min(r0 + tid, Lb - 1);
       const int64_t t = ((int64_t)b * p.L + tok0 + row) * p.H + h;
@@ -154,31 +181,66 @@ __global__ __launch_bounds__(kBwdThreads) void fdb_bwd_kernel(const FdbBwdParams
       st_reg[1] = p.delta[t];
     }
   };
-  if (y_lo < y_hi) {
-    btile_load<QT, D>(y1reg, y1b, y1_rsb, y_lo, Lb, tid);
-    btile_load<QT, D>(y2reg, y2b, y2_rsb, y_lo, Lb, tid);
-    stats_load(y_lo);
-  }
-  const float c_log2 = p.scale_log2, c_sm = p.sm_scale;
-  auto delta_of = [&](int r) __attribute__((always_inline)) -> int {
-    const int x = max(-p.R, min(p.R, r)) + p.R;
-    return lut_in_lds ? (int)lut_s[x] : (int)p.lut[x];
-  };
-
-  for (int y0 = y_lo; y0 < y_hi; y0 += kBwdStep) {
-    __syncthreads();  // every wave is done with the tiles of the step before (and the table is in LDS)
-    btile_store<QT, D>(Y1s, y1reg, tid);
-    btile_store<QT, D>(Y2s, y2reg, tid);
+  auto tiles_store = [&](int buf) __attribute__((always_inline)) {
+    btile_store<QT, D>(Ys + buf * 2 * C::TILE, y1reg, tid);
+    btile_store<QT, D>(Ys + buf * 2 * C::TILE + C::TILE, y2reg, tid);
     if (!kDQ && tid < kBwdStep) {
-      lse_s[tid] = st_reg[0];
-      del_s[tid] = st_reg[1];
+      stat_s[buf * 2 * kBwdStep + tid] = st_reg[0];
+      stat_s[buf * 2 * kBwdStep + kBwdStep + tid] = st_reg[1];
     }
-    __syncthreads();
-    if (y0 + kBwdStep < y_hi) {
-      btile_load<QT, D>(y1reg, y1b, y1_rsb, y0 + kBwdStep, Lb, tid);
-      btile_load<QT, D>(y2reg, y2b, y2_rsb, y0 + kBwdStep, Lb, tid);
-      stats_load(y0 + kBwdStep);
+  };
+  // Position scores of a step are requested one step ahead (their addresses depend on indices only), so that their
+  // round trip to memory runs behind the step before.  A far step (every relative position of the wave's 32 x 32
+  // block beyond the table radius: one table row) asks for two values per lane, the lane row's score and the score of
+  // loop row `li`; a near step asks for one value per element and tensor.  Rows past the end re-read the last valid
+  // row, lanes past the end read row 0: the loads are unconditional and only their use is masked.
+  constexpr bool kBias = C2P || P2C;
+  constexpr bool kLaneT = kDQ ? C2P : P2C, kLoopT = kDQ ? P2C : C2P;
+  const float* lane_t = kLaneT ? (kDQ ? p.c2p : p.p2c) + seq_base : nullptr;   // the lane side's tensor, this sequence and head
+  const float* loop_t = kLoopT ? (kDQ ? p.p2c : p.c2p) + seq_base : nullptr;   // the loop side's
+  float raw_lane[16], raw_loop[16];
+  bool far_n = false;
+  int dfar_n = 0;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) raw_lane[v] = raw_loop[v] = 0.f;
+  auto loop_off = [&](int yr) __attribute__((always_inline)) -> uint32_t {
+    return (uint32_t)min(yr, Lb - 1) * row_elems;
+  };
+  auto request = [&](int y0) __attribute__((always_inline)) {
+    if (!kBias) return;
+    const int r_min = kDQ ? xw0 - (y0 + kBwdStep - 1) : y0 - (xw0 + 31);      // over the wave's 32 x 32 block
+    const int r_max = kDQ ? xw0 + 31 - y0 : y0 + kBwdStep - 1 - xw0;
+    far_n = r_min >= p.R || r_max <= -p.R;
+    dfar_n = far_n ? delta_of(r_min) : 0;
+    if (far_n) {
+      if (kLaneT) raw_lane[0] = lane_t[x_off + (uint32_t)dfar_n];
+      if (kLoopT) raw_loop[0] = loop_t[loop_off(y0 + li) + (uint32_t)dfar_n];
+    } else {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int yr = y0 + 8 * (v >> 2) + 4 * g + (v & 3);
+        const int dl = delta_of(kDQ ? xr - yr : yr - xr);
+        if (kLaneT) raw_lane[v] = lane_t[x_off + (uint32_t)dl];
+        if (kLoopT) raw_loop[v] = loop_t[loop_off(yr) + (uint32_t)dl];
+      }
     }
+  };
+  if (y_lo < y_hi) {
+    tiles_load(y_lo);
+    __syncthreads();  // the table is in LDS
+    request(y_lo);
+    tiles_store(0);
+  }
+
+  int buf = 0;
+  for (int y0 = y_lo; y0 < y_hi; y0 += kBwdStep, buf ^= 1) {
+    __syncthreads();  // the tiles of this step are in LDS; every wave is done with the other buffer (and the table is there)
+    const bool has_next = y0 + kBwdStep < y_hi;
+    if (has_next) tiles_load(y0 + kBwdStep);
+    const char* Y1s = Ys + buf * 2 * C::TILE;
+    const char* Y2s = Y1s + C::TILE;
+    const float* lse_s = stat_s + buf * 2 * kBwdStep;
+    const float* del_s = lse_s + kBwdStep;
     // ---- S' and dP' ----------------------------------------------------------------------------------------
     f32x16 sacc, dpacc;
 #pragma unroll
@@ -190,54 +252,100 @@ __global__ __launch_bounds__(kBwdThreads) void fdb_bwd_kernel(const FdbBwdParams
       sacc = QT::mma(y1f, x1f[s], sacc);
       dpacc = QT::mma(y2f, x2f[s], dpacc);
     }
-    // ---- position scores, probabilities, score gradients -------------------------------------------------------
+    // ---- position scores (requested during the step before), probabilities, score gradients ----------------------
     // element v of lane (g, li): loop row yr = y0 + 8*(v/4) + 4g + v%4, lane row xr; i - j = +-(xr - yr)
-    const int r_min = kDQ ? xw0 - (y0 + kBwdStep - 1) : y0 - (xw0 + 31);      // over the wave's 32 x 32 block
-    const int r_max = kDQ ? xw0 + 31 - y0 : y0 + kBwdStep - 1 - xw0;
-    const bool far = (C2P || P2C) && (r_min >= p.R || r_max <= -p.R);  // one table row for the whole block
-    const int d_far = far ? delta_of(r_min) : 0;
-    float lane_bias = 0.f;
-    if (far) {
-      if (C2P && kDQ) lane_bias = cbx[d_far];
-      if (P2C && !kDQ) lane_bias = pbx[d_far];
+    const bool far = far_n;
+    const int d_far = dfar_n;
+    float bias[16];
+    if (kBias && far) {
+      if (kLoopT) {
+        if (g == 0) vec_w[li] = raw_loop[0];
+        wave_lds_fence();
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          const f32x4 t4 = *(const f32x4*)(vec_w + 8 * q4 + 4 * g);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) bias[4 * q4 + e] = t4[e] + raw_lane[0];
+        }
+        wave_lds_fence();
+      } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) bias[v] = raw_lane[0];
+      }
+    } else {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) bias[v] = raw_lane[v] + raw_loop[v];
     }
-    // Every position score of the step is requested before the first one is used: the loads are unconditional
-    // (rows past the end read the last valid row, lanes past the end read row 0) and only their use is masked,
-    // so that sixteen elements cost one round trip to memory, not sixteen.
-    float ds[16], pr[16], g_sum = 0.f, bias[16];
-    int dl[16];
+    if (has_next) request(y0 + kBwdStep);
+    float ds[16], ds_run[16], pr[16], g_sum = 0.f;
     bool ok[16];
-    int64_t goff[16];
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
-      const int yr = y0 + 8 * (v >> 2) + 4 * g + (v & 3);
+      const int yl = 8 * (v >> 2) + 4 * g + (v & 3), yr = y0 + yl;
       const int i = kDQ ? xr : yr, j = kDQ ? yr : xr;
       ok[v] = x_ok && yr < Lb && (!p.causal || j <= i);
-      dl[v] = far ? d_far : ((C2P || P2C) ? delta_of(i - j) : 0);
-      const int64_t tok_y = ((int64_t)b * p.L + tok0 + min(yr, Lb - 1)) * p.H + h;
-      float bv = 0.f;
-      if (C2P) bv += kDQ ? (far ? lane_bias : cbx[dl[v]]) : p.c2p[tok_y * S2 + dl[v]];
-      if (P2C) bv += kDQ ? p.p2c[tok_y * S2 + dl[v]] : (far ? lane_bias : pbx[dl[v]]);
-      bias[v] = bv;
-      goff[v] = tok_y * S2 + dl[v];
-    }
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int yl = 8 * (v >> 2) + 4 * g + (v & 3);
       const float lse_i = kDQ ? lse_x : lse_s[yl], del_i = kDQ ? del_x : del_s[yl];
       const float pv = ok[v] ? __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[v] + bias[v], c_log2, -lse_i)) : 0.f;
       pr[v] = pv;
       ds[v] = pv * (dpacc[v] - del_i) * c_sm;
       g_sum += ds[v];
     }
-    if (gy != nullptr && !far) {
+    if (kGrad) {
+      // LDS float atomics are served a lane at a time on this hardware (160 clocks per instruction), so the adds are
+      // plain reads and writes: the lanes of a half-wave own different rows, and the two halves (which share rows)
+      // take turns.  Within a lane the table rows of the 16 elements are sorted, so elements of one entry are
+      // neighbours: each write carries the sum of its run so far and the last write of a run, the complete one, wins.
+      if (far) {
+        g_sum = wave_half_sum(g_sum);
+        if (g == 0) ring_x[d_far & (kRing - 1)] += g_sum;
+      } else {
+        int dl[16];
 #pragma unroll
-      for (int v = 0; v < 16; ++v)
-        if (ok[v]) unsafeAtomicAdd(gy + goff[v], ds[v]);
-    }
-    if (gx != nullptr && far) {
-      g_sum = wave_half_sum(g_sum);
-      if (g == 0 && x_ok) unsafeAtomicAdd(gx + d_far, g_sum);
+        for (int v = 0; v < 16; ++v) {
+          const int yr = y0 + 8 * (v >> 2) + 4 * g + (v & 3);
+          dl[v] = delta_of(kDQ ? xr - yr : yr - xr);
+          if (v > 0) ds_run[v] = ds[v] + (dl[v] == dl[v - 1] ? ds_run[v - 1] : 0.f);
+          else ds_run[0] = ds[0];
+        }
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          if (g == half) {
+            float old[16];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) old[v] = ring_x[dl[v] & (kRing - 1)];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) ring_x[dl[v] & (kRing - 1)] = old[v] + ds_run[v];
+          }
+          wave_lds_fence();
+        }
+      }
+      // Entries behind the window: from the table row of this step's first loop row up to (not including) that of
+      // the next step's first loop row, at most 32; after the last step, the 32 entries the step can have touched.
+      const int d_first = delta_of(kDQ ? xr - y0 : y0 - xr);
+      const int n_out = !x_ok ? 0 : !has_next ? 32 : kDir * (delta_of(kDQ ? xr - (y0 + kBwdStep) : y0 + kBwdStep - xr) - d_first);
+      if (__builtin_amdgcn_ballot_w64(n_out > 0) != 0) {
+        // A half-wave per row, its lanes on neighbouring entries: one store instruction writes two runs of up to 128
+        // bytes.  The bounds of row rho sit in lane rho; all sixteen reads are under way before the first is used.
+        float val[16];
+        int dd[16];
+        bool act[16];
+#pragma unroll
+        for (int it = 0; it < 16; ++it) {
+          const int f0 = __builtin_amdgcn_readlane(d_first, 2 * it), f1 = __builtin_amdgcn_readlane(d_first, 2 * it + 1);
+          const int n0 = __builtin_amdgcn_readlane(n_out, 2 * it), n1 = __builtin_amdgcn_readlane(n_out, 2 * it + 1);
+          dd[it] = (g ? f1 : f0) + kDir * li;
+          act[it] = li < (g ? n1 : n0);
+          val[it] = ring_w[(2 * it + g) * kRingStride + (dd[it] & (kRing - 1))];
+        }
+#pragma unroll
+        for (int it = 0; it < 16; ++it) {
+          if (act[it]) {
+            ring_w[(2 * it + g) * kRingStride + (dd[it] & (kRing - 1))] = 0.f;
+            if (val[it] != 0.f && dd[it] >= 0 && dd[it] < S2) gw[(uint32_t)(xw0 + 2 * it + g) * row_elems + (uint32_t)dd[it]] = val[it];
+          }
+        }
+        wave_lds_fence();
+      }
     }
     // ---- outputs: contraction over the loop rows, which are the accumulator registers ------------------------------
 #pragma unroll
@@ -255,6 +363,7 @@ __global__ __launch_bounds__(kBwdThreads) void fdb_bwd_kernel(const FdbBwdParams
         if (!kDQ) acc2[d] = QT::mma(VtLoad<QT>::get(Y2s, C::RS, c, d, lane), pf, acc2[d]);  // dV^T += dO^T P'
       }
     }
+    if (has_next) tiles_store(buf ^ 1);
   }
 
   if (!x_ok) return;
@@ -277,10 +386,11 @@ __global__ __launch_bounds__(kBwdThreads) void fdb_bwd_kernel(const FdbBwdParams
 template <class QT, int D, int ROLE, bool C2P, bool P2C>
 int launch_bwd_one(const FdbBwdParams& p, hipStream_t stream) {
   auto kern = fdb_bwd_kernel<QT, D, ROLE, C2P, P2C>;
-  constexpr int lds = BCfg<QT, D>::lds_bytes();
-  static_assert(lds <= 160 * 1024, "LDS budget");
+  static_assert(BCfg<QT, D>::fixed_lds_bytes() + 4096 <= 160 * 1024, "LDS budget");
+  const int lds = BCfg<QT, D>::lds_bytes((C2P || P2C) ? p.R : 0);
+  if (lds > 160 * 1024) return FDB_ERR_SPAN;  // the table does not fit beside the tiles
   static std::atomic<uint64_t> lds_set{0};
-  hipError_t e = fdb_set_lds_once((const void*)kern, lds, lds_set);
+  hipError_t e = fdb_set_lds_once((const void*)kern, 160 * 1024, lds_set);
   if (e != hipSuccess) return (int)e;
   const unsigned tiles = (unsigned)((p.L + FDB_BM - 1) / FDB_BM);
   hipLaunchKernelGGL(kern, dim3(tiles, (unsigned)p.H, (unsigned)p.B), dim3(kBwdThreads), lds, stream, p);
