@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(_HERE, "libfdb_hip.so")
 
 FDB_F32, FDB_BF16, FDB_F16, FDB_FP8_E4M3 = 0, 1, 2, 3
 FDB_NOALLOC_SCRATCH_BYTES = 32 * 1024 * 1024
-FDB_VERSION = 5  # of include/fdb.h as mirrored below
+FDB_VERSION = 6  # of include/fdb.h as mirrored below
 
 
 class FdbAttnArgs(ctypes.Structure):
@@ -37,7 +37,7 @@ class FdbAttnBwdArgs(ctypes.Structure):
         [(n, ctypes.c_void_p) for n in (
             "q", "k", "v", "dout", "dq", "dk", "dv", "lse", "delta", "c2p_bias", "p2c_bias", "d_c2p_bias", "d_p2c_bias",
             "seq_start", "seq_len", "delta_lut")]
-        + [(n + s, ctypes.c_int64) for n in ("q", "k", "v", "do", "dq", "dk", "dv") for s in ("_stride_b", "_stride_t", "_stride_h")]
+        + [(n + s, ctypes.c_int64) for n in ("q", "k", "v", "do", "dq", "dk", "dv", "bias") for s in ("_stride_b", "_stride_t", "_stride_h")]
         + [(n, ctypes.c_int32) for n in ("batch", "heads", "head_dim", "seqlen", "att_span", "lut_radius", "dtype", "causal")]
         + [("sm_scale", ctypes.c_float)]
     )

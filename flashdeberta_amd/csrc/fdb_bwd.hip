@@ -134,9 +134,9 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
   }
   const int S2 = 2 * p.S;
   // Position-score tensors are addressed as one base per (batch row, head) plus 32-bit element offsets
-  // (token * H * 2S + table row; the launcher checks that L * H * 2S fits).
-  const int64_t seq_base = (((int64_t)b * p.L + tok0) * p.H + h) * S2;
-  const uint32_t row_elems = (uint32_t)p.H * (uint32_t)S2;           // elements between neighbouring tokens
+  // (token * row stride + table row; the entry point checks that L * row stride fits).
+  const int64_t seq_base = (int64_t)b * p.bias_sb + (int64_t)tok0 * p.bias_st + (int64_t)h * p.bias_sh;
+  const uint32_t row_elems = (uint32_t)p.bias_st;                     // elements between neighbouring tokens
   const uint32_t x_off = (uint32_t)(x_ok ? xr : 0) * row_elems;      // this lane's row
   // Score gradients of the lane side's tensor: ring rows of this wave in LDS, rows of this wave in the tensor.
   constexpr bool kGrad = kDQ ? C2P : P2C;

@@ -45,8 +45,8 @@ struct FdbKParams {
   float scale_log2; // sm_scale * log2(e)
 };
 
-// Backward launch (fdb_bwd.hip): fixed layout only.  Position scores and their gradients are fp32
-// [B, L, H, 2S] (token-major like lse); lse / delta are fp32 [B*L, H].
+// Backward launch (fdb_bwd.hip): fixed layout only.  Position scores and their gradients are fp32, element
+// (b, l, h, delta) at b * bias_sb + l * bias_st + h * bias_sh + delta; lse / delta are fp32 [B*L, H].
 struct FdbBwdParams {
   const char* q;
   const char* k;
@@ -59,7 +59,7 @@ struct FdbBwdParams {
   const float* delta;   // sum_d dO * O per row
   const float* c2p;     // q_i . K_r[delta] or NULL
   const float* p2c;     // k_j . Q_r[delta] or NULL
-  float* d_c2p;         // zero-initialised by the caller; scatter-added
+  float* d_c2p;         // zero-initialised by the caller; touched entries are stored once
   float* d_p2c;
   const int32_t* seq_start;
   const int32_t* seq_len;
@@ -71,6 +71,7 @@ struct FdbBwdParams {
   int64_t dq_sb, dq_st, dq_sh;
   int64_t dk_sb, dk_st, dk_sh;
   int64_t dv_sb, dv_st, dv_sh;
+  int64_t bias_sb, bias_st, bias_sh;
   int32_t B, H, L;
   int32_t S;        // att_span
   int32_t R;        // table radius

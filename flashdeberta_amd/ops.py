@@ -236,13 +236,24 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
     return (out, lse) if return_lse else out
 
 
+def _scores_f32(x, pos_t):
+    """x [H, N, D] . pos_t [H, D, 2S] -> fp32 [H, N, 2S].  16-bit operands go through the GEMM as they are, with an
+    fp32 result (exactly what converting them first would give, at half the traffic), where torch offers that."""
+    if x.dtype != torch.float32:
+        try:
+            return torch.bmm(x, pos_t.to(x.dtype), out_dtype=torch.float32)
+        except (TypeError, RuntimeError, NotImplementedError):
+            pass
+    return torch.bmm(x.to(torch.float32), pos_t.to(torch.float32))
+
+
 def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=None, *, sm_scale=None, position_buckets=0,
                                max_relative_positions=0, causal=False, seq_start=None, seq_len=None):
     """Backward of the fixed layout: q, k, v, out, dout [B, L, H, D], lse [B*L, H] as the forward returns it,
     pos_key = K_r / pos_query = Q_r [H, 2S, D] or None  ->  (dq, dk, dv, d pos_key, d pos_query).
     Counterpart of FlashAttentionDisentangled.backward (reference flash_attention.py:1066-1086), which hands
     flash_attn_v2_bwd_dise the position-score tensors and gets their gradients back; as there, those tensors
-    are two GEMMs around the kernel (here fp32 [B, L, H, 2S]) and the chain through K_r / Q_r and back into
+    are two GEMMs around the kernel (here fp32, head-major [H, B*L, 2S]) and the chain through K_r / Q_r and back into
     q / k is four more."""
     B, L, H, D = q.shape
     if q.dtype not in _DTYPES:
@@ -256,17 +267,21 @@ def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=
     a = _lib.FdbAttnBwdArgs()
     f32 = torch.float32
     c2p = p2c = d_c2p = d_p2c = None
+    # Position scores and their gradients are head-major, [H, B*L, 2S] fp32: what a batched GEMM over the heads
+    # writes and reads as it stands (a token-major tensor would cost a transposing copy of it each way).
+    heads_first = lambda x: x.permute(2, 0, 1, 3).reshape(H, B * L, D)  # a view of [B, L, H, D] when that is contiguous
     if pos_key is not None or pos_query is not None:
         lut, radius = delta_lut_device(position_buckets, max_relative_positions, q.device)
         a.delta_lut, a.lut_radius, a.att_span = lut.data_ptr(), radius, span
+        a.bias_stride_b, a.bias_stride_t, a.bias_stride_h = L * 2 * span, 2 * span, B * L * 2 * span
     if pos_key is not None:
-        pk32 = pos_key[:, :2 * span].to(f32)
-        c2p = torch.einsum("blhd,hsd->blhs", q.to(f32), pk32).contiguous()
+        qh, pk_t = heads_first(q), pos_key[:, :2 * span].transpose(1, 2)
+        c2p = _scores_f32(qh, pk_t)                              # [H, B*L, 2S] = q . K_r^T
         d_c2p = torch.zeros_like(c2p)
         a.c2p_bias, a.d_c2p_bias = c2p.data_ptr(), d_c2p.data_ptr()
     if pos_query is not None:
-        pq32 = pos_query[:, :2 * span].to(f32)
-        p2c = torch.einsum("blhd,hsd->blhs", k.to(f32), pq32).contiguous()
+        kh, pq_t = heads_first(k), pos_query[:, :2 * span].transpose(1, 2)
+        p2c = _scores_f32(kh, pq_t)
         d_p2c = torch.zeros_like(p2c)
         a.p2c_bias, a.d_p2c_bias = p2c.data_ptr(), d_p2c.data_ptr()
     delta = (dout.to(f32) * out.to(f32)).sum(dim=-1).contiguous()  # [B, L, H]
@@ -291,16 +306,20 @@ def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=
     with torch.cuda.device(q.device):
         check(lib.fdb_attn_bwd(ctypes.byref(a), _stream_ptr(q.device)), "fdb_attn_bwd")
     dpk = dpq = None
-    if pos_key is not None:  # score = q . K_r[delta]: both factors get their share
-        dq = (dq.to(f32) + torch.einsum("blhs,hsd->blhd", d_c2p, pk32)).to(q.dtype)
-        dpk = torch.zeros(pos_key.shape, dtype=f32, device=q.device)
-        dpk[:, :2 * span] = torch.einsum("blhs,blhd->hsd", d_c2p, q.to(f32))
-        dpk = dpk.to(pos_key.dtype)
+
+    def chain(d_scores, x, pos, dx):
+        """score = x . pos[delta]: both factors get their share.  d_scores [H, B*L, 2S] fp32."""
+        pos32 = pos[:, :2 * span].to(f32)
+        extra = torch.bmm(d_scores, pos32).view(H, B, L, D).permute(1, 2, 0, 3)          # into x: [B, L, H, D]
+        dx = (dx.to(f32) + extra).to(x.dtype)
+        dpos = torch.zeros(pos.shape, dtype=f32, device=x.device)
+        dpos[:, :2 * span] = torch.bmm(d_scores.transpose(1, 2), heads_first(x).to(f32))  # into pos: [H, 2S, D]
+        return dx, dpos.to(pos.dtype)
+
+    if pos_key is not None:
+        dq, dpk = chain(d_c2p, q, pos_key, dq)
     if pos_query is not None:
-        dk = (dk.to(f32) + torch.einsum("blhs,hsd->blhd", d_p2c, pq32)).to(k.dtype)
-        dpq = torch.zeros(pos_query.shape, dtype=f32, device=q.device)
-        dpq[:, :2 * span] = torch.einsum("blhs,blhd->hsd", d_p2c, k.to(f32))
-        dpq = dpq.to(pos_query.dtype)
+        dk, dpq = chain(d_p2c, k, pos_query, dk)
     return dq, dk, dv, dpk, dpq
 
 

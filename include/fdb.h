@@ -37,7 +37,7 @@ extern "C" {
 #endif
 
 /* bumped whenever fdb_attn_args or the meaning of an entry point changes: a binding checks it next to the struct size */
-#define FDB_VERSION 5
+#define FDB_VERSION 6
 
 /* element types of q/k/pos_key/pos_query (v and out: see fdb_attn_args.dtype) */
 enum fdb_dtype {
@@ -155,10 +155,14 @@ int fdb_attn_fwd_noalloc(const fdb_attn_args* a, void* stream);
  * Backward, fixed layout (optionally with seq_start / seq_len).  Replaces flash_attn_v2_bwd_dise and the three
  * kernels it launches (src/flashdeberta/ops/flash_attention.py:942-1030, :62-141, :581-941), called from
  * FlashAttentionDisentangled.backward (:1066-1086).  Same division of labour as there: the position scores come
- * in as tensors, c2p_bias[b,l,h,delta] = q . K_r[delta] and p2c_bias[b,l,h,delta] = k . Q_r[delta] (fp32,
- * [B, L, H, 2S] contiguous; the reference: [B,H,L,2S] in the input dtype), and the gradients with respect to them
- * leave in d_c2p_bias / d_p2c_bias (same shape, fp32, ZEROED BY THE CALLER: they are scatter-added); the chain
- * through K_r / Q_r and into q / k is the caller's GEMMs.  dq, dk, dv hold only the content part,
+ * in as tensors, c2p_bias[b,l,h,delta] = q . K_r[delta] and p2c_bias[b,l,h,delta] = k . Q_r[delta] (fp32; the
+ * reference: [B,H,L,2S] in the input dtype), and the gradients with respect to them leave in d_c2p_bias /
+ * d_p2c_bias (fp32, ZEROED BY THE CALLER: an entry is stored once, by plain stores, if any score maps to it and
+ * not touched otherwise).  The four tensors share one layout: element (b, l, h, delta) at
+ * b * bias_stride_b + l * bias_stride_t + h * bias_stride_h + delta (strides in elements; l * bias_stride_t
+ * + delta must stay below 2^31).  Head-major [H, B, L, 2S] is what a batched GEMM over the heads writes and
+ * reads without a transpose.  The chain through K_r / Q_r and into q / k is the caller's GEMMs.
+ * dq, dk, dv hold only the content part,
  *   dq_i = sum_j dS_ij k_j,  dk_j = sum_i dS_ij q_i,  dv_j = sum_i P_ij dO_i,  dS = P (dO V^T - delta) sm_scale,
  * with P recomputed from lse (the forward's log-sum-exp, [B*L, H]) and delta[row] = sum_d dO * O ([B*L, H] fp32).
  * Rows outside [seq_start, seq_start + seq_len) are not written.  q, k, v, dout, dq, dk, dv: element type of
@@ -188,6 +192,7 @@ typedef struct fdb_attn_bwd_args {
   int64_t dq_stride_b, dq_stride_t, dq_stride_h;
   int64_t dk_stride_b, dk_stride_t, dk_stride_h;
   int64_t dv_stride_b, dv_stride_t, dv_stride_h;
+  int64_t bias_stride_b, bias_stride_t, bias_stride_h;   /* of c2p_bias, p2c_bias, d_c2p_bias, d_p2c_bias */
   int32_t batch;
   int32_t heads;
   int32_t head_dim;

@@ -33,7 +33,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_struct_mirror_and_version():
     assert lib.fdb_attn_args_size() == ctypes.sizeof(FdbAttnArgs)
-    assert lib.fdb_version() == _lib.FDB_VERSION == 5
+    assert lib.fdb_version() == _lib.FDB_VERSION == 6
     assert lib.fdb_tile_rows() == 128
 
 
