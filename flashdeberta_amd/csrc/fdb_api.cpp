@@ -391,6 +391,9 @@ int fdb_attn_bwd(const fdb_attn_bwd_args* a, void* stream) {
   // the kernels address a sequence's rows of the position-score tensors with 32-bit element offsets
   if (has_pos && (a->bias_stride_t < 2 * a->att_span || a->bias_stride_b < 0 || a->bias_stride_h < 0 ||
                   (int64_t)a->seqlen * a->bias_stride_t > 0x7fffffffll)) return FDB_ERR_SHAPE;
+  // score gradients leave in aligned groups of four entries
+  if (has_pos && ((a->att_span & 1) || (a->bias_stride_b & 3) || (a->bias_stride_t & 3) || (a->bias_stride_h & 3) ||
+                  !aligned16(a->d_c2p_bias) || !aligned16(a->d_p2c_bias))) return FDB_ERR_ALIGN;
   const int sz = qk_elem_size(a->dtype);
   const void* ptrs[] = {a->q, a->k, a->v, a->dout, a->dq, a->dk, a->dv};
   for (const void* ptr : ptrs)
@@ -406,7 +409,7 @@ int fdb_attn_bwd(const fdb_attn_bwd_args* a, void* stream) {
   p.q = (const char*)a->q; p.k = (const char*)a->k; p.v = (const char*)a->v; p.dout = (const char*)a->dout;
   p.dq = (char*)a->dq; p.dk = (char*)a->dk; p.dv = (char*)a->dv;
   p.lse = a->lse; p.delta = a->delta;
-  p.c2p = a->c2p_bias; p.p2c = a->p2c_bias; p.d_c2p = a->d_c2p_bias; p.d_p2c = a->d_p2c_bias;
+  p.c2p = a->c2p_bias; p.p2c = a->p2c_bias; p.d_c2p = (char*)a->d_c2p_bias; p.d_p2c = (char*)a->d_p2c_bias;
   p.bias_sb = a->bias_stride_b; p.bias_st = a->bias_stride_t; p.bias_sh = a->bias_stride_h;
   p.seq_start = a->seq_start; p.seq_len = a->seq_len; p.lut = a->delta_lut;
   p.q_sb = a->q_stride_b; p.q_st = a->q_stride_t; p.q_sh = a->q_stride_h;

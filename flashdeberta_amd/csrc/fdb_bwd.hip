@@ -17,9 +17,10 @@
 // Score gradients without atomics.  Each role owns the tensor of its lane side (dQ role: d c2p, a row per query;
 // dK/dV role: d p2c, a row per key).  The table row delta(i - j) is monotone in the loop row with steps of 0 or 1, so
 // the entries a lane row can still receive form a window of at most 33 neighbours that slides one way as the loop
-// advances: a 64-entry ring per row in LDS takes the adds (ds_add_f32), and the entries the window has left behind
-// are stored once, row by row with the lanes on neighbouring entries, and cleared.  The tensors arrive zeroed;
-// entries no element maps to are never written.  Results do not depend on the order workgroups run in.
+// advances: a 64-entry ring per row in LDS takes the adds, and the entries the window has left behind are stored
+// once, in aligned groups of four (eight lanes per row, one 16- or 8-byte store each), and cleared.  The tensors have
+// the element type of q and arrive zeroed; entries no element maps to are written as zeros or not at all.  Results
+// do not depend on the order workgroups run in.
 // A step whose relative positions all lie beyond the table radius has one table row: its position scores are
 // one load per row and its score gradients enter the ring as one row sum per lane.
 #include <hip/hip_runtime.h>
@@ -49,8 +50,8 @@ struct BCfg {
   static constexpr int RS = D * QT::SZ + 16;                 // LDS row stride of a staged tile
   static constexpr int TILE = kBwdStep * RS;
   static constexpr int CHUNKS = (kBwdStep * D * QT::SZ / 16 + kBwdThreads - 1) / kBwdThreads;  // 16-byte chunks per thread
-  // two tile buffers, loop-row statistics, ring windows, far-step scores; the table follows
-  static constexpr int fixed_lds_bytes() { return 4 * TILE + 4 * kBwdStep * 4 + FDB_BM * kRingStrideMax * 4 + FDB_BM * 4; }
+  // two tile buffers, loop-row statistics, ring windows, far-step scores, groups to store; the table follows
+  static constexpr int fixed_lds_bytes() { return 4 * TILE + 4 * kBwdStep * 4 + FDB_BM * kRingStrideMax * 4 + FDB_BM * 4 + FDB_BM * 8; }
   static int lds_bytes(int radius) { return fixed_lds_bytes() + (((2 * radius + 1) * 2 + 15) & ~15); }
 };
 
@@ -88,7 +89,8 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
   float* stat_s = (float*)(Ys + 4 * C::TILE);         // dK/dV role: per buffer, log-sum-exp (base 2) and Delta of the 32 loop rows
   float* ring_s = stat_s + 4 * kBwdStep;              // [128 lane-side rows][kRingStride] score-gradient windows
   float* vec_s = ring_s + FDB_BM * kRingStrideMax;      // [4 waves][32] loop-side position scores of a far step
-  LDS_AS int16_t* lut_s = (LDS_AS int16_t*)(vec_s + FDB_BM);  // the whole table (the launcher sizes the allocation for it)
+  int2* inf_s = (int2*)(vec_s + FDB_BM);              // [4 waves][32] (first group, groups) to store per row
+  LDS_AS int16_t* lut_s = (LDS_AS int16_t*)(inf_s + FDB_BM);  // the whole table (the launcher sizes the allocation for it)
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -143,12 +145,14 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
   float* ring_w = ring_s + wave * 32 * kRingStride;
   float* ring_x = ring_w + li * kRingStride;
   float* vec_w = vec_s + wave * 32;
-  float* gw = nullptr;
+  int2* inf_w = inf_s + wave * 32;
+  char* gw = nullptr;   // this sequence and head of the gradient tensor (elements of the input type)
   if (kGrad) {
-    gw = (kDQ ? p.d_c2p : p.d_p2c) + seq_base;
+    gw = (kDQ ? p.d_c2p : p.d_p2c) + seq_base * QT::SZ;
     for (int e = lane; e < 32 * kRingStride; e += 64) ring_w[e] = 0.f;
   }
   constexpr int kDir = kDQ ? -1 : 1;        // the way the window moves as the loop row grows
+  int g_next = 0;                           // next group of four entries of this lane's row to store
 
   f32x16 acc1[DBLKS], acc2[DBLKS];  // dQ^T (dQ role) / dK^T and dV^T (dK/dV role)
 #pragma unroll
@@ -228,6 +232,7 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
   if (y_lo < y_hi) {
     tiles_load(y_lo);
     __syncthreads();  // the table is in LDS
+    if (kGrad) g_next = delta_of(kDQ ? xr - y_lo : y_lo - xr) >> 2;
     request(y_lo);
     tiles_store(0);
   }
@@ -319,32 +324,39 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
           wave_lds_fence();
         }
       }
-      // Entries behind the window: from the table row of this step's first loop row up to (not including) that of
-      // the next step's first loop row, at most 32; after the last step, the 32 entries the step can have touched.
-      const int d_first = delta_of(kDQ ? xr - y0 : y0 - xr);
-      const int n_out = !x_ok ? 0 : !has_next ? 32 : kDir * (delta_of(kDQ ? xr - (y0 + kBwdStep) : y0 + kBwdStep - xr) - d_first);
-      if (__builtin_amdgcn_ballot_w64(n_out > 0) != 0) {
-        // A half-wave per row, its lanes on neighbouring entries: one store instruction writes two runs of up to 128
-        // bytes.  The bounds of row rho sit in lane rho; all sixteen reads are under way before the first is used.
-        float val[16];
-        int dd[16];
-        bool act[16];
+      // Groups of four entries [4m, 4m + 3] the window has left behind: every later element of the row maps to a
+      // table row at or beyond `d_edge` (that of the next step's first loop row; after the last step, the last
+      // row's own entry, and its group goes too).  Up to eight groups per row and pass.
+      const int d_edge = delta_of(has_next ? (kDQ ? xr - (y0 + kBwdStep) : y0 + kBwdStep - xr) : (kDQ ? xr - (y_hi - 1) : y_hi - 1 - xr));
+      int n_g = !x_ok ? 0 : kDir * ((d_edge >> 2) - g_next) + (has_next ? 0 : 1);
+      while (__builtin_amdgcn_ballot_w64(n_g > 0) != 0) {
+        const int n_now = max(0, min(n_g, 8));
+        if (g == 0) inf_w[li] = int2{g_next, n_now};
+        wave_lds_fence();
+        f32x4 val[4];
+        int mm[4];
+        bool act[4];
 #pragma unroll
-        for (int it = 0; it < 16; ++it) {
-          const int f0 = __builtin_amdgcn_readlane(d_first, 2 * it), f1 = __builtin_amdgcn_readlane(d_first, 2 * it + 1);
-          const int n0 = __builtin_amdgcn_readlane(n_out, 2 * it), n1 = __builtin_amdgcn_readlane(n_out, 2 * it + 1);
-          dd[it] = (g ? f1 : f0) + kDir * li;
-          act[it] = li < (g ? n1 : n0);
-          val[it] = ring_w[(2 * it + g) * kRingStride + (dd[it] & (kRing - 1))];
+        for (int it = 0; it < 4; ++it) {
+          const int rho = 8 * it + (lane >> 3);
+          const int2 inf = inf_w[rho];
+          mm[it] = inf.x + kDir * (lane & 7);
+          act[it] = (lane & 7) < inf.y;
+          const float* e = ring_w + rho * kRingStride + ((4 * mm[it]) & (kRing - 1));
+          val[it] = f32x4{e[0], e[1], e[2], e[3]};
         }
 #pragma unroll
-        for (int it = 0; it < 16; ++it) {
+        for (int it = 0; it < 4; ++it) {
+          const int rho = 8 * it + (lane >> 3);
           if (act[it]) {
-            ring_w[(2 * it + g) * kRingStride + (dd[it] & (kRing - 1))] = 0.f;
-            if (val[it] != 0.f && dd[it] >= 0 && dd[it] < S2) gw[(uint32_t)(xw0 + 2 * it + g) * row_elems + (uint32_t)dd[it]] = val[it];
+            float* e = ring_w + rho * kRingStride + ((4 * mm[it]) & (kRing - 1));
+            e[0] = e[1] = e[2] = e[3] = 0.f;
+            QT::store4(gw + ((uint32_t)(xw0 + rho) * row_elems + (uint32_t)(4 * mm[it])) * QT::SZ, val[it][0], val[it][1], val[it][2], val[it][3]);
           }
         }
         wave_lds_fence();
+        g_next += kDir * n_now;
+        n_g -= n_now;
       }
     }
     // ---- outputs: contraction over the loop rows, which are the accumulator registers ------------------------------

@@ -59,8 +59,8 @@ struct FdbBwdParams {
   const float* delta;   // sum_d dO * O per row
   const float* c2p;     // q_i . K_r[delta] or NULL
   const float* p2c;     // k_j . Q_r[delta] or NULL
-  float* d_c2p;         // zero-initialised by the caller; touched entries are stored once
-  float* d_p2c;
+  char* d_c2p;          // element type of q; zero-initialised by the caller; touched entries are stored once
+  char* d_p2c;
   const int32_t* seq_start;
   const int32_t* seq_len;
   const int16_t* lut;

@@ -237,8 +237,8 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
 
 
 def _scores_f32(x, pos_t):
-    """x [H, N, D] . pos_t [H, D, 2S] -> fp32 [H, N, 2S].  16-bit operands go through the GEMM as they are, with an
-    fp32 result (exactly what converting them first would give, at half the traffic), where torch offers that."""
+    """Batched x [H, N, K] . pos_t [H, K, M] -> fp32 [H, N, M].  16-bit operands go through the GEMM as they are, with
+    an fp32 result (exactly what converting them first would give, at half the traffic), where torch offers that."""
     if x.dtype != torch.float32:
         try:
             return torch.bmm(x, pos_t.to(x.dtype), out_dtype=torch.float32)
@@ -277,12 +277,12 @@ def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=
     if pos_key is not None:
         qh, pk_t = heads_first(q), pos_key[:, :2 * span].transpose(1, 2)
         c2p = _scores_f32(qh, pk_t)                              # [H, B*L, 2S] = q . K_r^T
-        d_c2p = torch.zeros_like(c2p)
+        d_c2p = torch.zeros_like(c2p, dtype=q.dtype)            # gradient tensors: the inputs' type, as in the reference
         a.c2p_bias, a.d_c2p_bias = c2p.data_ptr(), d_c2p.data_ptr()
     if pos_query is not None:
         kh, pq_t = heads_first(k), pos_query[:, :2 * span].transpose(1, 2)
         p2c = _scores_f32(kh, pq_t)
-        d_p2c = torch.zeros_like(p2c)
+        d_p2c = torch.zeros_like(p2c, dtype=q.dtype)
         a.p2c_bias, a.d_p2c_bias = p2c.data_ptr(), d_p2c.data_ptr()
     delta = (dout.to(f32) * out.to(f32)).sum(dim=-1).contiguous()  # [B, L, H]
     lse = lse.contiguous()
@@ -308,12 +308,11 @@ def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=
     dpk = dpq = None
 
     def chain(d_scores, x, pos, dx):
-        """score = x . pos[delta]: both factors get their share.  d_scores [H, B*L, 2S] fp32."""
-        pos32 = pos[:, :2 * span].to(f32)
-        extra = torch.bmm(d_scores, pos32).view(H, B, L, D).permute(1, 2, 0, 3)          # into x: [B, L, H, D]
+        """score = x . pos[delta]: both factors get their share.  d_scores [H, B*L, 2S] in the inputs' type."""
+        extra = _scores_f32(d_scores, pos[:, :2 * span]).view(H, B, L, D).permute(1, 2, 0, 3)   # into x: [B, L, H, D]
         dx = (dx.to(f32) + extra).to(x.dtype)
         dpos = torch.zeros(pos.shape, dtype=f32, device=x.device)
-        dpos[:, :2 * span] = torch.bmm(d_scores.transpose(1, 2), heads_first(x).to(f32))  # into pos: [H, 2S, D]
+        dpos[:, :2 * span] = _scores_f32(d_scores.transpose(1, 2), heads_first(x))              # into pos: [H, 2S, D]
         return dx, dpos.to(pos.dtype)
 
     if pos_key is not None:
