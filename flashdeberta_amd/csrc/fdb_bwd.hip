@@ -284,12 +284,20 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
     if (has_next) request(y0 + kBwdStep);
     float ds[16], ds_run[16], pr[16], g_sum = 0.f;
     bool ok[16];
+    f32x4 lse4[4], del4[4];  // dK/dV role: statistics of this lane's 16 loop rows, four neighbours per read
+    if (!kDQ) {
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        lse4[q4] = *(const f32x4*)(lse_s + 8 * q4 + 4 * g);
+        del4[q4] = *(const f32x4*)(del_s + 8 * q4 + 4 * g);
+      }
+    }
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
       const int yl = 8 * (v >> 2) + 4 * g + (v & 3), yr = y0 + yl;
       const int i = kDQ ? xr : yr, j = kDQ ? yr : xr;
       ok[v] = x_ok && yr < Lb && (!p.causal || j <= i);
-      const float lse_i = kDQ ? lse_x : lse_s[yl], del_i = kDQ ? del_x : del_s[yl];
+      const float lse_i = kDQ ? lse_x : lse4[v >> 2][v & 3], del_i = kDQ ? del_x : del4[v >> 2][v & 3];
       const float pv = ok[v] ? __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[v] + bias[v], c_log2, -lse_i)) : 0.f;
       pr[v] = pv;
       ds[v] = pv * (dpacc[v] - del_i) * c_sm;
