@@ -35,9 +35,9 @@ class FdbAttnArgs(ctypes.Structure):
 class FdbAttnBwdArgs(ctypes.Structure):
     _fields_ = (
         [(n, ctypes.c_void_p) for n in (
-            "q", "k", "v", "dout", "dq", "dk", "dv", "lse", "delta", "c2p_bias", "p2c_bias", "d_c2p_bias", "d_p2c_bias",
+            "q", "k", "v", "dout", "dq", "dk", "dv", "lse", "delta", "out", "c2p_bias", "p2c_bias", "d_c2p_bias", "d_p2c_bias",
             "seq_start", "seq_len", "delta_lut")]
-        + [(n + s, ctypes.c_int64) for n in ("q", "k", "v", "do", "dq", "dk", "dv", "bias") for s in ("_stride_b", "_stride_t", "_stride_h")]
+        + [(n + s, ctypes.c_int64) for n in ("q", "k", "v", "do", "out", "dq", "dk", "dv", "bias") for s in ("_stride_b", "_stride_t", "_stride_h")]
         + [(n, ctypes.c_int32) for n in ("batch", "heads", "head_dim", "seqlen", "att_span", "lut_radius", "dtype", "causal")]
         + [("sm_scale", ctypes.c_float)]
     )

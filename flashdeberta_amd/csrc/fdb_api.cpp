@@ -395,20 +395,22 @@ int fdb_attn_bwd(const fdb_attn_bwd_args* a, void* stream) {
   if (has_pos && ((a->att_span & 1) || (a->bias_stride_b & 3) || (a->bias_stride_t & 3) || (a->bias_stride_h & 3) ||
                   !aligned16(a->d_c2p_bias) || !aligned16(a->d_p2c_bias))) return FDB_ERR_ALIGN;
   const int sz = qk_elem_size(a->dtype);
-  const void* ptrs[] = {a->q, a->k, a->v, a->dout, a->dq, a->dk, a->dv};
+  const void* ptrs[] = {a->q, a->k, a->v, a->dout, a->dq, a->dk, a->dv, a->out};
   for (const void* ptr : ptrs)
     if (!aligned16(ptr)) return FDB_ERR_ALIGN;
   const int64_t strides[] = {a->q_stride_b, a->q_stride_t, a->q_stride_h, a->k_stride_b, a->k_stride_t, a->k_stride_h,
                              a->v_stride_b, a->v_stride_t, a->v_stride_h, a->do_stride_b, a->do_stride_t, a->do_stride_h,
                              a->dq_stride_b, a->dq_stride_t, a->dq_stride_h, a->dk_stride_b, a->dk_stride_t, a->dk_stride_h,
-                             a->dv_stride_b, a->dv_stride_t, a->dv_stride_h};
+                             a->dv_stride_b, a->dv_stride_t, a->dv_stride_h,
+                             a->out ? a->out_stride_b : 0, a->out ? a->out_stride_t : 0, a->out ? a->out_stride_h : 0};
   for (int64_t st : strides)
     if ((st * sz) % 16 != 0) return FDB_ERR_ALIGN;
   FdbBwdParams p;
   memset(&p, 0, sizeof(p));
   p.q = (const char*)a->q; p.k = (const char*)a->k; p.v = (const char*)a->v; p.dout = (const char*)a->dout;
   p.dq = (char*)a->dq; p.dk = (char*)a->dk; p.dv = (char*)a->dv;
-  p.lse = a->lse; p.delta = a->delta;
+  p.lse = a->lse; p.delta = a->delta; p.out = (const char*)a->out;
+  p.o_sb = a->out_stride_b; p.o_st = a->out_stride_t; p.o_sh = a->out_stride_h;
   p.c2p = a->c2p_bias; p.p2c = a->p2c_bias; p.d_c2p = (char*)a->d_c2p_bias; p.d_p2c = (char*)a->d_p2c_bias;
   p.bias_sb = a->bias_stride_b; p.bias_st = a->bias_stride_t; p.bias_sh = a->bias_stride_h;
   p.seq_start = a->seq_start; p.seq_len = a->seq_len; p.lut = a->delta_lut;

@@ -130,9 +130,25 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
   // row statistics and position-score rows are token-major: row (b, tok0 + l), head h
   const int64_t tok_x = ((int64_t)b * p.L + tok0 + (x_ok ? xr : 0)) * p.H + h;
   float lse_x = 0.f, del_x = 0.f;
-  if (kDQ && x_ok) {
-    lse_x = p.lse[tok_x] * 1.4426950408889634f;
-    del_x = p.delta[tok_x];
+  if (kDQ) {
+    if (p.out != nullptr) {
+      // delta = dO . O of this lane's row (the reference's _bwd_preprocess): each half-wave has half of the row;
+      // left in p.delta for the dK/dV launch, which follows this one on the stream
+      const char* ob = base(p.out, p.o_sb, p.o_st, p.o_sh);
+      float dot = 0.f;
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        const f32x8 o8 = QT::to_f32(x_ok ? QT::load(ob + ((int64_t)xr * p.o_st + 16 * s + 8 * g) * QT::SZ) : QT::zero());
+        const f32x8 g8 = QT::to_f32(x2f[s]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) dot = __builtin_fmaf(o8[e], g8[e], dot);
+      }
+      del_x = wave_half_sum(dot);
+      if (x_ok && g == 0) p.delta[tok_x] = del_x;
+    } else if (x_ok) {
+      del_x = p.delta[tok_x];
+    }
+    if (x_ok) lse_x = p.lse[tok_x] * 1.4426950408889634f;
   }
   const int S2 = 2 * p.S;
   // Position-score tensors are addressed as one base per (batch row, head) plus 32-bit element offsets

@@ -56,7 +56,8 @@ struct FdbBwdParams {
   char* dk;
   char* dv;
   const float* lse;
-  const float* delta;   // sum_d dO * O per row
+  float* delta;         // sum_d dO * O per row: read, or written by the dQ role when `out` is given
+  const char* out;      // the forward's output or NULL
   const float* c2p;     // q_i . K_r[delta] or NULL
   const float* p2c;     // k_j . Q_r[delta] or NULL
   char* d_c2p;          // element type of q; zero-initialised by the caller; touched entries are stored once
@@ -68,6 +69,7 @@ struct FdbBwdParams {
   int64_t k_sb, k_st, k_sh;
   int64_t v_sb, v_st, v_sh;
   int64_t g_sb, g_st, g_sh;     // dout
+  int64_t o_sb, o_st, o_sh;     // out
   int64_t dq_sb, dq_st, dq_sh;
   int64_t dk_sb, dk_st, dk_sh;
   int64_t dv_sb, dv_st, dv_sh;

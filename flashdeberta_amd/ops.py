@@ -284,14 +284,15 @@ def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=
         p2c = _scores_f32(kh, pq_t)
         d_p2c = torch.zeros_like(p2c, dtype=q.dtype)
         a.p2c_bias, a.d_p2c_bias = p2c.data_ptr(), d_p2c.data_ptr()
-    delta = (dout.to(f32) * out.to(f32)).sum(dim=-1).contiguous()  # [B, L, H]
+    out = out if out.stride(-1) == 1 else out.contiguous()
+    delta = torch.empty((B * L, H), dtype=f32, device=q.device)     # dO . O per row: the dQ launch fills it
     lse = lse.contiguous()
     padded = seq_start is not None or seq_len is not None
     alloc = torch.zeros if padded else torch.empty
     dq, dk, dv = [alloc((B, L, H, D), dtype=q.dtype, device=q.device) for _ in range(3)]
     a.q, a.k, a.v, a.dout = q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr()
-    a.dq, a.dk, a.dv, a.lse, a.delta = dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), lse.data_ptr(), delta.data_ptr()
-    for n, x in (("q", q), ("k", k), ("v", v), ("do", dout), ("dq", dq), ("dk", dk), ("dv", dv)):
+    a.dq, a.dk, a.dv, a.lse, a.delta, a.out = dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), lse.data_ptr(), delta.data_ptr(), out.data_ptr()
+    for n, x in (("q", q), ("k", k), ("v", v), ("do", dout), ("out", out), ("dq", dq), ("dk", dk), ("dv", dv)):
         setattr(a, n + "_stride_b", x.stride(0))
         setattr(a, n + "_stride_t", x.stride(1))
         setattr(a, n + "_stride_h", x.stride(2))
@@ -310,10 +311,11 @@ def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=
     def chain(d_scores, x, pos, dx):
         """score = x . pos[delta]: both factors get their share.  d_scores [H, B*L, 2S] in the inputs' type."""
         extra = _scores_f32(d_scores, pos[:, :2 * span]).view(H, B, L, D).permute(1, 2, 0, 3)   # into x: [B, L, H, D]
-        dx = (dx.to(f32) + extra).to(x.dtype)
-        dpos = torch.zeros(pos.shape, dtype=f32, device=x.device)
-        dpos[:, :2 * span] = _scores_f32(d_scores.transpose(1, 2), heads_first(x))              # into pos: [H, 2S, D]
-        return dx, dpos.to(pos.dtype)
+        dx = extra.add_(dx).to(x.dtype, memory_format=torch.contiguous_format)
+        dpos = _scores_f32(d_scores.transpose(1, 2), heads_first(x)).to(pos.dtype)              # into pos: [H, 2S, D]
+        if pos.shape[1] > 2 * span:  # rows past 2S take no part
+            dpos = torch.cat([dpos, dpos.new_zeros(H, pos.shape[1] - 2 * span, D)], dim=1)
+        return dx, dpos
 
     if pos_key is not None:
         dq, dpk = chain(d_c2p, q, pos_key, dq)

@@ -165,7 +165,9 @@ int fdb_attn_fwd_noalloc(const fdb_attn_args* a, void* stream);
  * heads writes and reads without a transpose.  The chain through K_r / Q_r and into q / k is the caller's GEMMs.
  * dq, dk, dv hold only the content part,
  *   dq_i = sum_j dS_ij k_j,  dk_j = sum_i dS_ij q_i,  dv_j = sum_i P_ij dO_i,  dS = P (dO V^T - delta) sm_scale,
- * with P recomputed from lse (the forward's log-sum-exp, [B*L, H]) and delta[row] = sum_d dO * O ([B*L, H] fp32).
+ * with P recomputed from lse (the forward's log-sum-exp, [B*L, H]) and delta[row] = sum_d dO * O ([B*L, H] fp32;
+ * the reference's _bwd_preprocess, :62-141).  With `out` (the forward's output, strides like q) the call computes
+ * delta itself and leaves it in `delta`; with out == NULL it reads `delta` as given.
  * Rows outside [seq_start, seq_start + seq_len) are not written.  q, k, v, dout, dq, dk, dv: element type of
  * `dtype` (fp32 / bf16 / fp16), layout and strides as in fdb_attn_args.
  */
@@ -178,7 +180,8 @@ typedef struct fdb_attn_bwd_args {
   void* dk;
   void* dv;
   const float* lse;
-  const float* delta;
+  float* delta;            /* [B*L, H] fp32: written when `out` is given, read otherwise */
+  const void* out;         /* the forward's output or NULL */
   const float* c2p_bias;   /* or NULL: no content->position term */
   const float* p2c_bias;   /* or NULL: no position->content term */
   void* d_c2p_bias;        /* required with c2p_bias; elements of `dtype` */
@@ -190,6 +193,7 @@ typedef struct fdb_attn_bwd_args {
   int64_t k_stride_b, k_stride_t, k_stride_h;
   int64_t v_stride_b, v_stride_t, v_stride_h;
   int64_t do_stride_b, do_stride_t, do_stride_h;
+  int64_t out_stride_b, out_stride_t, out_stride_h;
   int64_t dq_stride_b, dq_stride_t, dq_stride_h;
   int64_t dk_stride_b, dk_stride_t, dk_stride_h;
   int64_t dv_stride_b, dv_stride_t, dv_stride_h;
