@@ -248,13 +248,14 @@ def _scores_f32(x, pos_t):
 
 
 def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=None, *, sm_scale=None, position_buckets=0,
-                               max_relative_positions=0, causal=False, seq_start=None, seq_len=None):
+                               max_relative_positions=0, causal=False, seq_start=None, seq_len=None, delta=None):
     """Backward of the fixed layout: q, k, v, out, dout [B, L, H, D], lse [B*L, H] as the forward returns it,
     pos_key = K_r / pos_query = Q_r [H, 2S, D] or None  ->  (dq, dk, dv, d pos_key, d pos_query).
     Counterpart of FlashAttentionDisentangled.backward (reference flash_attention.py:1066-1086), which hands
     flash_attn_v2_bwd_dise the position-score tensors and gets their gradients back; as there, those tensors
     are two GEMMs around the kernel (here fp32, head-major [H, B*L, 2S]) and the chain through K_r / Q_r and back into
-    q / k is four more."""
+    q / k is four more.  delta: (dout * out).sum(-1) as fp32 [B*L, H] if the caller has it (then `out` is not
+    read); by default the first launch computes it."""
     B, L, H, D = q.shape
     if q.dtype not in _DTYPES:
         raise ValueError("unsupported dtype %s" % q.dtype)
@@ -284,15 +285,21 @@ def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=
         p2c = _scores_f32(kh, pq_t)
         d_p2c = torch.zeros_like(p2c, dtype=q.dtype)
         a.p2c_bias, a.d_p2c_bias = p2c.data_ptr(), d_p2c.data_ptr()
-    out = out if out.stride(-1) == 1 else out.contiguous()
-    delta = torch.empty((B * L, H), dtype=f32, device=q.device)     # dO . O per row: the dQ launch fills it
+    if delta is None:
+        out = out if out.stride(-1) == 1 else out.contiguous()
+        delta = torch.empty((B * L, H), dtype=f32, device=q.device)  # dO . O per row: the dQ launch fills it
+    else:
+        out, delta = None, delta.to(f32).reshape(B * L, H).contiguous()
     lse = lse.contiguous()
     padded = seq_start is not None or seq_len is not None
     alloc = torch.zeros if padded else torch.empty
     dq, dk, dv = [alloc((B, L, H, D), dtype=q.dtype, device=q.device) for _ in range(3)]
     a.q, a.k, a.v, a.dout = q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr()
-    a.dq, a.dk, a.dv, a.lse, a.delta, a.out = dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), lse.data_ptr(), delta.data_ptr(), out.data_ptr()
+    a.dq, a.dk, a.dv, a.lse, a.delta = dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), lse.data_ptr(), delta.data_ptr()
+    a.out = None if out is None else out.data_ptr()
     for n, x in (("q", q), ("k", k), ("v", v), ("do", dout), ("out", out), ("dq", dq), ("dk", dk), ("dv", dv)):
+        if x is None:
+            continue
         setattr(a, n + "_stride_b", x.stride(0))
         setattr(a, n + "_stride_t", x.stride(1))
         setattr(a, n + "_stride_h", x.stride(2))

@@ -381,3 +381,13 @@ def test_bench_contract_without_a_gpu():
     assert (tv is None) == (src is None)
     t = bench.measured_traffic("v3base_L4096_B8_bf16")
     assert t is None or t > 2e8
+
+
+def test_delta_table_is_monotone_with_unit_steps():
+    """The backward keeps a sliding window of table rows per tensor row, which rests on delta(r + 1) - delta(r)
+    being 0 or 1 for every table the host builds."""
+    for pb, mr in [(256, 512), (32, 128), (0, 512), (0, 64), (8, 64), (16, 32), (256, 1024), (64, 256), (4, 16), (0, 15), (128, 4096)]:
+        lut, radius = ops.delta_lut_host(pb, mr)
+        steps = np.diff(lut.astype(np.int64))
+        assert steps.min() >= 0 and steps.max() <= 1, (pb, mr)
+        assert lut[0] >= 0 and lut[-1] <= 2 * ops.att_span(pb, mr) - 1

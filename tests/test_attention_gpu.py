@@ -924,6 +924,8 @@ BWD_CASES = [
     (1, 700, 1, 64, 256, 512, True, True, False, None),   # v3 buckets: linear + log zone + saturation
     (1, 150, 2, 32, 32, 64, True, True, False, None),
     (1, 150, 2, 128, 32, 64, True, True, False, None),
+    (1, 600, 1, 64, 0, 300, True, True, False, None),     # no buckets: 600 table rows, every block linear
+    (1, 1100, 2, 64, 256, 512, True, True, False, None),  # v3 buckets past the radius: far steps on both sides of every zone
 ]
 
 
@@ -1028,3 +1030,32 @@ def test_bad_arguments_raise():
                                        None, position_buckets=32, max_relative_positions=64)
     with pytest.raises(ValueError):
         ops.disentangled_attention_fwd(q, q, q.float())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_backward_is_reproducible_and_takes_a_given_delta(dtype):
+    """No atomics in the backward: two runs agree bit for bit.  And the call that is handed delta = sum(dO * O)
+    instead of the forward's output gives the same gradients as the one that computes it."""
+    B, L, H, D, pb, mr = 2, 333, 2, 64, 32, 64
+    q, k, v, pk, pq = [x.cuda() for x in _inputs(B, L, H, D, pb, mr, dtype, 4100, 1.0, True, True)]
+    dout = torch.randn(B, L, H, D, generator=torch.Generator().manual_seed(4101)).to(dtype).cuda()
+    kw = dict(position_buckets=pb, max_relative_positions=mr)
+    out, lse = ops.disentangled_attention_fwd(q, k, v, pk, pq, return_lse=True, **kw)
+    first = ops.disentangled_attention_bwd(q, k, v, out, lse, dout, pk, pq, **kw)
+    again = ops.disentangled_attention_bwd(q, k, v, out, lse, dout, pk, pq, **kw)
+    for a, b in zip(first, again):
+        assert torch.equal(a, b)
+    delta = (dout.float() * out.float()).sum(-1)
+    given = ops.disentangled_attention_bwd(q, k, v, out, lse, dout, pk, pq, delta=delta, **kw)
+    for n, a, b in zip(("dq", "dk", "dv", "dK_r", "dQ_r"), first, given):
+        scale = a.float().abs().max().item()
+        assert (a.float() - b.float()).abs().max().item() <= (1e-5 if dtype == torch.float32 else 2e-2) * scale, n
+
+
+def test_backward_refuses_an_odd_span():
+    """Score gradients leave in aligned groups of four entries: 2S must be a multiple of 4."""
+    B, L, H, D = 1, 64, 1, 64
+    q, k, v, pk, pq = [x.cuda() for x in _inputs(B, L, H, D, 0, 15, torch.float32, 4200, 1.0, True, True)]
+    out, lse = ops.disentangled_attention_fwd(q, k, v, pk, pq, return_lse=True, position_buckets=0, max_relative_positions=15)
+    with pytest.raises(ValueError):
+        ops.disentangled_attention_bwd(q, k, v, out, lse, torch.ones_like(out), pk, pq, position_buckets=0, max_relative_positions=15)
