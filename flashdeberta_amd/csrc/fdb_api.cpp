@@ -411,7 +411,7 @@ int fdb_attn_bwd(const fdb_attn_bwd_args* a, void* stream) {
   p.dq = (char*)a->dq; p.dk = (char*)a->dk; p.dv = (char*)a->dv;
   p.lse = a->lse; p.delta = a->delta; p.out = (const char*)a->out;
   p.o_sb = a->out_stride_b; p.o_st = a->out_stride_t; p.o_sh = a->out_stride_h;
-  p.c2p = a->c2p_bias; p.p2c = a->p2c_bias; p.d_c2p = (char*)a->d_c2p_bias; p.d_p2c = (char*)a->d_p2c_bias;
+  p.c2p = (const char*)a->c2p_bias; p.p2c = (const char*)a->p2c_bias; p.d_c2p = (char*)a->d_c2p_bias; p.d_p2c = (char*)a->d_p2c_bias;
   p.bias_sb = a->bias_stride_b; p.bias_st = a->bias_stride_t; p.bias_sh = a->bias_stride_h;
   p.seq_start = a->seq_start; p.seq_len = a->seq_len; p.lut = a->delta_lut;
   p.q_sb = a->q_stride_b; p.q_st = a->q_stride_t; p.q_sh = a->q_stride_h;

@@ -216,13 +216,14 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
   // row, lanes past the end read row 0: the loads are unconditional and only their use is masked.
   constexpr bool kBias = C2P || P2C;
   constexpr bool kLaneT = kDQ ? C2P : P2C, kLoopT = kDQ ? P2C : C2P;
-  const float* lane_t = kLaneT ? (kDQ ? p.c2p : p.p2c) + seq_base : nullptr;   // the lane side's tensor, this sequence and head
-  const float* loop_t = kLoopT ? (kDQ ? p.p2c : p.c2p) + seq_base : nullptr;   // the loop side's
-  float raw_lane[16], raw_loop[16];
+  using BT = typename QT::scratch_t;   // element type of the position-score tensors: that of q
+  const BT* lane_t = kLaneT ? (const BT*)(kDQ ? p.c2p : p.p2c) + seq_base : nullptr;   // the lane side's tensor, this sequence and head
+  const BT* loop_t = kLoopT ? (const BT*)(kDQ ? p.p2c : p.c2p) + seq_base : nullptr;   // the loop side's
+  BT raw_lane[16], raw_loop[16];   // as loaded: converting here would wait for the load
   bool far_n = false;
   int dfar_n = 0;
 #pragma unroll
-  for (int v = 0; v < 16; ++v) raw_lane[v] = raw_loop[v] = 0.f;
+  for (int v = 0; v < 16; ++v) raw_lane[v] = raw_loop[v] = (BT)0.f;
   auto loop_off = [&](int yr) __attribute__((always_inline)) -> uint32_t {
     return (uint32_t)min(yr, Lb - 1) * row_elems;
   };
@@ -280,22 +281,22 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
     float bias[16];
     if (kBias && far) {
       if (kLoopT) {
-        if (g == 0) vec_w[li] = raw_loop[0];
+        if (g == 0) vec_w[li] = (float)raw_loop[0];
         wave_lds_fence();
 #pragma unroll
         for (int q4 = 0; q4 < 4; ++q4) {
           const f32x4 t4 = *(const f32x4*)(vec_w + 8 * q4 + 4 * g);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) bias[4 * q4 + e] = t4[e] + raw_lane[0];
+          for (int e = 0; e < 4; ++e) bias[4 * q4 + e] = t4[e] + (float)raw_lane[0];
         }
         wave_lds_fence();
       } else {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) bias[v] = raw_lane[0];
+        for (int v = 0; v < 16; ++v) bias[v] = (float)raw_lane[0];
       }
     } else {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) bias[v] = raw_lane[v] + raw_loop[v];
+      for (int v = 0; v < 16; ++v) bias[v] = (float)raw_lane[v] + (float)raw_loop[v];
     }
     if (has_next) request(y0 + kBwdStep);
     float ds[16], ds_run[16], pr[16], g_sum = 0.f;

@@ -45,7 +45,7 @@ struct FdbKParams {
   float scale_log2; // sm_scale * log2(e)
 };
 
-// Backward launch (fdb_bwd.hip): fixed layout only.  Position scores and their gradients are fp32, element
+// Backward launch (fdb_bwd.hip): fixed layout only.  Position scores and their gradients have q's element type, element
 // (b, l, h, delta) at b * bias_sb + l * bias_st + h * bias_sh + delta; lse / delta are fp32 [B*L, H].
 struct FdbBwdParams {
   const char* q;
@@ -58,8 +58,8 @@ struct FdbBwdParams {
   const float* lse;
   float* delta;         // sum_d dO * O per row: read, or written by the dQ role when `out` is given
   const char* out;      // the forward's output or NULL
-  const float* c2p;     // q_i . K_r[delta] or NULL
-  const float* p2c;     // k_j . Q_r[delta] or NULL
+  const char* c2p;      // q_i . K_r[delta] or NULL; element type of q, like the gradient tensors below
+  const char* p2c;      // k_j . Q_r[delta] or NULL
   char* d_c2p;          // element type of q; zero-initialised by the caller; touched entries are stored once
   char* d_p2c;
   const int32_t* seq_start;

@@ -253,7 +253,7 @@ def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=
     pos_key = K_r / pos_query = Q_r [H, 2S, D] or None  ->  (dq, dk, dv, d pos_key, d pos_query).
     Counterpart of FlashAttentionDisentangled.backward (reference flash_attention.py:1066-1086), which hands
     flash_attn_v2_bwd_dise the position-score tensors and gets their gradients back; as there, those tensors
-    are two GEMMs around the kernel (here fp32, head-major [H, B*L, 2S]) and the chain through K_r / Q_r and back into
+    are two GEMMs around the kernel (here head-major [H, B*L, 2S]) and the chain through K_r / Q_r and back into
     q / k is four more.  delta: (dout * out).sum(-1) as fp32 [B*L, H] if the caller has it (then `out` is not
     read); by default the first launch computes it."""
     B, L, H, D = q.shape
@@ -268,7 +268,7 @@ def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=
     a = _lib.FdbAttnBwdArgs()
     f32 = torch.float32
     c2p = p2c = d_c2p = d_p2c = None
-    # Position scores and their gradients are head-major, [H, B*L, 2S] fp32: what a batched GEMM over the heads
+    # Position scores and their gradients are head-major, [H, B*L, 2S] in the inputs' type: what a batched GEMM over the heads
     # writes and reads as it stands (a token-major tensor would cost a transposing copy of it each way).
     heads_first = lambda x: x.permute(2, 0, 1, 3).reshape(H, B * L, D)  # a view of [B, L, H, D] when that is contiguous
     if pos_key is not None or pos_query is not None:
@@ -276,14 +276,14 @@ def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=
         a.delta_lut, a.lut_radius, a.att_span = lut.data_ptr(), radius, span
         a.bias_stride_b, a.bias_stride_t, a.bias_stride_h = L * 2 * span, 2 * span, B * L * 2 * span
     if pos_key is not None:
-        qh, pk_t = heads_first(q), pos_key[:, :2 * span].transpose(1, 2)
-        c2p = _scores_f32(qh, pk_t)                              # [H, B*L, 2S] = q . K_r^T
-        d_c2p = torch.zeros_like(c2p, dtype=q.dtype)            # gradient tensors: the inputs' type, as in the reference
+        qh, pk_t = heads_first(q), pos_key[:, :2 * span].transpose(1, 2).to(q.dtype)
+        c2p = torch.bmm(qh, pk_t)                                # [H, B*L, 2S] = q . K_r^T, in the inputs' type like the reference's
+        d_c2p = torch.zeros_like(c2p)
         a.c2p_bias, a.d_c2p_bias = c2p.data_ptr(), d_c2p.data_ptr()
     if pos_query is not None:
-        kh, pq_t = heads_first(k), pos_query[:, :2 * span].transpose(1, 2)
-        p2c = _scores_f32(kh, pq_t)
-        d_p2c = torch.zeros_like(p2c, dtype=q.dtype)
+        kh, pq_t = heads_first(k), pos_query[:, :2 * span].transpose(1, 2).to(k.dtype)
+        p2c = torch.bmm(kh, pq_t)
+        d_p2c = torch.zeros_like(p2c)
         a.p2c_bias, a.d_p2c_bias = p2c.data_ptr(), d_p2c.data_ptr()
     if delta is None:
         out = out if out.stride(-1) == 1 else out.contiguous()

@@ -155,14 +155,15 @@ int fdb_attn_fwd_noalloc(const fdb_attn_args* a, void* stream);
  * Backward, fixed layout (optionally with seq_start / seq_len).  Replaces flash_attn_v2_bwd_dise and the three
  * kernels it launches (src/flashdeberta/ops/flash_attention.py:942-1030, :62-141, :581-941), called from
  * FlashAttentionDisentangled.backward (:1066-1086).  Same division of labour as there: the position scores come
- * in as tensors, c2p_bias[b,l,h,delta] = q . K_r[delta] and p2c_bias[b,l,h,delta] = k . Q_r[delta] (fp32; the
- * reference: [B,H,L,2S] in the input dtype), and the gradients with respect to them leave in d_c2p_bias /
- * d_p2c_bias (element type of `dtype`, like the reference's; ZEROED BY THE CALLER: an entry is stored once, by
- * plain stores in aligned groups of four, if any score maps to its group, and not touched otherwise).  The four
- * tensors share one layout: element (b, l, h, delta) at b * bias_stride_b + l * bias_stride_t + h * bias_stride_h
- * + delta (strides in elements, multiples of 4; 2S a multiple of 4; the gradient tensors 16-byte aligned;
- * l * bias_stride_t + delta must stay below 2^31).  Head-major [H, B, L, 2S] is what a batched GEMM over the
- * heads writes and reads without a transpose.  The chain through K_r / Q_r and into q / k is the caller's GEMMs.
+ * in as tensors, c2p_bias[b,l,h,delta] = q . K_r[delta] and p2c_bias[b,l,h,delta] = k . Q_r[delta], and the
+ * gradients with respect to them leave in d_c2p_bias / d_p2c_bias; all four have the element type of `dtype`,
+ * like the reference's ([B,H,L,2S] in the input dtype).  The gradient tensors are ZEROED BY THE CALLER: an entry
+ * is stored once, by plain stores in aligned groups of four, if any score maps to its group, and not touched
+ * otherwise.  The four tensors share one layout: element (b, l, h, delta) at b * bias_stride_b + l * bias_stride_t
+ * + h * bias_stride_h + delta (strides in elements, multiples of 4; 2S a multiple of 4; the gradient tensors
+ * 16-byte aligned; l * bias_stride_t + delta must stay below 2^31).  Head-major [H, B, L, 2S] is what a batched
+ * GEMM over the heads writes and reads without a transpose.  The chain through K_r / Q_r and into q / k is the
+ * caller's GEMMs.
  * dq, dk, dv hold only the content part,
  *   dq_i = sum_j dS_ij k_j,  dk_j = sum_i dS_ij q_i,  dv_j = sum_i P_ij dO_i,  dS = P (dO V^T - delta) sm_scale,
  * with P recomputed from lse (the forward's log-sum-exp, [B*L, H]) and delta[row] = sum_d dO * O ([B*L, H] fp32;
@@ -182,8 +183,8 @@ typedef struct fdb_attn_bwd_args {
   const float* lse;
   float* delta;            /* [B*L, H] fp32: written when `out` is given, read otherwise */
   const void* out;         /* the forward's output or NULL */
-  const float* c2p_bias;   /* or NULL: no content->position term */
-  const float* p2c_bias;   /* or NULL: no position->content term */
+  const void* c2p_bias;    /* or NULL: no content->position term; elements of `dtype` */
+  const void* p2c_bias;    /* or NULL: no position->content term; elements of `dtype` */
   void* d_c2p_bias;        /* required with c2p_bias; elements of `dtype` */
   void* d_p2c_bias;        /* required with p2c_bias; elements of `dtype` */
   const int32_t* seq_start;
