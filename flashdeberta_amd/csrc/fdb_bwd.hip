@@ -279,6 +279,18 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
     const bool far = far_n;
     const int d_far = dfar_n;
     float bias[16];
+    // near step: table rows of this lane's 16 elements as offsets (0..31) from the first entry of its row's window,
+    // four to a register
+    int d_lo = 0;
+    uint32_t off4[4] = {0u, 0u, 0u, 0u};
+    if (kBias && !far) {
+      d_lo = delta_of(kDQ ? xr - (y0 + kBwdStep - 1) : y0 - xr);
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int yr = y0 + 8 * (v >> 2) + 4 * g + (v & 3);
+        off4[v >> 2] |= (uint32_t)(delta_of(kDQ ? xr - yr : yr - xr) - d_lo) << (8 * (v & 3));
+      }
+    }
     if (kBias && far) {
       if (kLoopT) {
         if (g == 0) vec_w[li] = (float)raw_loop[0];
@@ -298,27 +310,26 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
 #pragma unroll
       for (int v = 0; v < 16; ++v) bias[v] = (float)raw_lane[v] + (float)raw_loop[v];
     }
-    if (has_next) request(y0 + kBwdStep);
     float ds[16], ds_run[16], pr[16], g_sum = 0.f;
     bool ok[16];
-    f32x4 lse4[4], del4[4];  // dK/dV role: statistics of this lane's 16 loop rows, four neighbours per read
-    if (!kDQ) {
 #pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        lse4[q4] = *(const f32x4*)(lse_s + 8 * q4 + 4 * g);
-        del4[q4] = *(const f32x4*)(del_s + 8 * q4 + 4 * g);
+    for (int q4 = 0; q4 < 4; ++q4) {
+      f32x4 lse4 = {lse_x, lse_x, lse_x, lse_x}, del4 = {del_x, del_x, del_x, del_x};
+      if (!kDQ) {  // statistics of this lane's loop rows, four neighbours per read
+        lse4 = *(const f32x4*)(lse_s + 8 * q4 + 4 * g);
+        del4 = *(const f32x4*)(del_s + 8 * q4 + 4 * g);
       }
-    }
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int yl = 8 * (v >> 2) + 4 * g + (v & 3), yr = y0 + yl;
-      const int i = kDQ ? xr : yr, j = kDQ ? yr : xr;
-      ok[v] = x_ok && yr < Lb && (!p.causal || j <= i);
-      const float lse_i = kDQ ? lse_x : lse4[v >> 2][v & 3], del_i = kDQ ? del_x : del4[v >> 2][v & 3];
-      const float pv = ok[v] ? __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[v] + bias[v], c_log2, -lse_i)) : 0.f;
-      pr[v] = pv;
-      ds[v] = pv * (dpacc[v] - del_i) * c_sm;
-      g_sum += ds[v];
+      for (int e = 0; e < 4; ++e) {
+        const int v = 4 * q4 + e;
+        const int yr = y0 + 8 * q4 + 4 * g + e;
+        const int i = kDQ ? xr : yr, j = kDQ ? yr : xr;
+        ok[v] = x_ok && yr < Lb && (!p.causal || j <= i);
+        const float pv = ok[v] ? __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[v] + bias[v], c_log2, -lse4[e])) : 0.f;
+        pr[v] = pv;
+        ds[v] = pv * (dpacc[v] - del4[e]) * c_sm;
+        g_sum += ds[v];
+      }
     }
     if (kGrad) {
       // LDS float atomics are served a lane at a time on this hardware (160 clocks per instruction), so the adds are
@@ -332,8 +343,7 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
         int dl[16];
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          const int yr = y0 + 8 * (v >> 2) + 4 * g + (v & 3);
-          dl[v] = delta_of(kDQ ? xr - yr : yr - xr);
+          dl[v] = d_lo + (int)((off4[v >> 2] >> (8 * (v & 3))) & 255u);
           if (v > 0) ds_run[v] = ds[v] + (dl[v] == dl[v - 1] ? ds_run[v - 1] : 0.f);
           else ds_run[0] = ds[0];
         }
@@ -384,6 +394,7 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
         n_g -= n_now;
       }
     }
+    if (has_next) request(y0 + kBwdStep);  // here rather than earlier: the requested values occupy 32 registers until used
     // ---- outputs: contraction over the loop rows, which are the accumulator registers ------------------------------
 #pragma unroll
     for (int c = 0; c < 2; ++c) {
