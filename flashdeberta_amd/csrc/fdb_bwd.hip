@@ -48,34 +48,16 @@ template <class QT, int D>
 struct BCfg {
   static constexpr int KS = D / 16, DBLKS = D / 32;
   static constexpr int RS = D * QT::SZ + 16;                 // LDS row stride of a staged tile
-  static constexpr int TILE = kBwdStep * RS;
-  static constexpr int CHUNKS = (kBwdStep * D * QT::SZ / 16 + kBwdThreads - 1) / kBwdThreads;  // 16-byte chunks per thread
-  // two tile buffers, loop-row statistics, ring windows, far-step scores, groups to store; the table follows
-  static constexpr int fixed_lds_bytes() { return 4 * TILE + 4 * kBwdStep * 4 + FDB_BM * kRingStrideMax * 4 + FDB_BM * 4 + FDB_BM * 8; }
+  static constexpr int CPR = D * QT::SZ / 16;                // 16-byte chunks of a row
+  // Loop-side rows staged per barrier: two steps' worth where LDS allows (the barrier and the staging are then paid
+  // once per 64 rows), one for the widest rows.
+  static constexpr int TROWS = RS > 272 ? kBwdStep : 2 * kBwdStep;
+  static constexpr int TILE = TROWS * RS;                    // a multiple of 1024: RS is a multiple of 16
+  static constexpr int REGION = 2 * TILE;                    // [Y1 tile | Y2 tile] of one buffer
+  // two buffers, loop-row statistics, ring windows, far-step scores, groups to store; the table follows
+  static constexpr int fixed_lds_bytes() { return 2 * REGION + 4 * TROWS * 4 + FDB_BM * kRingStrideMax * 4 + FDB_BM * 4 + FDB_BM * 8; }
   static int lds_bytes(int radius) { return fixed_lds_bytes() + (((2 * radius + 1) * 2 + 15) & ~15); }
 };
-
-// [32 x D] tile: global -> registers -> LDS.  Rows past the end re-read the last valid row; their scores are masked.
-template <class QT, int D, int NCH>
-__device__ __forceinline__ void btile_load(u32x4 (&reg)[NCH], const char* gbase, int64_t row_stride_bytes,
-                                           int r0, int n_rows, int tid) {
-  constexpr int CPR = D * QT::SZ / 16, TOTAL = kBwdStep * CPR;
-#pragma unroll
-  for (int n = 0; n < NCH; ++n) {
-    const int c = tid + n * kBwdThreads;
-    const int row = min(r0 + min(c / CPR, kBwdStep - 1), n_rows - 1), cc = c % CPR;
-    if (TOTAL % kBwdThreads == 0 || c < TOTAL) reg[n] = *(const u32x4*)(gbase + (int64_t)row * row_stride_bytes + cc * 16);
-  }
-}
-template <class QT, int D, int NCH>
-__device__ __forceinline__ void btile_store(char* lds, const u32x4 (&reg)[NCH], int tid) {
-  constexpr int CPR = D * QT::SZ / 16, TOTAL = kBwdStep * CPR;
-#pragma unroll
-  for (int n = 0; n < NCH; ++n) {
-    const int c = tid + n * kBwdThreads;
-    if (TOTAL % kBwdThreads == 0 || c < TOTAL) *(u32x4*)(lds + (c / CPR) * BCfg<QT, D>::RS + (c % CPR) * 16) = reg[n];
-  }
-}
 
 template <class QT, int D, int ROLE, bool C2P, bool P2C>
 __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_bwd_kernel(const FdbBwdParams p) {
@@ -86,8 +68,8 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
   constexpr int kRingStride = ring_stride(kDQ);
   extern __shared__ __attribute__((aligned(16))) char smem[];
   char* Ys = smem;                                    // two buffers of [K | V] (dQ role) / [Q | dO] (dK/dV role)
-  float* stat_s = (float*)(Ys + 4 * C::TILE);         // dK/dV role: per buffer, log-sum-exp (base 2) and Delta of the 32 loop rows
-  float* ring_s = stat_s + 4 * kBwdStep;              // [128 lane-side rows][kRingStride] score-gradient windows
+  float* stat_s = (float*)(Ys + 2 * C::REGION);       // dK/dV role: per buffer, log-sum-exp (base 2) and Delta of the staged loop rows
+  float* ring_s = stat_s + 4 * C::TROWS;              // [128 lane-side rows][kRingStride] score-gradient windows
   float* vec_s = ring_s + FDB_BM * kRingStrideMax;      // [4 waves][32] loop-side position scores of a far step
   int2* inf_s = (int2*)(vec_s + FDB_BM);              // [4 waves][32] (first group, groups) to store per row
   LDS_AS int16_t* lut_s = (LDS_AS int16_t*)(inf_s + FDB_BM);  // the whole table (the launcher sizes the allocation for it)
@@ -187,26 +169,39 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
     const int x = max(-p.R, min(p.R, r)) + p.R;
     return (int)lut_s[x];
   };
-  // The two tiles of a step sit in one of two LDS buffers: the tiles of step t + 1 are on their way to registers
-  // while step t computes and go to the other buffer at its end, so a step has one barrier.
-  u32x4 y1reg[C::CHUNKS], y2reg[C::CHUNKS];
+  // The loop side's tiles go from global memory straight into one of two LDS buffers (no registers on the way):
+  // those of the rows after the current ones are on their way while the current ones are used, and a barrier per
+  // buffer makes them visible.  A wave instruction fills 1 KB of LDS, lane l the 16 bytes at 16 * l: with padded rows
+  // some lanes fall on the padding and fetch a chunk nobody reads.  Rows past the end re-read the last valid row;
+  // their scores are masked.
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(LDS_AS char*)smem;
+  auto tiles_dma = [&](int r0, int buf) __attribute__((always_inline)) {
+    constexpr int SPANS = C::REGION / 1024;
+#pragma unroll
+    for (int n = 0; n < (SPANS + 3) / 4; ++n) {
+      const int span = wave + 4 * n;
+      if (span < SPANS) {
+        const int o = span * 1024 + lane * 16;
+        const int t = o >= C::TILE ? 1 : 0, o2 = o - t * C::TILE;
+        const int row = o2 / C::RS, c = (o2 - row * C::RS) >> 4;
+        const char* src = (t ? y2b : y1b) + (int64_t)min(r0 + row, Lb - 1) * (t ? y2_rsb : y1_rsb) + (c < C::CPR ? c : 0) * 16;
+        dma16(src, lds0 + buf * C::REGION + span * 1024);
+      }
+    }
+  };
   float st_reg[2] = {0.f, 0.f};
-  auto tiles_load = [&](int r0) __attribute__((always_inline)) {
-    btile_load<QT, D>(y1reg, y1b, y1_rsb, r0, Lb, tid);
-    btile_load<QT, D>(y2reg, y2b, y2_rsb, r0, Lb, tid);
-    if (!kDQ && tid < kBwdStep) {
+  auto stats_load = [&](int r0) __attribute__((always_inline)) {
+    if (!kDQ && tid < C::TROWS) {
       const int row = min(r0 + tid, Lb - 1);
       const int64_t t = ((int64_t)b * p.L + tok0 + row) * p.H + h;
       st_reg[0] = p.lse[t] * 1.4426950408889634f;
       st_reg[1] = p.delta[t];
     }
   };
-  auto tiles_store = [&](int buf) __attribute__((always_inline)) {
-    btile_store<QT, D>(Ys + buf * 2 * C::TILE, y1reg, tid);
-    btile_store<QT, D>(Ys + buf * 2 * C::TILE + C::TILE, y2reg, tid);
-    if (!kDQ && tid < kBwdStep) {
-      stat_s[buf * 2 * kBwdStep + tid] = st_reg[0];
-      stat_s[buf * 2 * kBwdStep + kBwdStep + tid] = st_reg[1];
+  auto stats_store = [&](int buf) __attribute__((always_inline)) {
+    if (!kDQ && tid < C::TROWS) {
+      stat_s[buf * 2 * C::TROWS + tid] = st_reg[0];
+      stat_s[buf * 2 * C::TROWS + C::TROWS + tid] = st_reg[1];
     }
   };
   // Position scores of a step are requested one step ahead (their addresses depend on indices only), so that their
@@ -247,22 +242,32 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
     }
   };
   if (y_lo < y_hi) {
-    tiles_load(y_lo);
+    tiles_dma(y_lo, 0);
+    stats_load(y_lo);
     __syncthreads();  // the table is in LDS
     if (kGrad) g_next = delta_of(kDQ ? xr - y_lo : y_lo - xr) >> 2;
     request(y_lo);
-    tiles_store(0);
+    stats_store(0);
   }
 
   int buf = 0;
-  for (int y0 = y_lo; y0 < y_hi; y0 += kBwdStep, buf ^= 1) {
-    __syncthreads();  // the tiles of this step are in LDS; every wave is done with the other buffer (and the table is there)
+  for (int yt = y_lo; yt < y_hi; yt += C::TROWS, buf ^= 1) {
+  wait_vmcnt<0>();   // this wave's share of the buffer has landed (and the position scores asked for during the last step)
+  __syncthreads();   // ... and everybody's; every wave is done with the other buffer (and the table is in LDS)
+  const bool next_tiles = yt + C::TROWS < y_hi;
+  if (next_tiles) {
+    tiles_dma(yt + C::TROWS, buf ^ 1);
+    stats_load(yt + C::TROWS);
+  }
+#pragma unroll 1
+  for (int sub = 0; sub < C::TROWS / kBwdStep; ++sub) {
+    const int y0 = yt + sub * kBwdStep;
+    if (y0 >= y_hi) break;
     const bool has_next = y0 + kBwdStep < y_hi;
-    if (has_next) tiles_load(y0 + kBwdStep);
-    const char* Y1s = Ys + buf * 2 * C::TILE;
+    const char* Y1s = Ys + buf * C::REGION + sub * kBwdStep * C::RS;
     const char* Y2s = Y1s + C::TILE;
-    const float* lse_s = stat_s + buf * 2 * kBwdStep;
-    const float* del_s = lse_s + kBwdStep;
+    const float* lse_s = stat_s + buf * 2 * C::TROWS + sub * kBwdStep;
+    const float* del_s = lse_s + C::TROWS;
     // ---- S' and dP' ----------------------------------------------------------------------------------------
     f32x16 sacc, dpacc;
 #pragma unroll
@@ -411,7 +416,8 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
         if (!kDQ) acc2[d] = QT::mma(VtLoad<QT>::get(Y2s, C::RS, c, d, lane), pf, acc2[d]);  // dV^T += dO^T P'
       }
     }
-    if (has_next) tiles_store(buf ^ 1);
+  }
+  if (next_tiles) stats_store(buf ^ 1);
   }
 
   if (!x_ok) return;
