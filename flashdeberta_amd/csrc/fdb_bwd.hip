@@ -3,11 +3,13 @@
 // kernels (src/flashdeberta/ops/flash_attention.py:62-141 _bwd_preprocess, :581-760 _bwd_kv_dise_kernel,
 // :762-941 _bwd_q_dise_kernel, launcher :942-1030): like them it takes the position scores
 // c2p[b,i,h,delta] = q_i . K_r[delta] and p2c[b,j,h,delta] = k_j . Q_r[delta] as tensors, gathers them through
-// the bucketed relative position, and scatter-adds the score gradients into tensors of the same shape
-// (the reference: tl.atomic_add, :769-786); the chain through K_r / Q_r is left to the caller's GEMMs.
+// the bucketed relative position, and returns the score gradients as tensors of the same shape (the reference
+// scatter-adds them with tl.atomic_add, :769-786; here every entry is stored once, see below); the chain through
+// K_r / Q_r is left to the caller's GEMMs.
 //
 // One kernel in two roles.  A workgroup owns 128 rows of the "lane side" (4 waves x 32 rows, one row per
-// lane and its partner lane ^ 32) and walks the "loop side" 32 rows at a time through LDS:
+// lane and its partner lane ^ 32) and walks the "loop side" 32 rows at a time; the loop side's tiles come
+// from global memory straight into one of two LDS buffers, 64 rows (two steps) per buffer and barrier:
 //   role dQ    : lane side = queries (q, dO in registers), loop side = keys (K, V tiles)  ->  dQ, d c2p
 //   role dK/dV : lane side = keys (k, v in registers), loop side = queries (Q, dO tiles) ->  dK, dV, d p2c
 // Per step, with X the lane side and Y the loop side (MFMA 32x32, M = loop row, N = lane row):
