@@ -1059,3 +1059,57 @@ def test_backward_refuses_an_odd_span():
     out, lse = ops.disentangled_attention_fwd(q, k, v, pk, pq, return_lse=True, position_buckets=0, max_relative_positions=15)
     with pytest.raises(ValueError):
         ops.disentangled_attention_bwd(q, k, v, out, lse, torch.ones_like(out), pk, pq, position_buckets=0, max_relative_positions=15)
+
+
+def _random_case(seed):
+    r = np.random.RandomState(seed)
+    B = int(r.choice([1, 2, 3]))
+    L = int(r.choice([1, 31, 32, 33, 63, 64, 65, 96, 127, 128, 129, 160, 255, 257, 300, 420]))
+    H = int(r.choice([1, 2, 3]))
+    D = int(r.choice([32, 64, 64, 128]))
+    pb, mr = [(8, 16), (32, 64), (16, 96), (0, 40), (0, 150), (256, 512)][r.randint(6)]
+    terms = [(True, True), (True, True), (True, False), (False, True), (False, False)][r.randint(5)]
+    causal = bool(r.randint(4) == 0)
+    lens = None
+    if B > 1 and r.randint(2):
+        lens = [int(r.randint(1, L + 1)) for _ in range(B)]
+    dtype = [torch.float32, torch.bfloat16, torch.float16][r.randint(3)]
+    return B, L, H, D, pb, mr, terms[0], terms[1], causal, lens, dtype
+
+
+@pytest.mark.parametrize("seed", list(range(24)))
+def test_random_shapes_forward_and_backward(seed):
+    """Seeded random draws over batch, length (around the 32 / 64 / 128 tile edges), heads, head_dim, bucket
+    configuration, terms, causal, padded rows and element type: output and all five gradients against the oracle."""
+    B, L, H, D, pb, mr, c2p, p2c, causal, lens, dtype = _random_case(seed)
+    what = "B%d L%d H%d D%d b%d m%d c2p%d p2c%d causal%d lens%s %s" % (B, L, H, D, pb, mr, c2p, p2c, causal, lens, dtype)
+    print(what, flush=True)
+    q, k, v, pk, pq = _inputs(B, L, H, D, pb, mr, dtype, 5000 + seed, 1.0, c2p, p2c)
+    dout = torch.randn(B, L, H, D, generator=torch.Generator().manual_seed(6000 + seed)).to(dtype)
+    kw = dict(position_buckets=pb, max_relative_positions=mr, causal=causal)
+    mask = None
+    if lens is not None:
+        mask = np.arange(L)[None, :] < np.array(lens)[:, None]
+        dout = dout * torch.from_numpy(mask)[:, :, None, None].to(dtype)
+        kw["seq_len"] = torch.tensor(lens, dtype=torch.int32, device="cuda")
+        kw["out"] = torch.zeros(B, L, H, D, dtype=dtype, device="cuda")
+    t = lambda x: _np(x).transpose(0, 2, 1, 3)
+    ref_out = O.disentangled_attention(t(q), t(k), t(v), _np(pk), _np(pq), pb, mr, mask=mask, causal=causal).transpose(0, 2, 1, 3)
+    ref = O.disentangled_attention_backward(t(q), t(k), t(v), t(dout), _np(pk), _np(pq), pb, mr, mask=mask, causal=causal)
+    leaves = [None if x is None else x.cuda().requires_grad_(True) for x in (q, k, v, pk, pq)]
+    out = ops.disentangled_attention(*leaves, **kw)
+    tol = {torch.float32: 2e-4, torch.bfloat16: 3e-2, torch.float16: 6e-3}[dtype]
+    got_out = out.detach().float().cpu().numpy()
+    if mask is not None:
+        got_out, ref_out = got_out * mask[:, :, None, None], ref_out * mask[:, :, None, None]
+    assert np.abs(got_out - ref_out).max() <= tol * max(np.abs(ref_out).max(), 1e-3), what
+    out.backward(dout.cuda())
+    for n, leaf, r in zip(("dq", "dk", "dv", "dK_r", "dQ_r"), leaves, ref):
+        if leaf is None:
+            continue
+        got = leaf.grad.float().cpu().numpy()
+        r = r.transpose(0, 2, 1, 3) if r.ndim == 4 else r
+        if mask is not None and r.ndim == 4:
+            r = r * mask[:, :, None, None]
+        err = np.abs(got - r).max()
+        assert not np.isnan(got).any() and err <= tol * max(np.abs(r).max(), 1e-3), "%s %s: err %.3e, ref max %.3e" % (what, n, err, np.abs(r).max())
