@@ -224,7 +224,9 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
   auto loop_off = [&](int yr) __attribute__((always_inline)) -> uint32_t {
     return (uint32_t)min(yr, Lb - 1) * row_elems;
   };
-  auto request = [&](int y0) __attribute__((always_inline)) {
+  // Classifies the wave's block of the step at y0 and, if it is far, asks for its two values right away (they cost two
+  // registers); the 32 values of a near block are asked for later in the step by request_near (they would sit in 32).
+  auto request_far = [&](int y0) __attribute__((always_inline)) {
     if (!kBias) return;
     const int r_min = kDQ ? xw0 - (y0 + kBwdStep - 1) : y0 - (xw0 + 31);      // over the wave's 32 x 32 block
     const int r_max = kDQ ? xw0 + 31 - y0 : y0 + kBwdStep - 1 - xw0;
@@ -233,14 +235,16 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
     if (far_n) {
       if (kLaneT) raw_lane[0] = lane_t[x_off + (uint32_t)dfar_n];
       if (kLoopT) raw_loop[0] = loop_t[loop_off(y0 + li) + (uint32_t)dfar_n];
-    } else {
+    }
+  };
+  auto request_near = [&](int y0) __attribute__((always_inline)) {
+    if (!kBias || far_n) return;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int yr = y0 + 8 * (v >> 2) + 4 * g + (v & 3);
-        const int dl = delta_of(kDQ ? xr - yr : yr - xr);
-        if (kLaneT) raw_lane[v] = lane_t[x_off + (uint32_t)dl];
-        if (kLoopT) raw_loop[v] = loop_t[loop_off(yr) + (uint32_t)dl];
-      }
+    for (int v = 0; v < 16; ++v) {
+      const int yr = y0 + 8 * (v >> 2) + 4 * g + (v & 3);
+      const int dl = delta_of(kDQ ? xr - yr : yr - xr);
+      if (kLaneT) raw_lane[v] = lane_t[x_off + (uint32_t)dl];
+      if (kLoopT) raw_loop[v] = loop_t[loop_off(yr) + (uint32_t)dl];
     }
   };
   if (y_lo < y_hi) {
@@ -248,13 +252,19 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
     stats_load(y_lo);
     __syncthreads();  // the table is in LDS
     if (kGrad) g_next = delta_of(kDQ ? xr - y_lo : y_lo - xr) >> 2;
-    request(y_lo);
+    request_far(y_lo);
+    request_near(y_lo);
     stats_store(0);
   }
 
   int buf = 0;
   for (int yt = y_lo; yt < y_hi; yt += C::TROWS, buf ^= 1) {
-  wait_vmcnt<0>();   // this wave's share of the buffer has landed (and the position scores asked for during the last step)
+  // This wave's share of the buffer has landed: loads complete in issue order, and the only younger ones are the
+  // position scores the last step asked for (two per lane for a far block, up to 32 for a near one), which the step
+  // waits for where it uses them.
+  constexpr int kAsked = (kLaneT ? 1 : 0) + (kLoopT ? 1 : 0);
+  if (far_n) wait_vmcnt<kAsked>();
+  else wait_vmcnt<16 * kAsked>();
   __syncthreads();   // ... and everybody's; every wave is done with the other buffer (and the table is in LDS)
   const bool next_tiles = yt + C::TROWS < y_hi;
   if (next_tiles) {
@@ -317,6 +327,7 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
 #pragma unroll
       for (int v = 0; v < 16; ++v) bias[v] = (float)raw_lane[v] + (float)raw_loop[v];
     }
+    if (has_next) request_far(y0 + kBwdStep);
     float ds[16], ds_run[16], pr[16], g_sum = 0.f;
     bool ok[16];
 #pragma unroll
@@ -401,7 +412,7 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
         n_g -= n_now;
       }
     }
-    if (has_next) request(y0 + kBwdStep);  // here rather than earlier: the requested values occupy 32 registers until used
+    if (has_next) request_near(y0 + kBwdStep);  // here rather than earlier: the requested values occupy 32 registers until used
     // ---- outputs: contraction over the loop rows, which are the accumulator registers ------------------------------
 #pragma unroll
     for (int c = 0; c < 2; ++c) {

@@ -311,12 +311,12 @@ __device__ __forceinline__ void dma16s(const void* base, uint32_t lane_off, uint
 // Wait until at most N vector-memory loads of this wave are outstanding (loads complete in issue
 // order).  Issued through the builtin rather than asm, so that the compiler's own count of its
 // outstanding loads takes the wait into account and it does not wait a second time for a value
-// these waits have already covered.  Encoding (gfx9): vmcnt in bits 3:0 (and 15:14), expcnt 6:4 and
+// these waits have already covered.  Encoding (gfx9): vmcnt in bits 3:0 and 15:14, expcnt 6:4 and
 // lgkmcnt 11:8 left at their maxima (no wait).
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
-  static_assert(N >= 0 && N < 16, "counts used by the kernels");
-  __builtin_amdgcn_s_waitcnt(0x0F70 | N);
+  static_assert(N >= 0 && N < 64, "vmcnt has six bits");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
   asm volatile("" ::: "memory");
 }
 
