@@ -153,6 +153,7 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
   }
   constexpr int kDir = kDQ ? -1 : 1;        // the way the window moves as the loop row grows
   int g_next = 0;                           // next group of four entries of this lane's row to store
+  float g_far = 0.f;                        // row sum of a run of far blocks
 
   f32x16 acc1[DBLKS], acc2[DBLKS];  // dQ^T (dQ role) / dK^T and dV^T (dK/dV role)
 #pragma unroll
@@ -237,12 +238,19 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
       if (kLoopT) raw_loop[0] = loop_t[loop_off(y0 + li) + (uint32_t)dfar_n];
     }
   };
+  // The table rows of a near block's 16 elements stay with the lane until the block's score gradients are added: as
+  // offsets (0..31) from the first entry of the lane row's window, four to a register.
+  int d_lo = 0;
+  uint32_t off4[4] = {0u, 0u, 0u, 0u};
   auto request_near = [&](int y0) __attribute__((always_inline)) {
     if (!kBias || far_n) return;
+    d_lo = delta_of(kDQ ? xr - (y0 + kBwdStep - 1) : y0 - xr);
+    off4[0] = off4[1] = off4[2] = off4[3] = 0u;
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
       const int yr = y0 + 8 * (v >> 2) + 4 * g + (v & 3);
       const int dl = delta_of(kDQ ? xr - yr : yr - xr);
+      off4[v >> 2] |= (uint32_t)(dl - d_lo) << (8 * (v & 3));
       if (kLaneT) raw_lane[v] = lane_t[x_off + (uint32_t)dl];
       if (kLoopT) raw_loop[v] = loop_t[loop_off(yr) + (uint32_t)dl];
     }
@@ -296,18 +304,6 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
     const bool far = far_n;
     const int d_far = dfar_n;
     float bias[16];
-    // near step: table rows of this lane's 16 elements as offsets (0..31) from the first entry of its row's window,
-    // four to a register
-    int d_lo = 0;
-    uint32_t off4[4] = {0u, 0u, 0u, 0u};
-    if (kBias && !far) {
-      d_lo = delta_of(kDQ ? xr - (y0 + kBwdStep - 1) : y0 - xr);
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int yr = y0 + 8 * (v >> 2) + 4 * g + (v & 3);
-        off4[v >> 2] |= (uint32_t)(delta_of(kDQ ? xr - yr : yr - xr) - d_lo) << (8 * (v & 3));
-      }
-    }
     if (kBias && far) {
       if (kLoopT) {
         if (g == 0) vec_w[li] = (float)raw_loop[0];
@@ -354,9 +350,16 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
       // plain reads and writes: the lanes of a half-wave own different rows, and the two halves (which share rows)
       // take turns.  Within a lane the table rows of the 16 elements are sorted, so elements of one entry are
       // neighbours: each write carries the sum of its run so far and the last write of a run, the complete one, wins.
+      bool settled = false;  // nothing can have left the window
       if (far) {
-        g_sum = wave_half_sum(g_sum);
-        if (g == 0) ring_x[d_far & (kRing - 1)] += g_sum;
+        // a run of far blocks with one table row: the row sums add up in a register and enter the ring when the run ends
+        g_far += g_sum;
+        settled = has_next && far_n && dfar_n == d_far;  // the next block continues the run
+        if (!settled) {
+          const float run = wave_half_sum(g_far);
+          if (g == 0) ring_x[d_far & (kRing - 1)] += run;
+          g_far = 0.f;
+        }
       } else {
         int dl[16];
 #pragma unroll
@@ -380,8 +383,11 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
       // Groups of four entries [4m, 4m + 3] the window has left behind: every later element of the row maps to a
       // table row at or beyond `d_edge` (that of the next step's first loop row; after the last step, the last
       // row's own entry, and its group goes too).  Up to eight groups per row and pass.
-      const int d_edge = delta_of(has_next ? (kDQ ? xr - (y0 + kBwdStep) : y0 + kBwdStep - xr) : (kDQ ? xr - (y_hi - 1) : y_hi - 1 - xr));
-      int n_g = !x_ok ? 0 : kDir * ((d_edge >> 2) - g_next) + (has_next ? 0 : 1);
+      int n_g = 0;
+      if (!settled) {
+        const int d_edge = delta_of(has_next ? (kDQ ? xr - (y0 + kBwdStep) : y0 + kBwdStep - xr) : (kDQ ? xr - (y_hi - 1) : y_hi - 1 - xr));
+        n_g = !x_ok ? 0 : kDir * ((d_edge >> 2) - g_next) + (has_next ? 0 : 1);
+      }
       while (__builtin_amdgcn_ballot_w64(n_g > 0) != 0) {
         const int n_now = max(0, min(n_g, 8));
         if (g == 0) inf_w[li] = int2{g_next, n_now};
