@@ -288,22 +288,11 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
     const char* Y2s = Y1s + C::TILE;
     const float* lse_s = stat_s + buf * 2 * C::TROWS + sub * kBwdStep;
     const float* del_s = lse_s + C::TROWS;
-    // ---- S' and dP' ----------------------------------------------------------------------------------------
-    f32x16 sacc, dpacc;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) sacc[v] = dpacc[v] = 0.f;
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      const frag y1f = QT::load(Y1s + li * C::RS + (16 * s + 8 * g) * QT::SZ);
-      const frag y2f = QT::load(Y2s + li * C::RS + (16 * s + 8 * g) * QT::SZ);
-      sacc = QT::mma(y1f, x1f[s], sacc);
-      dpacc = QT::mma(y2f, x2f[s], dpacc);
-    }
-    // ---- position scores (requested during the step before), probabilities, score gradients ----------------------
+    // ---- position scores (requested during the step before) ---------------------------------------------------
     // element v of lane (g, li): loop row yr = y0 + 8*(v/4) + 4g + v%4, lane row xr; i - j = +-(xr - yr)
     const bool far = far_n;
     const int d_far = dfar_n;
-    float bias[16];
+    f32x16 sacc, dpacc;   // S' starts from the position scores, dP' from -Delta: the products add on top
     if (kBias && far) {
       if (kLoopT) {
         if (g == 0) vec_w[li] = (float)raw_loop[0];
@@ -312,36 +301,53 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
         for (int q4 = 0; q4 < 4; ++q4) {
           const f32x4 t4 = *(const f32x4*)(vec_w + 8 * q4 + 4 * g);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) bias[4 * q4 + e] = t4[e] + (float)raw_lane[0];
+          for (int e = 0; e < 4; ++e) sacc[4 * q4 + e] = t4[e] + (float)raw_lane[0];
         }
         wave_lds_fence();
       } else {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) bias[v] = (float)raw_lane[0];
+        for (int v = 0; v < 16; ++v) sacc[v] = (float)raw_lane[0];
       }
     } else {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) bias[v] = (float)raw_lane[v] + (float)raw_loop[v];
+      for (int v = 0; v < 16; ++v) sacc[v] = (float)raw_lane[v] + (float)raw_loop[v];
     }
     if (has_next) request_far(y0 + kBwdStep);
-    float ds[16], ds_run[16], pr[16], g_sum = 0.f;
-    bool ok[16];
 #pragma unroll
     for (int q4 = 0; q4 < 4; ++q4) {
-      f32x4 lse4 = {lse_x, lse_x, lse_x, lse_x}, del4 = {del_x, del_x, del_x, del_x};
-      if (!kDQ) {  // statistics of this lane's loop rows, four neighbours per read
-        lse4 = *(const f32x4*)(lse_s + 8 * q4 + 4 * g);
-        del4 = *(const f32x4*)(del_s + 8 * q4 + 4 * g);
-      }
+      f32x4 del4 = {del_x, del_x, del_x, del_x};
+      if (!kDQ) del4 = *(const f32x4*)(del_s + 8 * q4 + 4 * g);  // statistics of this lane's loop rows, four neighbours per read
+#pragma unroll
+      for (int e = 0; e < 4; ++e) dpacc[4 * q4 + e] = -del4[e];
+    }
+    // ---- S' and dP' ----------------------------------------------------------------------------------------
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const frag y1f = QT::load(Y1s + li * C::RS + (16 * s + 8 * g) * QT::SZ);
+      const frag y2f = QT::load(Y2s + li * C::RS + (16 * s + 8 * g) * QT::SZ);
+      sacc = QT::mma(y1f, x1f[s], sacc);
+      dpacc = QT::mma(y2f, x2f[s], dpacc);
+    }
+    // ---- probabilities and score gradients (without the factor sm_scale, which the outputs take at the end) -------
+    float ds[16], ds_run[16], pr[16], g_sum = 0.f;
+    // a block that touches the end of a sequence or the causal diagonal masks its elements one by one
+    const bool edge = xw0 + 31 >= Lb || y0 + kBwdStep > Lb ||
+                      (p.causal && (kDQ ? y0 + kBwdStep - 1 > xw0 : xw0 + 31 > y0));
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      f32x4 lse4 = {lse_x, lse_x, lse_x, lse_x};
+      if (!kDQ) lse4 = *(const f32x4*)(lse_s + 8 * q4 + 4 * g);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const int v = 4 * q4 + e;
-        const int yr = y0 + 8 * q4 + 4 * g + e;
-        const int i = kDQ ? xr : yr, j = kDQ ? yr : xr;
-        ok[v] = x_ok && yr < Lb && (!p.causal || j <= i);
-        const float pv = ok[v] ? __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[v] + bias[v], c_log2, -lse4[e])) : 0.f;
+        float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[v], c_log2, -lse4[e]));
+        if (edge) {
+          const int yr = y0 + 8 * q4 + 4 * g + e;
+          const int i = kDQ ? xr : yr, j = kDQ ? yr : xr;
+          if (!(x_ok && yr < Lb && (!p.causal || j <= i))) pv = 0.f;
+        }
         pr[v] = pv;
-        ds[v] = pv * (dpacc[v] - del4[e]) * c_sm;
+        ds[v] = pv * dpacc[v];
         g_sum += ds[v];
       }
     }
@@ -410,7 +416,8 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
           if (act[it]) {
             float* e = ring_w + rho * kRingStride + ((4 * mm[it]) & (kRing - 1));
             e[0] = e[1] = e[2] = e[3] = 0.f;
-            QT::store4(gw + ((uint32_t)(xw0 + rho) * row_elems + (uint32_t)(4 * mm[it])) * QT::SZ, val[it][0], val[it][1], val[it][2], val[it][3]);
+            QT::store4(gw + ((uint32_t)(xw0 + rho) * row_elems + (uint32_t)(4 * mm[it])) * QT::SZ,
+                       val[it][0] * c_sm, val[it][1] * c_sm, val[it][2] * c_sm, val[it][3] * c_sm);
           }
         }
         wave_lds_fence();
@@ -448,6 +455,10 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
       for (int q4 = 0; q4 < 4; ++q4)
         QT::store4(row + (32 * d + 8 * q4 + 4 * g) * QT::SZ, acc[d][4 * q4], acc[d][4 * q4 + 1], acc[d][4 * q4 + 2], acc[d][4 * q4 + 3]);
   };
+#pragma unroll
+  for (int d = 0; d < DBLKS; ++d)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc1[d][v] *= c_sm;  // dS' went into dQ / dK without sm_scale
   if (kDQ) {
     write(p.dq, p.dq_sb, p.dq_st, p.dq_sh, acc1);
   } else {
