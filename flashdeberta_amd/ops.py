@@ -275,15 +275,25 @@ def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=
         lut, radius = delta_lut_device(position_buckets, max_relative_positions, q.device)
         a.delta_lut, a.lut_radius, a.att_span = lut.data_ptr(), radius, span
         a.bias_stride_b, a.bias_stride_t, a.bias_stride_h = L * 2 * span, 2 * span, B * L * 2 * span
-    if pos_key is not None:
-        qh, pk_t = heads_first(q), pos_key[:, :2 * span].transpose(1, 2).to(q.dtype)
-        c2p = torch.bmm(qh, pk_t)                                # [H, B*L, 2S] = q . K_r^T, in the inputs' type like the reference's
+    both = pos_key is not None and pos_query is not None
+    if both:
+        # both terms: their tensors stacked, [2H, B*L, ...], so that each GEMM around the kernel is one call over 2H
+        # matrices instead of two over H (a third less time at 4 k tokens; the reduction over tokens, which has few
+        # output tiles, gains most)
+        x2 = torch.stack([heads_first(q), heads_first(k)]).view(2 * H, B * L, D)
+        pos2 = torch.stack([pos_key[:, :2 * span], pos_query[:, :2 * span]]).view(2 * H, 2 * span, D).to(q.dtype)
+        scores2 = torch.bmm(x2, pos2.transpose(1, 2))        # [2H, B*L, 2S] = (q . K_r^T, k . Q_r^T), in the inputs' type like the reference's
+        d_scores2 = torch.zeros_like(scores2)
+        c2p, p2c, d_c2p, d_p2c = scores2[:H], scores2[H:], d_scores2[:H], d_scores2[H:]
+    elif pos_key is not None:
+        c2p = torch.bmm(heads_first(q), pos_key[:, :2 * span].transpose(1, 2).to(q.dtype))
         d_c2p = torch.zeros_like(c2p)
-        a.c2p_bias, a.d_c2p_bias = c2p.data_ptr(), d_c2p.data_ptr()
-    if pos_query is not None:
-        kh, pq_t = heads_first(k), pos_query[:, :2 * span].transpose(1, 2).to(k.dtype)
-        p2c = torch.bmm(kh, pq_t)
+    elif pos_query is not None:
+        p2c = torch.bmm(heads_first(k), pos_query[:, :2 * span].transpose(1, 2).to(k.dtype))
         d_p2c = torch.zeros_like(p2c)
+    if c2p is not None:
+        a.c2p_bias, a.d_c2p_bias = c2p.data_ptr(), d_c2p.data_ptr()
+    if p2c is not None:
         a.p2c_bias, a.d_p2c_bias = p2c.data_ptr(), d_p2c.data_ptr()
     if delta is None:
         out = out if out.stride(-1) == 1 else out.contiguous()
@@ -315,19 +325,37 @@ def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=
         check(lib.fdb_attn_bwd(ctypes.byref(a), _stream_ptr(q.device)), "fdb_attn_bwd")
     dpk = dpq = None
 
-    def chain(d_scores, x, pos, dx):
-        """score = x . pos[delta]: both factors get their share.  d_scores [H, B*L, 2S] in the inputs' type."""
-        extra = _scores_f32(d_scores, pos[:, :2 * span]).view(H, B, L, D).permute(1, 2, 0, 3)   # into x: [B, L, H, D]
-        dx = extra.add_(dx).to(x.dtype, memory_format=torch.contiguous_format)
-        dpos = _scores_f32(d_scores.transpose(1, 2), heads_first(x)).to(pos.dtype)              # into pos: [H, 2S, D]
-        if pos.shape[1] > 2 * span:  # rows past 2S take no part
-            dpos = torch.cat([dpos, dpos.new_zeros(H, pos.shape[1] - 2 * span, D)], dim=1)
-        return dx, dpos
+    def into_x(dx, extra):  # the content part in the inputs' type plus the position part in fp32, [H', B*L, D] head-major
+        return extra.view(H, B, L, D).permute(1, 2, 0, 3).add_(dx).to(dx.dtype, memory_format=torch.contiguous_format)
 
-    if pos_key is not None:
-        dq, dpk = chain(d_c2p, q, pos_key, dq)
-    if pos_query is not None:
-        dk, dpq = chain(d_p2c, k, pos_query, dk)
+    def into_pos(d_scores, xh, pos):  # [H', B*L, 2S]^T . [H', B*L, D] -> [H', 2S, D]: a reduction over the tokens
+        n_mat, n_tok = d_scores.shape[0], d_scores.shape[1]
+        parts = 8 if n_tok % 8 == 0 and n_tok >= 4096 else 1  # few output tiles: split the tokens, add the parts
+        if parts > 1:
+            dpos = _scores_f32(d_scores.view(n_mat, parts, n_tok // parts, 2 * span).transpose(2, 3).reshape(n_mat * parts, 2 * span, n_tok // parts),
+                               xh.reshape(n_mat * parts, n_tok // parts, D)).view(n_mat, parts, 2 * span, D).sum(1)
+        else:
+            dpos = _scores_f32(d_scores.transpose(1, 2), xh)
+        return dpos
+
+    def pad_rows(dpos, pos):  # rows past 2S take no part
+        dpos = dpos.to(pos.dtype)
+        if pos.shape[1] > 2 * span:
+            dpos = torch.cat([dpos, dpos.new_zeros(H, pos.shape[1] - 2 * span, D)], dim=1)
+        return dpos
+
+    # score = x . pos[delta]: both factors get their share
+    if both:
+        extra2 = _scores_f32(d_scores2, pos2)                  # [2H, B*L, D]
+        dq, dk = into_x(dq, extra2[:H]), into_x(dk, extra2[H:])
+        dpos2 = into_pos(d_scores2, x2, None)
+        dpk, dpq = pad_rows(dpos2[:H], pos_key), pad_rows(dpos2[H:], pos_query)
+    elif pos_key is not None:
+        dq = into_x(dq, _scores_f32(d_c2p, pos_key[:, :2 * span]))
+        dpk = pad_rows(into_pos(d_c2p, heads_first(q), None), pos_key)
+    elif pos_query is not None:
+        dk = into_x(dk, _scores_f32(d_p2c, pos_query[:, :2 * span]))
+        dpq = pad_rows(into_pos(d_p2c, heads_first(k), None), pos_query)
     return dq, dk, dv, dpk, dpq
 
 
