@@ -392,8 +392,10 @@ int fdb_attn_bwd(const fdb_attn_bwd_args* a, void* stream) {
   if (has_pos && (a->bias_stride_t < 2 * a->att_span || a->bias_stride_b < 0 || a->bias_stride_h < 0 ||
                   (int64_t)a->seqlen * a->bias_stride_t > 0x7fffffffll)) return FDB_ERR_SHAPE;
   // score gradients leave in aligned groups of four entries
+  const uintptr_t group_bytes = 4u * (uintptr_t)qk_elem_size(a->dtype);  // one store: four entries
   if (has_pos && ((a->att_span & 1) || (a->bias_stride_b & 3) || (a->bias_stride_t & 3) || (a->bias_stride_h & 3) ||
-                  !aligned16(a->d_c2p_bias) || !aligned16(a->d_p2c_bias))) return FDB_ERR_ALIGN;
+                  reinterpret_cast<uintptr_t>(a->d_c2p_bias) % group_bytes || reinterpret_cast<uintptr_t>(a->d_p2c_bias) % group_bytes))
+    return FDB_ERR_ALIGN;
   const int sz = qk_elem_size(a->dtype);
   const void* ptrs[] = {a->q, a->k, a->v, a->dout, a->dq, a->dk, a->dv, a->out};
   for (const void* ptr : ptrs)

@@ -105,6 +105,19 @@ def test_causal(dtype):
     _check(out, ref, TOL[dtype])
 
 
+@pytest.mark.parametrize("terms", [(False, False), (True, False), (False, True)], ids=["content", "c2p", "p2c"])
+@pytest.mark.parametrize("L,D", [(64, 64), (129, 32), (300, 64), (700, 128)])
+def test_causal_with_fewer_terms(terms, L, D):
+    """Causal runs with no or one position term: without a position term no tile is near, and the tiles that
+    cross the diagonal still have to be masked (they were not, once)."""
+    c2p, p2c = terms
+    q, k, v, pk, pq = _inputs(2, L, 2, D, 32, 64, torch.float32, 70 + L, 1.0, c2p, p2c)
+    ref = _oracle_blhd(q, k, v, pk, pq, 32, 64, causal=True)
+    out = ops.disentangled_attention_fwd(_dev(q), _dev(k), _dev(v), _dev(pk), _dev(pq), position_buckets=32,
+                                         max_relative_positions=64, causal=True)
+    _check(out, ref, TOL[torch.float32])
+
+
 def test_strided_inputs_and_reference_call_shape():
     # [B, H, L, D] tensors as the reference op takes them (flash_attention.py:1088) and a fused qkv buffer
     B, L, H, D = 2, 160, 2, 64
@@ -1077,7 +1090,7 @@ def _random_case(seed):
     return B, L, H, D, pb, mr, terms[0], terms[1], causal, lens, dtype
 
 
-@pytest.mark.parametrize("seed", list(range(24)))
+@pytest.mark.parametrize("seed", list(range(int(os.environ.get("FDB_RANDOM_CASES", "64")))))
 def test_random_shapes_forward_and_backward(seed):
     """Seeded random draws over batch, length (around the 32 / 64 / 128 tile edges), heads, head_dim, bucket
     configuration, terms, causal, padded rows and element type: output and all five gradients against the oracle."""
@@ -1112,4 +1125,5 @@ def test_random_shapes_forward_and_backward(seed):
         if mask is not None and r.ndim == 4:
             r = r * mask[:, :, None, None]
         err = np.abs(got - r).max()
-        assert not np.isnan(got).any() and err <= tol * max(np.abs(r).max(), 1e-3), "%s %s: err %.3e, ref max %.3e" % (what, n, err, np.abs(r).max())
+        # (a gradient that is zero by construction, e.g. dq of a single-token sequence, comes out as rounding noise)
+        assert not np.isnan(got).any() and err <= tol * max(np.abs(r).max(), 1e-2), "%s %s: err %.3e, ref max %.3e" % (what, n, err, np.abs(r).max())
