@@ -1127,3 +1127,62 @@ def test_random_shapes_forward_and_backward(seed):
         err = np.abs(got - r).max()
         # (a gradient that is zero by construction, e.g. dq of a single-token sequence, comes out as rounding noise)
         assert not np.isnan(got).any() and err <= tol * max(np.abs(r).max(), 1e-2), "%s %s: err %.3e, ref max %.3e" % (what, n, err, np.abs(r).max())
+
+
+@pytest.mark.parametrize("seed", list(range(int(os.environ.get("FDB_RANDOM_CASES", "64")))))
+def test_random_forward_variants(seed):
+    """Seeded random draws over what selects a code path of the forward: element type, head_dim, which position
+    terms (none included), causal, fixed / padded / packed layout, length, shared far and near keys, the one-kernel
+    mode and the entry point that allocates nothing; output against the oracle."""
+    r = np.random.RandomState(10_000 + seed)
+    dtype = [torch.bfloat16, torch.float16, torch.float32][r.randint(3)]
+    D = int(r.choice([32, 64, 64, 128]))
+    pb, mr = [(256, 512), (32, 64), (0, 48), (16, 32), (8, 16), (64, 512)][r.randint(6)]
+    c2p, p2c = [(True, True), (True, True), (True, False), (False, True), (False, False)][r.randint(5)]
+    causal = bool(r.randint(4) == 0)
+    L = int(r.choice([r.randint(1, 130), r.randint(130, 400), r.randint(400, 1000)]))
+    H = int(r.choice([1, 2]))
+    layout = ["fixed", "padded", "packed"][r.randint(3)]
+    kw = dict(position_buckets=pb, max_relative_positions=mr, causal=causal)
+    if r.randint(5) == 0:
+        kw["single_kernel"] = True
+    else:
+        kw["far_splits"], kw["near_splits"] = int(r.randint(4)), int(r.randint(3))
+        if r.randint(4) == 0:
+            kw["no_alloc"] = True
+    what = "seed %d %s D%d %d/%d terms %d%d causal %d L%d H%d %s %s" % (seed, str(dtype)[6:], D, pb, mr, c2p, p2c, causal, L, H, layout, kw)
+    print(what, flush=True)
+    tol = TOL[dtype]
+    if layout == "packed":
+        lens = [int(r.randint(1, L + 1)) for _ in range(int(r.randint(1, 4)))] + [L]
+        q, k, v, pk, pq = _inputs(1, sum(lens), H, D, pb, mr, dtype, 20_000 + seed, 1.0, c2p, p2c)
+        cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+        if kw.get("no_alloc"):
+            kw["out"] = torch.empty(sum(lens), H, D, dtype=dtype, device="cuda")
+        out = ops.disentangled_attention_fwd(_dev(q[0]), _dev(k[0]), _dev(v[0]), _dev(pk), _dev(pq), cu_seqlens=cu.cuda(), max_seqlen=max(lens), **kw)
+        off = 0
+        for n in lens:
+            sl = slice(off, off + n)
+            _check(out[sl][None], _oracle_blhd(q[:, sl], k[:, sl], v[:, sl], pk, pq, pb, mr, causal=causal), tol, what + " length %d" % n)
+            off += n
+        return
+    B = int(r.choice([1, 2, 3]))
+    q, k, v, pk, pq = _inputs(B, L, H, D, pb, mr, dtype, 20_000 + seed, 1.0, c2p, p2c)
+    if layout == "padded":
+        lens = [int(r.randint(1, L + 1)) for _ in range(B)]
+        starts = [int(r.randint(0, L - n + 1)) for n in lens]
+        kw["seq_len"] = torch.tensor(lens, dtype=torch.int32, device="cuda")
+        kw["seq_start"] = torch.tensor(starts, dtype=torch.int32, device="cuda")
+        kw["out"] = torch.zeros(B, L, H, D, dtype=dtype, device="cuda")
+        out = ops.disentangled_attention_fwd(_dev(q), _dev(k), _dev(v), _dev(pk), _dev(pq), **kw)
+        for b in range(B):
+            sl = slice(starts[b], starts[b] + lens[b])
+            ref = _oracle_blhd(q[b:b + 1, sl], k[b:b + 1, sl], v[b:b + 1, sl], pk, pq, pb, mr, causal=causal)
+            _check(out[b:b + 1, sl], ref, tol, what + " row %d" % b)
+            rest = torch.cat([out[b, :starts[b]], out[b, starts[b] + lens[b]:]])
+            assert not rest.any(), what + ": rows outside the sequence were written"
+        return
+    if kw.get("no_alloc"):
+        kw["out"] = torch.empty(B, L, H, D, dtype=dtype, device="cuda")
+    out = ops.disentangled_attention_fwd(_dev(q), _dev(k), _dev(v), _dev(pk), _dev(pq), **kw)
+    _check(out, _oracle_blhd(q, k, v, pk, pq, pb, mr, causal=causal), tol, what)
