@@ -1186,3 +1186,71 @@ def test_random_forward_variants(seed):
         kw["out"] = torch.empty(B, L, H, D, dtype=dtype, device="cuda")
     out = ops.disentangled_attention_fwd(_dev(q), _dev(k), _dev(v), _dev(pk), _dev(pq), **kw)
     _check(out, _oracle_blhd(q, k, v, pk, pq, pb, mr, causal=causal), tol, what)
+
+
+@pytest.mark.parametrize("seed", list(range(int(os.environ.get("FDB_RANDOM_MODULE_CASES", "24")))))
+def test_random_module_configurations_against_live_eager(seed):
+    """Seeded random draws over the module's configuration space (which position terms, shared or separate
+    position projections, bucketed or not, relative attention off) and mask forms (none, right / left padding as a
+    2-D mask, the encoder's 4-D outer product): forward and, through autograd, the gradients of the hidden states,
+    the relative embeddings and every weight, fp32, against transformers' eager class on the host."""
+    from transformers.models.deberta_v2.modeling_deberta_v2 import DisentangledSelfAttention
+
+    from flashdeberta_amd import FlashDisentangledSelfAttention
+
+    r = np.random.RandomState(30_000 + seed)
+    heads = int(r.choice([1, 2, 4]))
+    hd = int(r.choice([32, 64]))
+    rel_att = bool(r.randint(5) != 0)
+    buckets, max_rel = [(-1, 40), (32, 64), (256, 512), (16, -1), (8, 24)][r.randint(5)]
+
+    class Cfg:
+        hidden_size, num_attention_heads = heads * hd, heads
+        attention_probs_dropout_prob = hidden_dropout_prob = 0.0
+        pos_att_type = [[], ["c2p"], ["p2c"], ["c2p", "p2c"], ["p2c", "c2p"]][r.randint(5)] if rel_att else []
+        relative_attention, position_buckets, max_relative_positions = rel_att, buckets, max_rel
+        max_position_embeddings, share_att_key = 64, bool(r.randint(2))
+
+    B, L = int(r.choice([1, 2, 3])), int(r.choice([5, 33, 64, 100, 129, 200]))
+    what = "seed %d heads %d x %d rel %d terms %s buckets %d max_rel %d share %d B%d L%d" % (
+        seed, heads, hd, rel_att, Cfg.pos_att_type, buckets, max_rel, Cfg.share_att_key, B, L)
+    torch.manual_seed(40_000 + seed)
+    eager = DisentangledSelfAttention(Cfg()).train()
+    flash = FlashDisentangledSelfAttention(Cfg()).train()
+    flash.load_state_dict(eager.state_dict())
+    flash = flash.cuda()
+    span = eager.pos_ebd_size if rel_att else 1
+    hidden, rel, gout = torch.randn(B, L, Cfg.hidden_size), torch.randn(2 * span, Cfg.hidden_size), torch.randn(B, L, Cfg.hidden_size)
+    form = ["none", "right", "left", "4d"][r.randint(4)]
+    mask2 = torch.ones(B, L)
+    if form != "none":
+        for b in range(B):
+            n = int(r.randint(1, L + 1))
+            if form == "left":
+                mask2[b, :L - n] = 0
+            else:
+                mask2[b, n:] = 0
+    ext = mask2[:, None, None, :] * mask2[:, None, :, None]
+    what += " mask " + form
+    print(what, flush=True)
+    gout = gout * mask2[:, :, None]
+    h0 = hidden.clone().requires_grad_(True)
+    r0 = rel.clone().requires_grad_(True)
+    ref = eager(h0, ext, rel_embeddings=r0 if rel_att else None)[0]
+    (ref * gout).sum().backward()
+    h1 = hidden.cuda().requires_grad_(True)
+    r1 = rel.cuda().requires_grad_(True)
+    am = {"none": None, "right": mask2.cuda(), "left": mask2.cuda(), "4d": ext.cuda()}[form]
+    out = flash(h1, am, rel_embeddings=r1 if rel_att else None)[0]
+    (out * gout.cuda()).sum().backward()
+    valid = mask2.bool().numpy()[:, :, None]
+    _check(out.detach(), np.where(valid, ref.detach().numpy(), 0), 2e-4, what)
+    pairs = [("hidden", h0.grad, h1.grad)] + ([("rel", r0.grad, r1.grad)] if rel_att and Cfg.pos_att_type else []) + [
+        (n, p0.grad, p1.grad) for (n, p0), (_, p1) in zip(eager.named_parameters(), flash.named_parameters())]
+    for name, a, b in pairs:
+        if a is None:
+            assert b is None or not b.any(), (what, name)
+            continue
+        refg = a.numpy()
+        err = np.abs(b.float().cpu().numpy() - refg).max()
+        assert err <= 5e-4 * max(np.abs(refg).max(), 1e-2), (what, name, err, np.abs(refg).max())
