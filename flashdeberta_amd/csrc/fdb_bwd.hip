@@ -111,7 +111,7 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
     x1f[s] = x_ok ? QT::load(x1b + ((int64_t)xr * x1_st + 16 * s + 8 * g) * QT::SZ) : QT::zero();
     x2f[s] = x_ok ? QT::load(x2b + ((int64_t)xr * x2_st + 16 * s + 8 * g) * QT::SZ) : QT::zero();
   }
-  // row statistics and position-score rows are token-major: row (b, tok0 + l), head h
+  // row statistics (log-sum-exp, delta) are token-major: row (b, tok0 + l), head h
   const int64_t tok_x = ((int64_t)b * p.L + tok0 + (x_ok ? xr : 0)) * p.H + h;
   float lse_x = 0.f, del_x = 0.f;
   if (kDQ) {
