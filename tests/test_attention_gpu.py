@@ -1140,7 +1140,7 @@ def test_random_forward_variants(seed):
     pb, mr = [(256, 512), (32, 64), (0, 48), (16, 32), (8, 16), (64, 512)][r.randint(6)]
     c2p, p2c = [(True, True), (True, True), (True, False), (False, True), (False, False)][r.randint(5)]
     causal = bool(r.randint(4) == 0)
-    L = int(r.choice([r.randint(1, 130), r.randint(130, 400), r.randint(400, 1000)]))
+    L = int(r.choice([r.randint(1, 130), r.randint(130, 400), r.randint(400, int(os.environ.get("FDB_RANDOM_MAXLEN", "1000")))]))
     H = int(r.choice([1, 2]))
     layout = ["fixed", "padded", "packed"][r.randint(3)]
     kw = dict(position_buckets=pb, max_relative_positions=mr, causal=causal)
@@ -1254,3 +1254,48 @@ def test_random_module_configurations_against_live_eager(seed):
         refg = a.numpy()
         err = np.abs(b.float().cpu().numpy() - refg).max()
         assert err <= 5e-4 * max(np.abs(refg).max(), 1e-2), (what, name, err, np.abs(refg).max())
+
+
+@pytest.mark.parametrize("seed", list(range(int(os.environ.get("FDB_RANDOM_FP8_CASES", "16")))))
+def test_random_fp8_variants(seed):
+    """Seeded random draws over the FP8 Q/K variant: head_dim (64: expanded to bf16 by default; 128: always the fp8
+    MFMA kernel), one or two position terms, causal, fixed / packed layout, the one-kernel mode; against the oracle on
+    the de-quantised operands."""
+    r = np.random.RandomState(50_000 + seed)
+    D = int(r.choice([64, 64, 128, 32]))
+    pb, mr = [(256, 512), (32, 64), (0, 48), (16, 32)][r.randint(4)]
+    c2p, p2c = [(True, True), (True, True), (True, False), (False, True), (False, False)][r.randint(5)]
+    causal = bool(r.randint(4) == 0)
+    L = int(r.choice([r.randint(1, 130), r.randint(130, 500), r.randint(500, 1200)]))
+    H, B = int(r.choice([1, 2, 3])), int(r.choice([1, 2]))
+    single = bool(r.randint(3) == 0)
+    packed = bool(r.randint(3) == 0)
+    what = "seed %d D%d %d/%d terms %d%d causal %d L%d H%d B%d single %d packed %d" % (seed, D, pb, mr, c2p, p2c, causal, L, H, B, single, packed)
+    print(what, flush=True)
+    lens = [int(r.randint(1, L + 1)) for _ in range(2)] + [L] if packed else None
+    T = sum(lens) if packed else L
+    q, k, v, pk, pq = _inputs(1 if packed else B, T, H, D, pb, mr, torch.bfloat16, 60_000 + seed, 1.0, c2p, p2c)
+    quant = lambda x: ops.quantize_e4m3_per_head(x.cuda().reshape(-1, H, D))
+    q8, qs = quant(q)
+    k8, ks = quant(k)
+    kw = dict(position_buckets=pb, max_relative_positions=mr, causal=causal, single_kernel=single, q_scale=qs, k_scale=ks)
+    dq = lambda y, s: y.float().cpu() * s.cpu()[:, None]
+    pk_dq = pq_dq = pk8 = pq8 = None
+    if c2p:
+        pk8, kw["pos_key_scale"] = ops.quantize_e4m3_per_head(pk.cuda().transpose(0, 1))
+        pk_dq, pk8 = dq(pk8, kw["pos_key_scale"]).transpose(0, 1), pk8.transpose(0, 1)
+    if p2c:
+        pq8, kw["pos_query_scale"] = ops.quantize_e4m3_per_head(pq.cuda().transpose(0, 1))
+        pq_dq, pq8 = dq(pq8, kw["pos_query_scale"]).transpose(0, 1), pq8.transpose(0, 1)
+    q_dq, k_dq = dq(q8, qs).view(q.shape), dq(k8, ks).view(k.shape)
+    if packed:
+        cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+        out = ops.disentangled_attention_fwd(q8, k8, v[0].cuda(), pk8, pq8, cu_seqlens=cu.cuda(), max_seqlen=max(lens), **kw)
+        off = 0
+        for n in lens:
+            sl = slice(off, off + n)
+            _check(out[sl][None], _oracle_blhd(q_dq[:, sl], k_dq[:, sl], v[:, sl], pk_dq, pq_dq, pb, mr, causal=causal), TOL[torch.bfloat16], what + " length %d" % n)
+            off += n
+    else:
+        out = ops.disentangled_attention_fwd(q8.view(B, L, H, D), k8.view(B, L, H, D), v.cuda(), pk8, pq8, **kw)
+        _check(out, _oracle_blhd(q_dq, k_dq, v, pk_dq, pq_dq, pb, mr, causal=causal), TOL[torch.bfloat16], what)
