@@ -1077,7 +1077,7 @@ def test_backward_refuses_an_odd_span():
 def _random_case(seed):
     r = np.random.RandomState(seed)
     B = int(r.choice([1, 2, 3]))
-    L = int(r.choice([1, 31, 32, 33, 63, 64, 65, 96, 127, 128, 129, 160, 255, 257, 300, 420]))
+    L = int(r.choice([1, 31, 32, 33, 63, 64, 65, 96, 127, 128, 129, 160, 255, 257, 300, 420, int(r.randint(420, int(os.environ.get("FDB_RANDOM_MAXLEN", "700"))))]))
     H = int(r.choice([1, 2, 3]))
     D = int(r.choice([32, 64, 64, 128]))
     pb, mr = [(8, 16), (32, 64), (16, 96), (0, 40), (0, 150), (256, 512)][r.randint(6)]
