@@ -391,3 +391,74 @@ def test_delta_table_is_monotone_with_unit_steps():
         steps = np.diff(lut.astype(np.int64))
         assert steps.min() >= 0 and steps.max() <= 1, (pb, mr)
         assert lut[0] >= 0 and lut[-1] <= 2 * ops.att_span(pb, mr) - 1
+
+
+def _header_struct_fields(name):
+    """(field name, C type) pairs of `typedef struct <name> { ... } <name>;` in include/fdb.h, in order."""
+    text = open(os.path.join(ROOT, "include", "fdb.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    body = text[text.index("typedef struct %s {" % name):text.index("} %s;" % name)].split("{", 1)[1]
+    out = []
+    for decl in body.split(";"):
+        decl = " ".join(decl.split())
+        if not decl:
+            continue
+        m = re.match(r"((?:const )?[a-z0-9_]+\s*\*?)\s*(.*)", decl)
+        ctype, names = m.group(1).replace(" *", "*").strip(), m.group(2)
+        for n in names.split(","):
+            n = n.strip()
+            if n.startswith("*"):
+                n, t = n[1:].strip(), ctype + "*"
+            else:
+                t = ctype
+            out.append((n, t))
+    return out
+
+
+@pytest.mark.parametrize("name,mirror", [("fdb_attn_args", _lib.FdbAttnArgs), ("fdb_attn_bwd_args", _lib.FdbAttnBwdArgs)])
+def test_struct_mirrors_follow_the_header_field_by_field(name, mirror):
+    ctype_of = {"int64_t": ctypes.c_int64, "int32_t": ctypes.c_int32, "float": ctypes.c_float}
+    fields = _header_struct_fields(name)
+    assert [n for n, _ in fields] == [n for n, _ in mirror._fields_]
+    for (n, t), (_, ct) in zip(fields, mirror._fields_):
+        assert ct is (ctypes.c_void_p if t.endswith("*") else ctype_of[t]), (n, t, ct)
+    size = lib.fdb_attn_args_size() if name == "fdb_attn_args" else lib.fdb_attn_bwd_args_size()
+    assert size == ctypes.sizeof(mirror)
+
+
+def _good_bwd_args():
+    a = _lib.FdbAttnBwdArgs()
+    for n in ("q", "k", "v", "dout", "dq", "dk", "dv", "out"):
+        setattr(a, n, 0x1000)
+    a.lse = a.delta = 0x2000
+    a.c2p_bias = a.p2c_bias = 0x3000
+    a.d_c2p_bias = a.d_p2c_bias = 0x4000
+    a.delta_lut = 0x5000
+    for n in ("q", "k", "v", "do", "out", "dq", "dk", "dv"):
+        setattr(a, n + "_stride_b", 512 * 768)
+        setattr(a, n + "_stride_t", 768)
+        setattr(a, n + "_stride_h", 64)
+    a.bias_stride_b, a.bias_stride_t, a.bias_stride_h = 512 * 512, 512, 2 * 512 * 512
+    a.batch, a.heads, a.head_dim, a.seqlen = 2, 12, 64, 512
+    a.att_span, a.lut_radius, a.dtype, a.sm_scale = 256, 512, _lib.FDB_BF16, 0.0721
+    return a
+
+
+def test_backward_argument_validation_codes():
+    """Every refusal of fdb_attn_bwd comes before anything touches the GPU, so it can be checked without one."""
+    call = lambda a: lib.fdb_attn_bwd(ctypes.byref(a), None)
+    assert lib.fdb_attn_bwd(None, None) == -1
+    a = _good_bwd_args(); a.dq = None; assert call(a) == -1
+    a = _good_bwd_args(); a.d_c2p_bias = None; assert call(a) == -1       # a term without its gradient tensor
+    a = _good_bwd_args(); a.dtype = _lib.FDB_FP8_E4M3; assert call(a) == -2
+    a = _good_bwd_args(); a.head_dim = 48; assert call(a) == -3
+    a = _good_bwd_args(); a.k = 0x1008; assert call(a) == -4
+    a = _good_bwd_args(); a.dk_stride_t = 772; assert call(a) == -4
+    a = _good_bwd_args(); a.att_span = 255; a.bias_stride_t = 512; assert call(a) == -4   # 2S must be a multiple of 4
+    a = _good_bwd_args(); a.bias_stride_h = 2 * 512 * 512 + 2; assert call(a) == -4
+    a = _good_bwd_args(); a.d_p2c_bias = 0x4004; assert call(a) == -4      # a store group is four elements
+    a = _good_bwd_args(); a.d_p2c_bias = 0x4008; a.seqlen = 0; assert call(a) == -5       # (8-byte alignment is enough for 16-bit types)
+    a = _good_bwd_args(); a.bias_stride_t = 500; assert call(a) == -5      # rows shorter than 2S
+    a = _good_bwd_args(); a.seqlen, a.bias_stride_t = 1 << 20, 1 << 12; assert call(a) == -5  # 32-bit offsets
+    a = _good_bwd_args(); a.delta_lut = None; assert call(a) == -6
+    a = _good_bwd_args(); a.lut_radius = 0; assert call(a) == -6
