@@ -247,50 +247,28 @@ def _scores_f32(x, pos_t):
     return torch.bmm(x.to(torch.float32), pos_t.to(torch.float32))
 
 
-def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=None, *, sm_scale=None, position_buckets=0,
-                               max_relative_positions=0, causal=False, seq_start=None, seq_len=None, delta=None):
-    """Backward of the fixed layout: q, k, v, out, dout [B, L, H, D], lse [B*L, H] as the forward returns it,
-    pos_key = K_r / pos_query = Q_r [H, 2S, D] or None  ->  (dq, dk, dv, d pos_key, d pos_query).
-    Counterpart of FlashAttentionDisentangled.backward (reference flash_attention.py:1066-1086), which hands
-    flash_attn_v2_bwd_dise the position-score tensors and gets their gradients back; as there, those tensors
-    are two GEMMs around the kernel (here head-major [H, B*L, 2S]) and the chain through K_r / Q_r and back into
-    q / k is four more.  delta: (dout * out).sum(-1) as fp32 [B*L, H] if the caller has it (then `out` is not
-    read); by default the first launch computes it."""
+def attention_bwd_kernels(q, k, v, dout, lse, *, out=None, delta=None, c2p=None, p2c=None, d_c2p=None, d_p2c=None, sm_scale,
+                          position_buckets=0, max_relative_positions=0, causal=False, seq_start=None, seq_len=None):
+    """The two backward launches (fdb_attn_bwd) on tensors the caller made: q, k, v, dout [B, L, H, D]; lse [B*L, H];
+    either `out` (the forward's output; the call then computes delta itself) or `delta` [B*L, H] fp32; the position
+    scores c2p = q . K_r^T / p2c = k . Q_r^T and their zeroed gradient tensors as views of logical shape
+    [B, L, H, 2S] with a unit stride on the last axis and any memory layout behind it (all four the same, in q's
+    element type).  Returns dq, dk, dv (content part) and leaves the score gradients in d_c2p / d_p2c."""
     B, L, H, D = q.shape
-    if q.dtype not in _DTYPES:
-        raise ValueError("unsupported dtype %s" % q.dtype)
     span = att_span(position_buckets, max_relative_positions)
-    pos_key = _pos_arg(pos_key, H, D, span, "pos_key")
-    pos_query = _pos_arg(pos_query, H, D, span, "pos_query")
-    if sm_scale is None:
-        sm_scale = 1.0 / math.sqrt(D * (1 + (pos_key is not None) + (pos_query is not None)))
     q, k, v, dout = [x if x.stride(-1) == 1 else x.contiguous() for x in (q, k, v, dout)]
     a = _lib.FdbAttnBwdArgs()
     f32 = torch.float32
-    c2p = p2c = d_c2p = d_p2c = None
-    # Position scores and their gradients are head-major, [H, B*L, 2S] in the inputs' type: what a batched GEMM over the heads
-    # writes and reads as it stands (a token-major tensor would cost a transposing copy of it each way).
-    heads_first = lambda x: x.permute(2, 0, 1, 3).reshape(H, B * L, D)  # a view of [B, L, H, D] when that is contiguous
-    if pos_key is not None or pos_query is not None:
+    scores = [x for x in (c2p, p2c, d_c2p, d_p2c) if x is not None]
+    if scores:
         lut, radius = delta_lut_device(position_buckets, max_relative_positions, q.device)
         a.delta_lut, a.lut_radius, a.att_span = lut.data_ptr(), radius, span
-        a.bias_stride_b, a.bias_stride_t, a.bias_stride_h = L * 2 * span, 2 * span, B * L * 2 * span
-    both = pos_key is not None and pos_query is not None
-    if both:
-        # both terms: their tensors stacked, [2H, B*L, ...], so that each GEMM around the kernel is one call over 2H
-        # matrices instead of two over H (a third less time at 4 k tokens; the reduction over tokens, which has few
-        # output tiles, gains most)
-        x2 = torch.stack([heads_first(q), heads_first(k)]).view(2 * H, B * L, D)
-        pos2 = torch.stack([pos_key[:, :2 * span], pos_query[:, :2 * span]]).view(2 * H, 2 * span, D).to(q.dtype)
-        scores2 = torch.bmm(x2, pos2.transpose(1, 2))        # [2H, B*L, 2S] = (q . K_r^T, k . Q_r^T), in the inputs' type like the reference's
-        d_scores2 = torch.zeros_like(scores2)
-        c2p, p2c, d_c2p, d_p2c = scores2[:H], scores2[H:], d_scores2[:H], d_scores2[H:]
-    elif pos_key is not None:
-        c2p = torch.bmm(heads_first(q), pos_key[:, :2 * span].transpose(1, 2).to(q.dtype))
-        d_c2p = torch.zeros_like(c2p)
-    elif pos_query is not None:
-        p2c = torch.bmm(heads_first(k), pos_query[:, :2 * span].transpose(1, 2).to(k.dtype))
-        d_p2c = torch.zeros_like(p2c)
+        st = scores[0].stride()
+        for x in scores:
+            if tuple(x.shape) != (B, L, H, 2 * span) or x.stride() != st or st[3] != 1 or x.dtype != q.dtype:
+                raise ValueError("position-score tensors: views of shape [B, L, H, 2S] = %s with one layout and q's element type"
+                                 % ((B, L, H, 2 * span),))
+        a.bias_stride_b, a.bias_stride_t, a.bias_stride_h = st[0], st[1], st[2]
     if c2p is not None:
         a.c2p_bias, a.d_c2p_bias = c2p.data_ptr(), d_c2p.data_ptr()
     if p2c is not None:
@@ -323,6 +301,52 @@ def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=
     a.dtype, a.causal, a.sm_scale = _DTYPES[q.dtype], int(bool(causal)), float(sm_scale)
     with torch.cuda.device(q.device):
         check(lib.fdb_attn_bwd(ctypes.byref(a), _stream_ptr(q.device)), "fdb_attn_bwd")
+    return dq, dk, dv
+
+
+def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=None, *, sm_scale=None, position_buckets=0,
+                               max_relative_positions=0, causal=False, seq_start=None, seq_len=None, delta=None):
+    """Backward of the fixed layout: q, k, v, out, dout [B, L, H, D], lse [B*L, H] as the forward returns it,
+    pos_key = K_r / pos_query = Q_r [H, 2S, D] or None  ->  (dq, dk, dv, d pos_key, d pos_query).
+    Counterpart of FlashAttentionDisentangled.backward (reference flash_attention.py:1066-1086), which hands
+    flash_attn_v2_bwd_dise the position-score tensors and gets their gradients back; as there, those tensors
+    are two GEMMs around the kernel (here head-major [H, B*L, 2S]) and the chain through K_r / Q_r and back into
+    q / k is four more.  delta: (dout * out).sum(-1) as fp32 [B*L, H] if the caller has it (then `out` is not
+    read); by default the first launch computes it."""
+    B, L, H, D = q.shape
+    if q.dtype not in _DTYPES:
+        raise ValueError("unsupported dtype %s" % q.dtype)
+    span = att_span(position_buckets, max_relative_positions)
+    pos_key = _pos_arg(pos_key, H, D, span, "pos_key")
+    pos_query = _pos_arg(pos_query, H, D, span, "pos_query")
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(D * (1 + (pos_key is not None) + (pos_query is not None)))
+    q, k, v, dout = [x if x.stride(-1) == 1 else x.contiguous() for x in (q, k, v, dout)]
+    f32 = torch.float32
+    c2p = p2c = d_c2p = d_p2c = None
+    # Position scores and their gradients are head-major, [H, B*L, 2S] in the inputs' type: what a batched GEMM over the heads
+    # writes and reads as it stands (a token-major tensor would cost a transposing copy of it each way).
+    heads_first = lambda x: x.permute(2, 0, 1, 3).reshape(H, B * L, D)  # a view of [B, L, H, D] when that is contiguous
+    both = pos_key is not None and pos_query is not None
+    if both:
+        # both terms: their tensors stacked, [2H, B*L, ...], so that each GEMM around the kernel is one call over 2H
+        # matrices instead of two over H (a third less time at 4 k tokens; the reduction over tokens, which has few
+        # output tiles, gains most)
+        x2 = torch.stack([heads_first(q), heads_first(k)]).view(2 * H, B * L, D)
+        pos2 = torch.stack([pos_key[:, :2 * span], pos_query[:, :2 * span]]).view(2 * H, 2 * span, D).to(q.dtype)
+        scores2 = torch.bmm(x2, pos2.transpose(1, 2))        # [2H, B*L, 2S] = (q . K_r^T, k . Q_r^T), in the inputs' type like the reference's
+        d_scores2 = torch.zeros_like(scores2)
+        c2p, p2c, d_c2p, d_p2c = scores2[:H], scores2[H:], d_scores2[:H], d_scores2[H:]
+    elif pos_key is not None:
+        c2p = torch.bmm(heads_first(q), pos_key[:, :2 * span].transpose(1, 2).to(q.dtype))
+        d_c2p = torch.zeros_like(c2p)
+    elif pos_query is not None:
+        p2c = torch.bmm(heads_first(k), pos_query[:, :2 * span].transpose(1, 2).to(k.dtype))
+        d_p2c = torch.zeros_like(p2c)
+    blhs = lambda x: None if x is None else x.view(H, B, L, 2 * span).permute(1, 2, 0, 3)  # the logical [B, L, H, 2S] view
+    dq, dk, dv = attention_bwd_kernels(q, k, v, dout, lse, out=out, delta=delta, c2p=blhs(c2p), p2c=blhs(p2c), d_c2p=blhs(d_c2p),
+                                       d_p2c=blhs(d_p2c), sm_scale=sm_scale, position_buckets=position_buckets,
+                                       max_relative_positions=max_relative_positions, causal=causal, seq_start=seq_start, seq_len=seq_len)
     dpk = dpq = None
 
     def into_x(dx, extra):  # the content part in the inputs' type plus the position part in fp32, [H', B*L, D] head-major

@@ -1299,3 +1299,35 @@ def test_random_fp8_variants(seed):
     else:
         out = ops.disentangled_attention_fwd(q8.view(B, L, H, D), k8.view(B, L, H, D), v.cuda(), pk8, pq8, **kw)
         _check(out, _oracle_blhd(q_dq, k_dq, v, pk_dq, pq_dq, pb, mr, causal=causal), TOL[torch.bfloat16], what)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_backward_kernels_take_any_layout_of_the_score_tensors(dtype):
+    """fdb_attn_bwd addresses the position-score tensors through three strides: head-major [H, B, L, 2S] (what the
+    operator uses), token-major [B, L, H, 2S] and the reference's [B, H, L, 2S] give the same dq, dk, dv and the same
+    score gradients, bit for bit."""
+    B, L, H, D, pb, mr = 2, 300, 3, 64, 32, 64
+    S2 = 2 * ops.att_span(pb, mr)
+    q, k, v, pk, pq = [x.cuda() for x in _inputs(B, L, H, D, pb, mr, dtype, 4400, 1.0, True, True)]
+    dout = torch.randn(B, L, H, D, generator=torch.Generator().manual_seed(4401)).to(dtype).cuda()
+    kw = dict(position_buckets=pb, max_relative_positions=mr)
+    out, lse = ops.disentangled_attention_fwd(q, k, v, pk, pq, return_lse=True, **kw)
+    c2p = torch.einsum("blhd,hsd->blhs", q.float(), pk.float()).to(dtype)   # logical [B, L, H, 2S]
+    p2c = torch.einsum("blhd,hsd->blhs", k.float(), pq.float()).to(dtype)
+    results = []
+    for order in ((2, 0, 1, 3), (0, 1, 2, 3), (0, 2, 1, 3)):   # memory order of the axes (b, l, h, s)
+        back = tuple(order.index(ax) for ax in range(4))
+        lay = lambda x: x.permute(order).contiguous().permute(back)   # same logical tensor, another layout behind it
+        cc, pp = lay(c2p), lay(p2c)
+        dc, dp = torch.zeros_like(cc), torch.zeros_like(pp)
+        assert cc.shape == (B, L, H, S2) and dc.stride() == cc.stride()
+        dq, dk, dv = ops.attention_bwd_kernels(q, k, v, dout, lse, out=out, c2p=cc, p2c=pp, d_c2p=dc, d_p2c=dp,
+                                               sm_scale=1.0 / np.sqrt(3 * D), **kw)
+        results.append((dq, dk, dv, dc.contiguous(), dp.contiguous()))
+    for other in results[1:]:
+        for a, b in zip(results[0], other):
+            assert torch.equal(a, b)
+    # and a mismatch between the four tensors is refused
+    with pytest.raises(ValueError):
+        ops.attention_bwd_kernels(q, k, v, dout, lse, out=out, c2p=c2p, p2c=p2c.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3),
+                                  d_c2p=torch.zeros_like(c2p), d_p2c=torch.zeros_like(p2c), sm_scale=0.07, **kw)
