@@ -1184,8 +1184,24 @@ def test_random_forward_variants(seed):
         return
     if kw.get("no_alloc"):
         kw["out"] = torch.empty(B, L, H, D, dtype=dtype, device="cuda")
-    out = ops.disentangled_attention_fwd(_dev(q), _dev(k), _dev(v), _dev(pk), _dev(pq), **kw)
-    _check(out, _oracle_blhd(q, k, v, pk, pq, pb, mr, causal=causal), tol, what)
+    qd, kd, vd = _dev(q), _dev(k), _dev(v)
+    views = int(r.randint(3))
+    if views == 1:    # slices of one fused projection buffer [B, L, 3, H, D]
+        qd, kd, vd = torch.stack([qd, kd, vd], dim=2).unbind(2)
+    elif views == 2:  # [B, H, L, D] tensors seen as [B, L, H, D], the reference op's layout
+        qd, kd, vd = [x.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3) for x in (qd, kd, vd)]
+    out = ops.disentangled_attention_fwd(qd, kd, vd, _dev(pk), _dev(pq), **kw)
+    _check(out, _oracle_blhd(q, k, v, pk, pq, pb, mr, causal=causal), tol, what + " views %d" % views)
+    if not kw.get("single_kernel") and not kw.get("no_alloc") and r.randint(2):
+        # the backward on the same strided operands, against the one on contiguous copies
+        bkw = {n: kw[n] for n in ("position_buckets", "max_relative_positions", "causal")}
+        out2, lse = ops.disentangled_attention_fwd(qd, kd, vd, _dev(pk), _dev(pq), return_lse=True, **bkw)
+        dout = torch.randn(B, L, H, D, generator=torch.Generator().manual_seed(seed)).to(dtype).cuda()
+        dd = dout.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3) if views == 2 else dout
+        got = ops.disentangled_attention_bwd(qd, kd, vd, out2, lse, dd, _dev(pk), _dev(pq), **bkw)
+        want = ops.disentangled_attention_bwd(_dev(q), _dev(k), _dev(v), out2.contiguous(), lse, dout, _dev(pk), _dev(pq), **bkw)
+        for a, b in zip(got, want):
+            assert (a is None and b is None) or torch.equal(a, b), what + " backward on strided operands"
 
 
 @pytest.mark.parametrize("seed", list(range(int(os.environ.get("FDB_RANDOM_MODULE_CASES", "24")))))
