@@ -1347,3 +1347,42 @@ def test_backward_kernels_take_any_layout_of_the_score_tensors(dtype):
     with pytest.raises(ValueError):
         ops.attention_bwd_kernels(q, k, v, dout, lse, out=out, c2p=c2p, p2c=p2c.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3),
                                   d_c2p=torch.zeros_like(c2p), d_p2c=torch.zeros_like(p2c), sm_scale=0.07, **kw)
+
+
+@pytest.mark.parametrize("what", ["no_alloc_forward", "backward"])
+def test_more_replays_from_a_hip_graph(what):
+    """The entry point that allocates nothing (the case it exists for) and the backward operator (two launches and
+    torch's fills and GEMMs around them) captured into a HIP graph: three replays on fresh input values, with eager
+    work and synchronisations in between, each equal to the eager result on the same values."""
+    B, L, H, D, pb, mr = 2, 700, 2, 64, 32, 64
+    kw = dict(position_buckets=pb, max_relative_positions=mr)
+    q, k, v, pk, pq = [_dev(x) for x in _inputs(B, L, H, D, pb, mr, torch.bfloat16, 910, 1.0)]
+    dout = torch.randn(B, L, H, D, generator=torch.Generator().manual_seed(911)).to(torch.bfloat16).cuda()
+    out_buf = torch.empty_like(q)
+
+    def call():
+        if what == "no_alloc_forward":
+            return (ops.disentangled_attention_fwd(q, k, v, pk, pq, out=out_buf, no_alloc=True, **kw),)
+        out, lse = ops.disentangled_attention_fwd(q, k, v, pk, pq, return_lse=True, **kw)
+        return ops.disentangled_attention_bwd(q, k, v, out, lse, dout, pk, pq, **kw)
+
+    call()  # the delta table reaches the device, and the GEMM library gets its workspaces, outside the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            captured = call()
+    torch.cuda.current_stream().wait_stream(side)
+    g = torch.Generator().manual_seed(912)
+    for it in range(3):
+        for x in (q, k, v, dout):
+            x.copy_(torch.randn(x.shape, generator=g).to(torch.bfloat16))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [x.clone() for x in captured]
+        eager = call()
+        torch.cuda.synchronize()
+        for a, b in zip(got, eager):
+            assert torch.equal(a, b), "%s: replay %d differs from the eager call" % (what, it)
