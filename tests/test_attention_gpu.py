@@ -1386,3 +1386,57 @@ def test_more_replays_from_a_hip_graph(what):
         torch.cuda.synchronize()
         for a, b in zip(got, eager):
             assert torch.equal(a, b), "%s: replay %d differs from the eager call" % (what, it)
+
+
+@pytest.mark.parametrize("seed", list(range(int(os.environ.get("FDB_RANDOM_MODULE_CASES", "24")) // 2)))
+def test_random_encoder_configurations_patched_against_eager(seed):
+    """Seeded random draws over small DeBERTa-v2 encoders of transformers (two layers; terms, buckets, shared or
+    separate position projections, normalised relative embeddings or not, absolute positions or not, relative
+    attention off) with right-padded batches: last hidden state and the gradient of every parameter of the patched
+    model against the same model before patching, fp32."""
+    import copy
+
+    from transformers.models.deberta_v2.modeling_deberta_v2 import DebertaV2Config, DebertaV2Model
+
+    from flashdeberta_amd import patch_model
+
+    r = np.random.RandomState(70_000 + seed)
+    heads = int(r.choice([2, 4]))
+    rel_att = bool(r.randint(6) != 0)
+    cfg = DebertaV2Config(
+        vocab_size=97, hidden_size=heads * 32, num_hidden_layers=2, num_attention_heads=heads, intermediate_size=96,
+        relative_attention=rel_att, pos_att_type=["", "c2p", "p2c", "p2c|c2p"][r.randint(4)] if rel_att else "",
+        position_buckets=int(r.choice([-1, 16, 32])), max_relative_positions=int(r.choice([-1, 24])),
+        share_att_key=bool(r.randint(2)), norm_rel_ebd=["none", "layer_norm"][r.randint(2)],
+        position_biased_input=bool(r.randint(2)), max_position_embeddings=64, hidden_dropout_prob=0.0,
+        attention_probs_dropout_prob=0.0, initializer_range=0.2)
+    B, L = int(r.choice([1, 2, 3])), int(r.choice([7, 33, 64]))
+    what = "seed %d heads %d rel %d terms %r buckets %d max_rel %d share %d norm %s abs %d B%d L%d" % (
+        seed, heads, rel_att, cfg.pos_att_type, cfg.position_buckets, cfg.max_relative_positions, cfg.share_att_key,
+        cfg.norm_rel_ebd, cfg.position_biased_input, B, L)
+    print(what, flush=True)
+    torch.manual_seed(80_000 + seed)
+    eager = DebertaV2Model(cfg).train().cuda()
+    ours = patch_model(copy.deepcopy(eager))
+    ids = torch.randint(0, 97, (B, L), device="cuda")
+    mask = torch.ones(B, L, dtype=torch.long, device="cuda")
+    for b in range(B):
+        mask[b, int(r.randint(1, L + 1)):] = 0
+    gout = torch.randn(B, L, cfg.hidden_size, device="cuda") * mask[:, :, None]
+    outs = []
+    for m in (eager, ours):
+        h = m(input_ids=ids, attention_mask=mask).last_hidden_state
+        (h * gout).sum().backward()
+        outs.append(h.detach() * mask[:, :, None])
+    scale = outs[0].abs().max().item()
+    assert (outs[0] - outs[1]).abs().max().item() <= 2e-4 * max(scale, 1.0), what
+    # (gradients that are zero in exact arithmetic, e.g. of the key bias, are rounding noise on both sides: the floor of
+    # the bound follows the largest gradient of the model)
+    g_all = max(p.grad.abs().max().item() for p in eager.parameters() if p.grad is not None)
+    for (n, p0), (_, p1) in zip(eager.named_parameters(), ours.named_parameters()):
+        if p0.grad is None:
+            assert p1.grad is None or not p1.grad.any(), (what, n)
+            continue
+        assert p1.grad is not None, (what, n)
+        err, ref = (p0.grad - p1.grad).abs().max().item(), p0.grad.abs().max().item()
+        assert err <= 1e-3 * max(ref, 0.02 * g_all), (what, n, err, ref, g_all)
