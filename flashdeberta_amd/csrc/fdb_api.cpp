@@ -108,10 +108,16 @@ bool has_far_launch(const fdb_attn_args* a) {
 int far_parts_wanted(const fdb_attn_args* a) {
   if (!has_far_launch(a) || !fdb_near32_supported(a->dtype, a->head_dim)) return 1;
   if (a->far_splits > 0) return a->far_splits;
-  if (a->cu_seqlens) return 1;  // the lengths, and with them the far tiles per query tile, are on the device
+  // A packed batch has its lengths on the device: the host goes by the mean length (the kernel divides each query
+  // tile's own far tiles among the shares, whatever they are), and only shares when that mean leaves far tiles at all.
+  int32_t typical = a->max_seqlen;
+  if (a->cu_seqlens) {
+    typical = a->total_tokens / a->batch;
+    if (typical < 2 * a->lut_radius + FDB_BM) return 1;
+  }
   const int64_t wgs = query_tiles(a) * a->heads, slots = 3 * (int64_t)cu_count();
   if (wgs >= slots) return 1;
-  const int n64 = (a->max_seqlen + FDB_BN - 1) / FDB_BN;
+  const int n64 = (typical + FDB_BN - 1) / FDB_BN;
   const int near64 = (FDB_BM + 2 * a->lut_radius + 3 * (FDB_BN - 1)) / FDB_BN;  // of a query tile in mid-sequence
   const int most = (n64 - near64) / 8 < FDB_MAX_FAR_PARTS ? (n64 - near64) / 8 : FDB_MAX_FAR_PARTS;
   const int64_t fit = slots / wgs;

@@ -1440,3 +1440,27 @@ def test_random_encoder_configurations_patched_against_eager(seed):
         assert p1.grad is not None, (what, n)
         err, ref = (p0.grad - p1.grad).abs().max().item(), p0.grad.abs().max().item()
         assert err <= 1e-3 * max(ref, 0.02 * g_all), (what, n, err, ref, g_all)
+
+
+def test_packed_batch_of_few_long_sequences_shares_its_far_keys(monkeypatch):
+    """A packed batch whose query tiles leave most of the GPU idle shares the far keys of a tile among workgroups
+    without being told to (the library goes by the mean length; each tile's shares follow its own sequence):
+    same output as without shares, and against the oracle per sequence."""
+    H, D, pb, mr = 2, 64, 256, 512
+    lens = [4096, 3000]
+    q, k, v, pk, pq = _inputs(1, sum(lens), H, D, pb, mr, torch.bfloat16, 930, 1.0)
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32).cuda()
+    kw = dict(cu_seqlens=cu, max_seqlen=max(lens), position_buckets=pb, max_relative_positions=mr)
+    args = (_dev(q[0]), _dev(k[0]), _dev(v[0]), _dev(pk), _dev(pq))
+    asked = []
+    real = ops.lib.fdb_attn_workspace_bytes
+    monkeypatch.setattr(ops.lib, "fdb_attn_workspace_bytes", lambda a: asked.append(real(a)) or asked[-1])
+    auto = ops.disentangled_attention_fwd(*args, **kw)
+    assert asked and asked[0] > 0, "the library asked for no workspace: the far keys are not shared"
+    alone = ops.disentangled_attention_fwd(*args, far_splits=1, near_splits=1, **kw)
+    assert (auto.float() - alone.float()).abs().max().item() <= TOL[torch.bfloat16]
+    off = 0
+    for n in lens:
+        sl = slice(off, off + n)
+        _check(auto[sl][None], _oracle_blhd(q[:, sl], k[:, sl], v[:, sl], pk, pq, pb, mr), TOL[torch.bfloat16], "length %d" % n)
+        off += n
