@@ -223,15 +223,29 @@ def main():
         src = torch.empty(args.copy_calibration << 20, dtype=torch.uint8, device=device)
         dst = torch.empty_like(src)
         dst.copy_(src)
-    # Untimed settle phase before the warm-up: the first ~100 ms after idle run a few percent slower (clocks
-    # and power management), which a short timed region (the driver's 20 steps are 15 ms) would measure
-    # instead of the kernels.  Batches of steps are run until a batch is no faster than the one before
-    # (within 1 %), for at most 0.5 s; the time spent is reported as settle_ms.
+    def timed(warmup, steps):
+        """(wall ms per step, HIP-event ms per step) of `steps` steps after `warmup` untimed ones."""
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        ev0.record()  # same stream the kernel is launched on (torch's current stream)
+        for _ in range(steps):
+            step()
+        ev1.record()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps, ev0.elapsed_time(ev1) / steps
+
+    # First the plain reading of the flags: W warm-up steps, K timed steps, straight from idle (`unsettled` in the
+    # JSON line).  The first ~100 ms after idle run a few percent slower (clocks and power management), and a short
+    # timed region (20 steps are 15 ms) measures that ramp instead of the kernels.  So an untimed settle phase
+    # follows -- batches of steps until a batch is no faster than the one before (within 1 %), for at most 0.5 s,
+    # reported as settle_ms -- and then W warm-up + K timed steps once more: `value`.
+    cold_wall_ms, cold_kern_ms = timed(args.warmup, args.steps)
     settle_t0 = time.perf_counter()
     if not args.no_settle:
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        step()
-        torch.cuda.synchronize()
         prev = None
         while time.perf_counter() - settle_t0 < 0.5:
             e0.record()
@@ -244,18 +258,7 @@ def main():
                 break
             prev = cur
     settle_ms = (time.perf_counter() - settle_t0) * 1e3
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    ev0.record()  # same stream the kernel is launched on (torch's current stream)
-    for _ in range(args.steps):
-        step()
-    ev1.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    kern_ms = ev0.elapsed_time(ev1) / args.steps
+    wall_ms, kern_ms = (cold_wall_ms, cold_kern_ms) if args.no_settle else timed(args.warmup, args.steps)
     fl = flops(lens, H, D) * (3.5 if args.backward else 1.0)
     tokens = sum(lens)
     # e4m3 operands at head_dim <= 64 are expanded to bf16 inside the step (ops.disentangled_attention_fwd) and
@@ -270,7 +273,7 @@ def main():
         far_t, near_t = tile_census(lens)
         split = {}
         for name, mask in (("far", 1), ("near", 2)):
-            run = lambda: ops.disentangled_attention_fwd(*tensors, out=out, _launch_mask=mask, **kw)
+            run = lambda: ops.disentangled_attention_fwd(*tensors, out=out, _part=mask, **kw)
             if (far_t if name == "far" else near_t) == 0:
                 continue
             for _ in range(5):
@@ -295,6 +298,9 @@ def main():
         "metric": "disentangled_attn_fwd_bwd_tflops" if args.backward else "disentangled_attn_fwd_tflops", "value": round(fl / (wall_ms * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 4),
         "settle_ms": round(settle_ms, 1),
+        "unsettled": {"value": round(fl / (cold_wall_ms * 1e-3) / 1e12, 2), "ms_per_step": round(cold_wall_ms, 4),
+                      "kernel_ms": round(cold_kern_ms, 4),
+                      "note": "the same warm-up and steps straight from idle, before the settle phase"},
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": arith, "data": "synthetic",
         "tokens_per_s": round(tokens / (wall_ms * 1e-3), 1),
         "content_only_tflops": round(sum(H * 4 * l * l * D for l in lens) / (wall_ms * 1e-3) / 1e12, 2),

@@ -13,7 +13,8 @@ LIB_PATH = os.path.join(_HERE, "libfdb_hip.so")
 
 FDB_F32, FDB_BF16, FDB_F16, FDB_FP8_E4M3 = 0, 1, 2, 3
 FDB_NOALLOC_SCRATCH_BYTES = 32 * 1024 * 1024
-FDB_VERSION = 6  # of include/fdb.h as mirrored below
+FDB_BWD_MAX_WINDOW = 60  # of include/fdb.h: table rows beyond the first that one 32-row backward step may reach
+FDB_VERSION = 7  # of include/fdb.h as mirrored below
 
 
 class FdbAttnArgs(ctypes.Structure):
@@ -28,7 +29,7 @@ class FdbAttnArgs(ctypes.Structure):
         + [(n, ctypes.c_int32) for n in (
             "batch", "heads", "head_dim", "max_seqlen", "total_tokens", "att_span", "lut_radius", "dtype", "causal", "far_splits",
             "near_splits")]
-        + [("sm_scale", ctypes.c_float), ("launch_mask", ctypes.c_int32)]
+        + [("sm_scale", ctypes.c_float)]
     )
 
 
@@ -38,15 +39,15 @@ class FdbAttnBwdArgs(ctypes.Structure):
             "q", "k", "v", "dout", "dq", "dk", "dv", "lse", "delta", "out", "c2p_bias", "p2c_bias", "d_c2p_bias", "d_p2c_bias",
             "seq_start", "seq_len", "delta_lut")]
         + [(n + s, ctypes.c_int64) for n in ("q", "k", "v", "do", "out", "dq", "dk", "dv", "bias") for s in ("_stride_b", "_stride_t", "_stride_h")]
-        + [(n, ctypes.c_int32) for n in ("batch", "heads", "head_dim", "seqlen", "att_span", "lut_radius", "dtype", "causal")]
+        + [(n, ctypes.c_int32) for n in ("batch", "heads", "head_dim", "seqlen", "att_span", "lut_radius", "lut_window", "dtype", "causal")]
         + [("sm_scale", ctypes.c_float)]
     )
 
 
 EXPORTS = (
-    "fdb_version", "fdb_attn_args_size", "fdb_strerror", "fdb_attn_check", "fdb_attn_fwd", "fdb_attn_fwd_noalloc", "fdb_attn_bwd", "fdb_attn_bwd_args_size", "fdb_attn_workspace_bytes",
+    "fdb_version", "fdb_attn_args_size", "fdb_strerror", "fdb_attn_check", "fdb_attn_fwd", "fdb_attn_fwd_part", "fdb_attn_fwd_noalloc", "fdb_attn_bwd", "fdb_attn_bwd_args_size", "fdb_attn_workspace_bytes",
     "fdb_worklist_ints",
-    "fdb_worklist_max_tiles", "fdb_tile_rows", "fdb_build_worklist", "fdb_delta_lut_radius", "fdb_delta_lut",
+    "fdb_worklist_max_tiles", "fdb_tile_rows", "fdb_build_worklist", "fdb_delta_lut_radius", "fdb_delta_lut", "fdb_delta_lut_window",
     "fdb_quant_e4m3_per_head", "fdb_dequant_e4m3_per_head",
 )
 
@@ -72,6 +73,8 @@ def _load():
     lib.fdb_attn_check.argtypes = [ctypes.POINTER(FdbAttnArgs)]
     lib.fdb_attn_fwd.restype = ctypes.c_int
     lib.fdb_attn_fwd.argtypes = [ctypes.POINTER(FdbAttnArgs), vp]
+    lib.fdb_attn_fwd_part.restype = ctypes.c_int
+    lib.fdb_attn_fwd_part.argtypes = [ctypes.POINTER(FdbAttnArgs), i32, vp]
     lib.fdb_attn_fwd_noalloc.restype = ctypes.c_int
     lib.fdb_attn_fwd_noalloc.argtypes = [ctypes.POINTER(FdbAttnArgs), vp]
     lib.fdb_attn_bwd_args_size.restype = ctypes.c_size_t
@@ -91,6 +94,8 @@ def _load():
     lib.fdb_build_worklist.argtypes = [vp, i32, i32, vp, vp]
     lib.fdb_delta_lut_radius.restype = i32
     lib.fdb_delta_lut_radius.argtypes = [i32, i32]
+    lib.fdb_delta_lut_window.restype = i32
+    lib.fdb_delta_lut_window.argtypes = [i32, i32]
     lib.fdb_delta_lut.restype = ctypes.c_int
     lib.fdb_delta_lut.argtypes = [i32, i32, i32, vp]
     lib.fdb_quant_e4m3_per_head.restype = ctypes.c_int

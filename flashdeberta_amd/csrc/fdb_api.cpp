@@ -221,7 +221,7 @@ const char* fdb_strerror(int code) {
     case FDB_ERR_HEAD_DIM: return "unsupported head_dim (supported: 32, 64, 128)";
     case FDB_ERR_ALIGN: return "pointer or stride is not 16-byte aligned";
     case FDB_ERR_SHAPE: return "batch/heads/max_seqlen/total_tokens invalid";
-    case FDB_ERR_SPAN: return "att_span/lut_radius/delta_lut invalid while a position term is present";
+    case FDB_ERR_SPAN: return "att_span/lut_radius/delta_lut invalid while a position term is present (backward: or lut_window beyond FDB_BWD_MAX_WINDOW)";
     case FDB_ERR_SCALE: return "fp8 dtype needs q_scale, k_scale and a scale for each position tensor";
     case FDB_ERR_WORKLIST: return "cu_seqlens given without a work-list buffer";
     case FDB_ERR_LUT_ARGS: return "invalid position_buckets/max_position/radius/out for the delta table";
@@ -257,7 +257,7 @@ int fdb_attn_check(const fdb_attn_args* a) {
   if (a->batch < 1 || a->heads < 1 || a->heads > 65535 || a->max_seqlen < 1 || a->total_tokens < 1)
     return FDB_ERR_SHAPE;
   if (a->far_splits < 0 || a->far_splits > FDB_MAX_FAR_SPLITS || a->near_splits < 0 ||
-      a->near_splits > FDB_MAX_FAR_SPLITS || a->workspace_bytes < 0 || a->launch_mask < 0 || a->launch_mask > 2)
+      a->near_splits > FDB_MAX_FAR_SPLITS || a->workspace_bytes < 0)
     return FDB_ERR_SHAPE;
   if (a->workspace && !aligned16(a->workspace)) return FDB_ERR_ALIGN;
   if (!a->cu_seqlens && (int64_t)a->batch * a->max_seqlen != a->total_tokens) return FDB_ERR_SHAPE;
@@ -291,7 +291,12 @@ int64_t fdb_attn_workspace_bytes(const fdb_attn_args* a) {
   return (far_parts_wanted(a) - 1 + (near > 1 ? near : 0)) * far_part_bytes(a);
 }
 
-int fdb_attn_fwd(const fdb_attn_args* a, void* stream) {
+}  // extern "C"
+
+namespace {
+
+// launch_mask 0: the whole call; 1 / 2: only the launch over the far / the near keys (fdb_attn_fwd_part)
+int attn_fwd_impl(const fdb_attn_args* a, int launch_mask, void* stream) {
   const int rc = fdb_attn_check(a);
   if (rc != FDB_OK) return rc;
   FdbKParams p;
@@ -320,6 +325,8 @@ int fdb_attn_fwd(const fdb_attn_args* a, void* stream) {
   p.R = a->lut_radius > 0 ? a->lut_radius : 1;
   p.causal = a->causal ? 1 : 0;
   p.scale_log2 = a->sm_scale * 1.4426950408889634f;
+  // padded fixed layout: the first launch of the call also writes the rows of out outside the real tokens
+  p.fill_pad = (!a->cu_seqlens && (a->seq_start || a->seq_len)) ? 1 : 0;
   const int64_t grid_x = query_tiles(a);
   if (grid_x < 1 || grid_x * a->heads > INT32_MAX) return FDB_ERR_SHAPE;
   p.grid_x = (int32_t)grid_x;
@@ -337,11 +344,12 @@ int fdb_attn_fwd(const fdb_attn_args* a, void* stream) {
     p.ws_slots = p.far_parts - 1 + (p.near_parts > 1 ? p.near_parts : 0);
     p.ws = (char*)a->workspace;
     p.ws_rows = lse_rows(a);
-    if (need_far && a->launch_mask != 2) {
+    if (need_far && launch_mask != 2) {
       const int rc_far = fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, FDB_MODE_FAR_ONLY, stream);
       if (rc_far != 0) return rc_far;
+      p.fill_pad = 0;
     }
-    if (a->launch_mask == 1) return FDB_OK;
+    if (launch_mask == 1) return FDB_OK;
     p.far_done = need_far ? 1 : 0;
     // head_dim 64: the near kernel (32-key steps, two workgroups per CU); head_dim 32: the fused kernel's ring mode
     if (fdb_near32_supported(a->dtype, a->head_dim)) {
@@ -351,7 +359,19 @@ int fdb_attn_fwd(const fdb_attn_args* a, void* stream) {
     }
     return fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, FDB_MODE_NEAR_RING, stream);
   }
+  if (launch_mask != 0) return FDB_ERR_UNSUPPORTED;  // a single kernel has no parts
   return fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, FDB_MODE_FUSED, stream);
+}
+
+}  // namespace
+
+extern "C" {
+
+int fdb_attn_fwd(const fdb_attn_args* a, void* stream) { return attn_fwd_impl(a, 0, stream); }
+
+int fdb_attn_fwd_part(const fdb_attn_args* a, int32_t part, void* stream) {
+  if (part != 1 && part != 2) return FDB_ERR_SHAPE;
+  return attn_fwd_impl(a, part, stream);
 }
 
 int fdb_attn_fwd_noalloc(const fdb_attn_args* a, void* stream) {
@@ -394,6 +414,8 @@ int fdb_attn_bwd(const fdb_attn_bwd_args* a, void* stream) {
   const bool has_pos = a->c2p_bias || a->p2c_bias;
   if ((a->c2p_bias && !a->d_c2p_bias) || (a->p2c_bias && !a->d_p2c_bias)) return FDB_ERR_NULL;
   if (has_pos && (a->att_span < 1 || a->lut_radius < 1 || !a->delta_lut)) return FDB_ERR_SPAN;
+  // the ring that collects a row's score gradients holds the table rows of one 32-row step plus a partly stored group
+  if (has_pos && (a->lut_window < 0 || a->lut_window > FDB_BWD_MAX_WINDOW)) return FDB_ERR_SPAN;
   // the kernels address a sequence's rows of the position-score tensors with 32-bit element offsets
   if (has_pos && (a->bias_stride_t < 2 * a->att_span || a->bias_stride_b < 0 || a->bias_stride_h < 0 ||
                   (int64_t)a->seqlen * a->bias_stride_t > 0x7fffffffll)) return FDB_ERR_SHAPE;
@@ -454,6 +476,18 @@ int32_t fdb_delta_lut_radius(int32_t position_buckets, int32_t max_position) {
                              delta_of(-r, position_buckets, max_position) == 0))
     ++r;
   return r;
+}
+
+int32_t fdb_delta_lut_window(int32_t position_buckets, int32_t max_position) {
+  const int32_t radius = fdb_delta_lut_radius(position_buckets, max_position);
+  if (radius < 1) return FDB_ERR_LUT_ARGS;
+  // delta is constant beyond +-radius, so every 32-row window that matters starts in [-radius - 31, radius]
+  int32_t worst = 0;
+  for (int32_t r = -radius - 31; r <= radius; ++r) {
+    const int32_t w = delta_of(r + 31, position_buckets, max_position) - delta_of(r, position_buckets, max_position);
+    if (w > worst) worst = w;
+  }
+  return worst;
 }
 
 int fdb_delta_lut(int32_t position_buckets, int32_t max_position, int32_t radius, int16_t* out) {

@@ -17,9 +17,10 @@
 //   dS' = P' (dP' - Delta_i) c, and the outputs contract over the loop rows, which sit in the accumulator
 //   registers: out^T += Y^T dS' (or P'), with Y^T read transposed from LDS -- the layout trick of the forward.
 // Score gradients without atomics.  Each role owns the tensor of its lane side (dQ role: d c2p, a row per query;
-// dK/dV role: d p2c, a row per key).  The table row delta(i - j) is monotone in the loop row with steps of 0 or 1, so
-// the entries a lane row can still receive form a window of at most 33 neighbours that slides one way as the loop
-// advances: a 64-entry ring per row in LDS takes the adds, and the entries the window has left behind are stored
+// dK/dV role: d p2c, a row per key).  The table row delta(i - j) is monotone in the loop row, so the entries a lane
+// row can still receive form a window that slides one way as the loop advances; the entry point refuses tables in
+// which 32 consecutive relative positions span more than 61 rows (steps of 0 or 1, the usual case, span at most 32):
+// a 64-entry ring per row in LDS takes the adds, and the entries the window has left behind are stored
 // once, in aligned groups of four (eight lanes per row, one 16- or 8-byte store each), and cleared.  The tensors have
 // the element type of q and arrive zeroed; entries no element maps to are written as zeros or not at all.  Results
 // do not depend on the order workgroups run in.
@@ -40,7 +41,9 @@ namespace {
 
 constexpr int kBwdThreads = 256;
 constexpr int kBwdStep = 32;    // loop-side rows per step
-constexpr int kRing = 64;       // score-gradient entries kept per lane-side row (the live window is at most 33 wide)
+constexpr int kRing = FDB_BWD_RING;  // score-gradient entries kept per lane-side row: the table rows of one 32-row step
+                                     // (at most lut_window + 1, which the entry point bounds) plus a partly stored group
+static_assert(kRing == 64 && FDB_BWD_MAX_WINDOW + 4 <= kRing, "ring slots are taken modulo 64");
 // Row stride of the ring in floats.  The lanes of a half-wave hit entry (delta0 -+ lane) of row `lane` (dQ role: +,
 // dK/dV role: -): with stride 65 resp. 67 that is bank 2 * lane, no two lanes alike.
 constexpr int ring_stride(bool dq) { return dq ? kRing + 1 : kRing + 3; }

@@ -32,6 +32,7 @@ constexpr float kLazyTau = 8.f;  // the running reference point of a row is move
 // elements are k = 16*step + 8*(l/32) + 0..7).
 struct Bf16Tr {
   static constexpr int SZ = 2;
+  static constexpr uint32_t NAN_WORD = 0x7FC07FC0u;  // a quiet NaN in every element of a 32-bit word
   using frag = bf16x8;
   using scratch_t = __bf16;
   static __device__ __forceinline__ frag zero() { return frag{0, 0, 0, 0, 0, 0, 0, 0}; }
@@ -63,6 +64,7 @@ struct Bf16Tr {
 
 struct F16Tr {
   static constexpr int SZ = 2;
+  static constexpr uint32_t NAN_WORD = 0x7E007E00u;
   using frag = f16x8;
   using scratch_t = _Float16;
   static __device__ __forceinline__ frag zero() { return frag{0, 0, 0, 0, 0, 0, 0, 0}; }
@@ -90,6 +92,7 @@ struct F16Tr {
 
 struct F32Tr {
   static constexpr int SZ = 4;
+  static constexpr uint32_t NAN_WORD = 0x7FC00000u;
   using frag = f32x8;
   using scratch_t = float;
   static __device__ __forceinline__ frag zero() { return frag{0, 0, 0, 0, 0, 0, 0, 0}; }
@@ -318,6 +321,21 @@ __device__ __forceinline__ void wait_vmcnt() {
   static_assert(N >= 0 && N < 64, "vmcnt has six bits");
   __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
   asm volatile("" ::: "memory");
+}
+
+// Padded fixed layout: the rows of `out` outside a batch row's real tokens, written by the workgroup whose tile index t
+// covers them in absolute terms (rows [128 t, 128 t + 128), two threads per row of ROW_BYTES): zeros, or `word` = the
+// element type's NaN pattern for a batch row the caller marked with a negative token count.
+template <int ROW_BYTES>
+__device__ __forceinline__ void fill_pad_rows(char* out_bh, int64_t row_stride_bytes, int t, int L, int tok0, int Lb,
+                                              uint32_t word, int tid) {
+  static_assert(ROW_BYTES % 32 == 0, "two threads per row, 16-byte stores");
+  const int row = t * 128 + (tid >> 1);
+  if (row >= L || (row >= tok0 && row < tok0 + Lb)) return;
+  char* dst = out_bh + (int64_t)row * row_stride_bytes + (tid & 1) * (ROW_BYTES / 2);
+  const u32x4 w = {word, word, word, word};
+#pragma unroll
+  for (int c = 0; c < ROW_BYTES / 32; ++c) *(u32x4*)(dst + 16 * c) = w;
 }
 
 // Number of direct loads (dma16 / dma16s) a wave issues per K/V tile of the far-only staging: the waits

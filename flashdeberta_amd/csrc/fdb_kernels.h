@@ -42,6 +42,8 @@ struct FdbKParams {
   char* ws;          // [ws_slots][ws_rows][H][D] elements of v's type (rows normalised over the keys seen), then
   int64_t ws_rows;   // [ws_slots][ws_rows][H] float log-sum-exps (-inf: no key seen); ws_rows = rows of the lse buffer
   int32_t causal;
+  int32_t fill_pad; // padded fixed layout, first launch of a call: write the rows of out outside the real tokens (zeros; NaN
+                    // for batch rows whose seq_len is negative)
   float scale_log2; // sm_scale * log2(e)
 };
 

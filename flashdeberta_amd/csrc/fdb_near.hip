@@ -105,7 +105,11 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
     b = xq / p.tiles_per_seq;
     m0 = (xq % p.tiles_per_seq) * FDB_BM;
     tok0 = p.seq_start ? min(max(p.seq_start[b], 0), p.L) : 0;
-    Lb = p.seq_len ? min(max(p.seq_len[b], 0), p.L - tok0) : p.L;
+    const int sl = p.seq_len ? p.seq_len[b] : p.L;  // negative: a batch row the caller could not express, NaN throughout
+    Lb = min(max(sl, 0), p.L - tok0);
+    if (p.fill_pad && blockIdx.y == 0)
+      fill_pad_rows<kRowBytes>(p.out + ((int64_t)b * p.o_sb + (int64_t)h * p.o_sh) * 2, p.o_st * 2, xq % p.tiles_per_seq, p.L, tok0, Lb,
+                               sl < 0 ? VT::NAN_WORD : 0u, tid);
     if (m0 >= Lb) return;
     qo = b * p.q_sb; ko = b * p.k_sb; vo = b * p.v_sb; oo = b * p.o_sb;
   }

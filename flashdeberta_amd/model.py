@@ -38,38 +38,35 @@ class _Memo:
     `extra` compares equal.  The tensors are held weakly."""
 
     def __init__(self):
-        self._refs, self._stamps, self._extra, self._value = (), (), None, None
+        self._state = ((), (), None, None)  # (weak references, stamps, extra, value): replaced as a whole, read once
 
     def get(self, tensors, extra=None):
-        if len(self._refs) != len(tensors) or extra != self._extra:
+        refs, stamps, old_extra, value = self._state
+        if len(refs) != len(tensors) or extra != old_extra:
             return None
-        for ref, stamp, t in zip(self._refs, self._stamps, tensors):
+        for ref, stamp, t in zip(refs, stamps, tensors):
             if ref() is not t or _stamp(t) != stamp:
                 return None
-        return self._value
+        return value
 
     def put(self, tensors, value, extra=None):
-        self._refs = tuple(weakref.ref(t) for t in tensors)
-        self._stamps = tuple(_stamp(t) for t in tensors)
-        self._extra, self._value = extra, value
+        self._state = (tuple(weakref.ref(t) for t in tensors), tuple(_stamp(t) for t in tensors), extra, value)
         return value
 
     def __reduce__(self):  # copies and pickles of a module start with nothing remembered
         return (_Memo, ())
 
 
-def _seq_bounds_of(attention_mask):
-    """(seq_start, seq_len, fill) of a mask; every layer of an encoder receives the same mask object, so
-    the reductions run once per forward instead of once per layer.  The result rides on the mask tensor
-    itself (no state outside it) and is dropped when the mask is written in place or re-seated."""
-    hit = attention_mask.__dict__.get("_fdb_bounds")
-    if hit is None or hit[0] != _stamp(attention_mask):
-        start, length, holes = seq_bounds(key_padding_mask(attention_mask))
-        # what the rows of the output start from: zero, or NaN for a row whose mask the kernels cannot honour
-        fill = torch.where(holes, float("nan"), 0.0).view(-1, 1, 1, 1)
-        hit = (_stamp(attention_mask), (start, length, fill))
-        attention_mask._fdb_bounds = hit
-    return hit[1]
+def _seq_bounds_of(attention_mask, memo):
+    """(seq_start, seq_len) of a mask.  Every layer of an encoder receives the same mask object, so the
+    reductions run once per forward instead of once per layer: `memo` (a _Memo that the layers of a patched
+    model share, see patch_model) holds the result for as long as the mask is the same object, unwritten and
+    in place.  Nothing is stored on the caller's tensor and nothing is process-global."""
+    hit = memo.get((attention_mask,))
+    if hit is None:
+        start, length, _ = seq_bounds(key_padding_mask(attention_mask))
+        hit = memo.put((attention_mask,), (start, length))
+    return hit
 
 
 class FlashDisentangledSelfAttention(DisentangledSelfAttention):
@@ -87,7 +84,7 @@ class FlashDisentangledSelfAttention(DisentangledSelfAttention):
     def __init__(self, config, fp8_qk=None):
         super().__init__(config)
         self.fp8_qk = bool(getattr(config, "fp8_qk", False)) if fp8_qk is None else bool(fp8_qk)
-        self._qkv_memo, self._pos_memo = _Memo(), _Memo()
+        self._qkv_memo, self._pos_memo, self._mask_memo = _Memo(), _Memo(), _Memo()
 
     def _fused_qkv(self):
         """Concatenated [3*H*D, hidden] weight and bias of the query, key and value projections."""
@@ -170,14 +167,12 @@ class FlashDisentangledSelfAttention(DisentangledSelfAttention):
         sm_scale = 1.0 / math.sqrt(D * scale_factor)
 
         seq_start = seq_len = None
-        out = None
         if attention_mask is not None:
-            seq_start, seq_len, fill = _seq_bounds_of(attention_mask)
-            # Padded rows stay zero.  The kernels take the real tokens of a row as one contiguous run; a row
-            # whose mask has a hole inside that run gets no tokens (seq_len 0) and NaN in every position, so
-            # the unsupported mask cannot pass for a result (the eager module honours arbitrary masks).
-            out = torch.empty((B, L, H, D), dtype=v.dtype, device=v.device)
-            out.copy_(fill.expand(B, L, H, D))  # one fill kernel per layer
+            # The kernels take the real tokens of a row as one contiguous run and write zeros into the padded
+            # rows themselves; a row whose mask has a hole inside that run carries seq_len -1 and comes back as
+            # NaN in every position, so the unsupported mask cannot pass for a result (the eager module honours
+            # arbitrary masks).
+            seq_start, seq_len = _seq_bounds_of(attention_mask, self._mask_memo)
 
         kw = {}
         if self.fp8_qk:
@@ -196,7 +191,7 @@ class FlashDisentangledSelfAttention(DisentangledSelfAttention):
             q, k, v, pos_key, pos_query, sm_scale=sm_scale,
             position_buckets=self.position_buckets if self.relative_attention else 0,
             max_relative_positions=self.max_relative_positions if self.relative_attention else 0,
-            seq_start=seq_start, seq_len=seq_len, out=out, **kw)
+            seq_start=seq_start, seq_len=seq_len, **kw)
         return (ctx.view(B, L, H * D), None)
 
 
@@ -255,15 +250,20 @@ def patch_model(model, attn_implementation="flash_attention_2", fp8_qk=False, sk
     if encoder is None:
         raise ValueError("no DebertaV2 encoder found in %s" % type(model).__name__)
     config = model.config
+    mask_memo = _Memo()  # the layers of one model see the same mask object: its bounds are derived once per forward
     for layer in encoder.layer:
         old = layer.attention.self
         if type(old) is cls:
+            if cls is FlashDisentangledSelfAttention:
+                old._mask_memo = mask_memo
             continue
         new = cls(config, fp8_qk=fp8_qk) if cls is FlashDisentangledSelfAttention else cls(config)
         new.load_state_dict(old.state_dict())
         p = next(old.parameters())
         new.to(device=p.device, dtype=p.dtype)
         new.train(old.training)
+        if cls is FlashDisentangledSelfAttention:
+            new._mask_memo = mask_memo
         layer.attention.self = new
     flash = cls is FlashDisentangledSelfAttention
     # The encoder-side shortcuts live in a subclass that differs from transformers' encoder in three methods

@@ -44,6 +44,15 @@ def delta_lut_host(position_buckets, max_relative_positions):
     return out, radius
 
 
+def delta_lut_window(position_buckets, max_relative_positions):
+    """The largest delta(r + 31) - delta(r) of the table: what the backward's score-gradient ring has to hold."""
+    w = lib.fdb_delta_lut_window(int(position_buckets), int(max_relative_positions))
+    if w < 0:
+        raise ValueError("unsupported relative-position config position_buckets=%d max_relative_positions=%d: %s"
+                         % (position_buckets, max_relative_positions, _lib.strerror(w)))
+    return w
+
+
 def delta_lut_device(position_buckets, max_relative_positions, device):
     key = (int(position_buckets), int(max_relative_positions), torch.device(device))
     hit = _lut_dev_cache.get(key)
@@ -81,7 +90,7 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
                                sm_scale=None, position_buckets=0, max_relative_positions=0, causal=False,
                                return_lse=False, seq_start=None, seq_len=None, q_scale=None, k_scale=None, pos_key_scale=None,
                                pos_query_scale=None, out=None, single_kernel=False, far_splits=0, near_splits=0, workspace=None,
-                               no_alloc=False, _launch_mask=0):
+                               no_alloc=False, _part=0):
     """Fused forward.  Layouts (strides are free except a unit stride on D):
          fixed length : q, k, v  [B, L, H, D]   -> out [B, L, H, D] (contiguous: a free view of [B, L, H*D])
          packed varlen: q, k, v  [T, H, D] + cu_seqlens int32 [B+1] (+ max_seqlen upper bound) -> out [T, H, D]
@@ -142,7 +151,7 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
                 cu_seqlens=cu_seqlens, max_seqlen=max_seqlen, sm_scale=sm_scale, position_buckets=position_buckets,
                 max_relative_positions=max_relative_positions, causal=causal, return_lse=return_lse,
                 seq_start=seq_start, seq_len=seq_len, out=out, far_splits=far_splits, near_splits=near_splits,
-                workspace=workspace, _launch_mask=_launch_mask)
+                workspace=workspace, _part=_part)
         dt = _lib.FDB_FP8_E4M3
     else:
         if q.dtype not in _DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
@@ -216,7 +225,6 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
     a.batch, a.heads, a.head_dim, a.max_seqlen, a.total_tokens = B, H, D, L, T
     a.dtype, a.causal, a.sm_scale, a.far_splits = dt, int(bool(causal)), float(sm_scale), int(far_splits)
     a.near_splits = int(near_splits)
-    a.launch_mask = int(_launch_mask)  # measurement only: 1 = far launch alone, 2 = near launch alone
     with torch.cuda.device(q.device):
         if no_alloc:
             check(lib.fdb_attn_fwd_noalloc(ctypes.byref(a), _stream_ptr(q.device)), "fdb_attn_fwd_noalloc")
@@ -232,7 +240,10 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
                 ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
                 keep.append(ws)
                 a.workspace, a.workspace_bytes = ws.data_ptr(), ws_bytes
-        check(lib.fdb_attn_fwd(ctypes.byref(a), _stream_ptr(q.device)), "fdb_attn_fwd")
+        if _part:  # measurement only (bench.py): 1 = the far launch alone, 2 = the near launch alone; `out` is then no result
+            check(lib.fdb_attn_fwd_part(ctypes.byref(a), int(_part), _stream_ptr(q.device)), "fdb_attn_fwd_part")
+        else:
+            check(lib.fdb_attn_fwd(ctypes.byref(a), _stream_ptr(q.device)), "fdb_attn_fwd")
     return (out, lse) if return_lse else out
 
 
@@ -263,6 +274,12 @@ def attention_bwd_kernels(q, k, v, dout, lse, *, out=None, delta=None, c2p=None,
     if scores:
         lut, radius = delta_lut_device(position_buckets, max_relative_positions, q.device)
         a.delta_lut, a.lut_radius, a.att_span = lut.data_ptr(), radius, span
+        a.lut_window = delta_lut_window(position_buckets, max_relative_positions)
+        if a.lut_window > _lib.FDB_BWD_MAX_WINDOW:
+            raise ValueError("backward: position_buckets=%d, max_relative_positions=%d map 32 consecutive relative positions onto "
+                             "%d table rows; the score-gradient window of the kernels holds %d (use the eager implementation "
+                             "for training with this configuration)"
+                             % (position_buckets, max_relative_positions, a.lut_window + 1, _lib.FDB_BWD_MAX_WINDOW + 1))
         st = scores[0].stride()
         for x in scores:
             if tuple(x.shape) != (B, L, H, 2 * span) or x.stride() != st or st[3] != 1 or x.dtype != q.dtype:
@@ -403,6 +420,9 @@ class _DisentangledAttention(torch.autograd.Function):
         kw = {n: kwargs[n] for n in ("sm_scale", "position_buckets", "max_relative_positions", "causal", "seq_start", "seq_len")
               if n in kwargs}
         dq, dk, dv, dpk, dpq = disentangled_attention_bwd(q, k, v, out, lse, dout, pk, pq, **kw)
+        # a position tensor handed in as [1, H, 2S, D] takes its gradient in that shape
+        dpk = dpk if dpk is None else dpk.reshape(pk.shape)
+        dpq = dpq if dpq is None else dpq.reshape(pq.shape)
         return None, dq, dk, dv, dpk, dpq
 
 
@@ -435,19 +455,19 @@ def disentangled_attention(q, k, v, pos_key=None, pos_query=None, **kwargs):
     return disentangled_attention_fwd(q, k, v, pos_key, pos_query, **kwargs)
 
 
-disentangled_attention_forward_only = disentangled_attention  # earlier name
-
 
 def flash_attention_with_disentangled(q, k, v, k_pos, q_pos, causal=False, sm_scale=None,
                                       position_buckets=0, max_relative_distance=0):
     """Same call shape as the reference op (flash_attention.py:1088-1091): q, k, v [B, H, L, D],
     returns [B, H, L, D].  k_pos / q_pos are K_r / Q_r [H, 2S, D] (see the module docstring).
-    As in the reference, sm_scale=None means 1/sqrt(D) (flash_attention.py:1042-1043)."""
+    As in the reference, sm_scale=None means 1/sqrt(D) (flash_attention.py:1042-1043), and the op is
+    differentiable like FlashAttentionDisentangled.apply (flash_attention.py:1032-1086): gradients reach
+    q, k, v, k_pos and q_pos."""
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(q.shape[-1])
-    o = disentangled_attention_fwd(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), k_pos, q_pos,
-                                   sm_scale=sm_scale, position_buckets=position_buckets,
-                                   max_relative_positions=max_relative_distance, causal=causal)
+    o = disentangled_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), k_pos, q_pos,
+                               sm_scale=sm_scale, position_buckets=position_buckets,
+                               max_relative_positions=max_relative_distance, causal=causal)
     return o.transpose(1, 2)
 
 
@@ -457,15 +477,16 @@ def flash_attention_with_disentangled_varlen(q, k, v, q_pos, k_pos, cu_seqlens_q
     """Same call shape as the reference op (flash_attention_varlen.py:485-511): q, k, v [T, H, D].
     Positional order follows the reference: the 4th argument feeds the content->position term
     (K_r), the 5th the position->content term (Q_r) (flash_attention_varlen.py:445,470).
-    Self-attention only: cu_seqlens_q must equal cu_seqlens_k."""
+    Self-attention only: cu_seqlens_q must equal cu_seqlens_k.  Forward-only like the reference's packed op:
+    under autograd it is a node whose backward raises (flash_attention_varlen.py:480-483)."""
     if cu_seqlens_q is not cu_seqlens_k and not torch.equal(cu_seqlens_q, cu_seqlens_k):
         raise ValueError("self-attention only: cu_seqlens_q and cu_seqlens_k must match")
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(q.shape[-1])
-    return disentangled_attention_fwd(q, k, v, q_pos, k_pos, cu_seqlens=cu_seqlens_q.to(torch.int32),
-                                      max_seqlen=max(int(max_seqlen_q), int(max_seqlen_k)), sm_scale=sm_scale,
-                                      position_buckets=position_buckets,
-                                      max_relative_positions=max_relative_distance, causal=causal)
+    return disentangled_attention(q, k, v, q_pos, k_pos, cu_seqlens=cu_seqlens_q.to(torch.int32),
+                                  max_seqlen=max(int(max_seqlen_q), int(max_seqlen_k)), sm_scale=sm_scale,
+                                  position_buckets=position_buckets,
+                                  max_relative_positions=max_relative_distance, causal=causal)
 
 
 def quantize_e4m3_per_head(x):

@@ -4,11 +4,10 @@ Counterpart of the reference's src/flashdeberta/padding.py (`_get_unpad_data` :7
 :113-166, `pad_input` :30-44).  The reference gathers the real tokens into a packed [T, H, D]
 tensor (with `.item()` host syncs) and scatters the result back.  Here the kernel reads the padded
 [B, L, H, D] layout in place, given each row's first real token and its count, so nothing is
-gathered, scattered or synchronised; the packed helpers remain for callers that already hold
-packed tensors.
+gathered, scattered or synchronised.  Callers that already hold packed [T, H, D] tensors pass
+cu_seqlens to the operator instead.
 """
 import torch
-import torch.nn.functional as F
 
 
 def key_padding_mask(attention_mask):
@@ -28,15 +27,15 @@ def key_padding_mask(attention_mask):
 def seq_bounds(mask2d):
     """[B, L] bool -> (seq_start int32 [B], seq_len int32 [B], holes bool [B]) on the mask's device, no
     host sync.  The kernels take the real tokens of a row as one contiguous run (left or right padding).
-    A row whose ones are not contiguous is flagged in `holes` and given seq_len 0, so that nothing is
-    computed from a mask the kernels cannot honour."""
+    A row whose ones are not contiguous is flagged in `holes` and given seq_len -1, the kernels' mark for
+    "write NaN": nothing is computed from a mask they cannot honour, and nothing passes for a result."""
     m = mask2d.to(torch.int32)
     L = m.shape[-1]
     count = m.sum(dim=-1, dtype=torch.int32)
     first = torch.argmax(m, dim=-1).to(torch.int32)  # first 1; 0 for an all-padding row
     last = (L - 1 - torch.argmax(m.flip(-1), dim=-1)).to(torch.int32)
     holes = (count > 0) & (last - first + 1 != count)
-    return first, torch.where(holes, torch.zeros_like(count), count), holes
+    return first, torch.where(holes, torch.full_like(count, -1), count), holes
 
 
 def assert_contiguous_mask(attention_mask):
@@ -46,25 +45,3 @@ def assert_contiguous_mask(attention_mask):
     if bool(holes.any()):
         raise ValueError("attention_mask rows %s have masked tokens between real ones; the fused attention takes "
                          "the real tokens of a row as one contiguous run" % holes.nonzero().flatten().tolist())
-
-
-def get_unpad_data(mask2d):
-    """(indices of real tokens in the flattened [B*L] batch, cu_seqlens int32 [B+1], longest length).
-    The longest length is returned as a 0-d tensor: turning it into a python int is the caller's
-    choice (it is the only step that would synchronise)."""
-    seqlens = mask2d.sum(dim=-1, dtype=torch.int32)
-    indices = torch.nonzero(mask2d.flatten(), as_tuple=False).flatten()
-    cu_seqlens = F.pad(torch.cumsum(seqlens, dim=0, dtype=torch.int32), (1, 0))
-    return indices, cu_seqlens, seqlens.max()
-
-
-def unpad_input(x, indices):
-    """x [B, L, ...] -> [T, ...] rows of the real tokens."""
-    return x.reshape(-1, *x.shape[2:]).index_select(0, indices)
-
-
-def pad_input(x, indices, batch, seqlen):
-    """x [T, ...] -> [B, L, ...] with zeros in the padded rows."""
-    out = torch.zeros((batch * seqlen,) + tuple(x.shape[1:]), dtype=x.dtype, device=x.device)
-    out.index_copy_(0, indices, x)
-    return out.view(batch, seqlen, *x.shape[1:])

@@ -37,7 +37,7 @@ extern "C" {
 #endif
 
 /* bumped whenever fdb_attn_args or the meaning of an entry point changes: a binding checks it next to the struct size */
-#define FDB_VERSION 6
+#define FDB_VERSION 7
 
 /* element types of q/k/pos_key/pos_query (v and out: see fdb_attn_args.dtype) */
 enum fdb_dtype {
@@ -70,7 +70,11 @@ enum fdb_status {
  *                                                      seq_len (padded batches) the real tokens of row b are
  *                                                      l in [seq_start[b], seq_start[b]+seq_len[b]), they
  *                                                      attend only to each other with positions counted
- *                                                      from seq_start[b]; other rows of `out` are not written
+ *                                                      from seq_start[b]; the other rows of `out` are written
+ *                                                      as zeros (what the eager module leaves in padded rows);
+ *                                                      a negative seq_len[b] marks a batch row whose mask the
+ *                                                      caller could not express as one run of tokens: all its
+ *                                                      rows of `out` are written as NaN
  *                  packed varlen (cu_seqlens != NULL): tok0_b = cu_seqlens[b], stride_b ignored,
  *                                                      0 <= l < cu_seqlens[b+1]-cu_seqlens[b]
  *   pos_key  (K_r): element (h, r, d) at base + h*pk_stride_h + r*pk_stride_r + d, 0 <= r < 2S
@@ -117,8 +121,6 @@ typedef struct fdb_attn_args {
   int32_t far_splits;      /* 0: the library decides; 1 .. FDB_MAX_FAR_SPLITS: workgroups that share the far keys of a query tile */
   int32_t near_splits;     /* the same for the near keys (those whose bucketed relative position varies)                  */
   float sm_scale;
-  int32_t launch_mask;     /* 0: the whole call.  Measurement only (the output of such a call is not a result): 1 = only the
-                              launch over the far keys, 2 = only the launch over the near keys (and its merge kernel)       */
 } fdb_attn_args;
 
 #define FDB_MAX_FAR_SPLITS 4
@@ -131,8 +133,20 @@ const char* fdb_strerror(int code);
 /* Host-only validation of an argument block (what fdb_attn_fwd checks before launching). */
 int fdb_attn_check(const fdb_attn_args* a);
 
-/* Enqueue the fused forward on `stream` (a hipStream_t). */
+/* Enqueue the fused forward on `stream` (a hipStream_t).
+ * A packed call (cu_seqlens) whose total_tokens exceed lut_radius + 63 always includes the launch over the far
+ * keys, because max_seqlen is the caller's word and the token count is the one bound the library can trust: for a
+ * batch of many short sequences that launch finds no far key tile and costs a few microseconds. */
 int fdb_attn_fwd(const fdb_attn_args* a, void* stream);
+
+/*
+ * Measurement hook, not a result: one of the launches fdb_attn_fwd makes for this argument block, alone, so that a
+ * profiler-free harness can time them one at a time.  part 1 = the launch over the far keys (those whose bucketed
+ * relative position is constant), part 2 = the launch over the near keys with its merge kernel.  What `out` and
+ * `lse` hold afterwards is a partial result.  FDB_ERR_UNSUPPORTED for calls that are a single kernel.  No
+ * counterpart in the reference.
+ */
+int fdb_attn_fwd_part(const fdb_attn_args* a, int32_t part, void* stream);
 
 /*
  * fdb_attn_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving
@@ -147,6 +161,8 @@ int fdb_attn_fwd(const fdb_attn_args* a, void* stream);
  * left and the call shares less when that is small (same result up to rounding).  Nothing in the scratch
  * has to start at zero (every word read was written earlier in the same call).  All calls on one GPU
  * share its scratch: calls that overlap in time on one GPU (two streams, two threads) race; serialise them.
+ * The first call on a device asks the runtime for the scratch's address (hipGetSymbolAddress): make that first
+ * call outside stream capture; every later call on the device is capture-safe.
  */
 #define FDB_NOALLOC_SCRATCH_BYTES (32 * 1024 * 1024)
 int fdb_attn_fwd_noalloc(const fdb_attn_args* a, void* stream);
@@ -171,7 +187,14 @@ int fdb_attn_fwd_noalloc(const fdb_attn_args* a, void* stream);
  * delta itself and leaves it in `delta`; with out == NULL it reads `delta` as given.
  * Rows outside [seq_start, seq_start + seq_len) are not written.  q, k, v, dout, dq, dk, dv: element type of
  * `dtype` (fp32 / bf16 / fp16), layout and strides as in fdb_attn_args.
+ * The score gradients of a row are collected in a sliding window of FDB_BWD_RING table rows, which holds the rows
+ * 32 consecutive relative positions map to plus one partly stored group: a table whose lut_window (the largest
+ * delta(r + 31) - delta(r)) exceeds FDB_BWD_MAX_WINDOW is refused with FDB_ERR_SPAN.  Every table with steps of
+ * 0 or 1 passes (window <= 31), so does every log-bucket table with max_position >= position_buckets; the
+ * reference scatters with atomics and takes any table (flash_attention.py:769-786).
  */
+#define FDB_BWD_RING 64
+#define FDB_BWD_MAX_WINDOW (FDB_BWD_RING - 4)
 typedef struct fdb_attn_bwd_args {
   const void* q;
   const void* k;
@@ -205,6 +228,7 @@ typedef struct fdb_attn_bwd_args {
   int32_t seqlen;
   int32_t att_span;
   int32_t lut_radius;
+  int32_t lut_window;      /* fdb_delta_lut_window(...) of the table behind delta_lut (with a position term) */
   int32_t dtype;           /* FDB_F32, FDB_BF16 or FDB_F16 */
   int32_t causal;
   float sm_scale;
@@ -249,6 +273,9 @@ int fdb_build_worklist(const int32_t* cu_seqlens, int32_t batch, int32_t total_t
  */
 int32_t fdb_delta_lut_radius(int32_t position_buckets, int32_t max_position);
 int fdb_delta_lut(int32_t position_buckets, int32_t max_position, int32_t radius, int16_t* out);
+/* Host: the largest delta(r + 31) - delta(r) over all r, i.e. how many table rows beyond the first the 32 loop
+ * rows of one backward step can reach (negative: FDB_ERR_LUT_ARGS).  What fdb_attn_bwd_args.lut_window takes. */
+int32_t fdb_delta_lut_window(int32_t position_buckets, int32_t max_position);
 
 /*
  * Per-head absmax quantisation to OCP e4m3: for each head h,

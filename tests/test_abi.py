@@ -33,7 +33,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_struct_mirror_and_version():
     assert lib.fdb_attn_args_size() == ctypes.sizeof(FdbAttnArgs)
-    assert lib.fdb_version() == _lib.FDB_VERSION == 6
+    assert lib.fdb_version() == _lib.FDB_VERSION == 7
     assert lib.fdb_tile_rows() == 128
 
 
@@ -298,18 +298,24 @@ def test_module_projection_memos():
     patch_model(hf, "eager")
     assert type(hf.encoder).__name__ == "DebertaV2Encoder"
 
-    # mask bounds: once per mask object and version
-    m = torch.tensor([[1, 1, 1, 0, 0], [0, 0, 1, 1, 1]])
-    s0, n0, f0 = _seq_bounds_of(m)
-    assert _seq_bounds_of(m)[0] is s0 and s0.tolist() == [0, 2] and n0.tolist() == [3, 3] and f0.flatten().tolist() == [0.0, 0.0]
+    # mask bounds: once per mask object and version, remembered by the memo the layers of a patched model share
+    from flashdeberta_amd.model import _Memo
+    memo = _Memo()
+    m = torch.tensor([[1, 1, 1, 0, 0], [0, 0, 1, 1, 1], [1, 0, 1, 1, 0]])
+    s0, n0 = _seq_bounds_of(m, memo)
+    assert _seq_bounds_of(m, memo)[0] is s0 and s0.tolist()[:2] == [0, 2] and n0.tolist() == [3, 3, -1]  # -1: a hole
     m[0, 3] = 1
-    s1, n1, _ = _seq_bounds_of(m)
-    assert s1 is not s0 and n1.tolist() == [4, 3]
-    assert _seq_bounds_of(m.clone())[0] is not s1  # the result rides on the mask object: nothing global
+    s1, n1 = _seq_bounds_of(m, memo)
+    assert s1 is not s0 and n1.tolist() == [4, 3, -1]
+    assert _seq_bounds_of(m.clone(), memo)[0] is not s1  # another mask object
+    assert not hasattr(m, "_fdb_bounds")                 # nothing rides on the caller's tensor
+    layers = patch_model(DebertaV2Model(DebertaV2Config(**kw))).encoder.layer
+    assert layers[0].attention.self._mask_memo is layers[1].attention.self._mask_memo
+    assert FlashDisentangledSelfAttention(DebertaV2Config(**kw))._mask_memo is not layers[0].attention.self._mask_memo
 
 
 def test_padding_helpers():
-    from flashdeberta_amd.padding import get_unpad_data, key_padding_mask, pad_input, seq_bounds, unpad_input
+    from flashdeberta_amd.padding import key_padding_mask, seq_bounds
 
     m = torch.tensor([[1, 1, 1, 0, 0], [0, 0, 1, 1, 1], [1, 1, 1, 1, 1]])
     ext = m[:, None, None, :] * m[:, None, :, None]
@@ -319,18 +325,15 @@ def test_padding_helpers():
     # masked tokens between real ones: flagged, and the row gets no tokens
     mh = torch.tensor([[1, 1, 0, 1, 1], [0, 1, 1, 1, 0], [0, 0, 0, 0, 0], [1, 0, 0, 0, 1]]).bool()
     s, n, holes = seq_bounds(mh)
-    assert holes.tolist() == [True, False, False, True] and n.tolist() == [0, 3, 0, 0] and s.tolist()[1] == 1
+    assert holes.tolist() == [True, False, False, True] and n.tolist() == [-1, 3, 0, -1] and s.tolist()[1] == 1
     from flashdeberta_amd.padding import assert_contiguous_mask
     assert_contiguous_mask(m)
     with pytest.raises(ValueError, match="rows \\[0, 3\\]"):
         assert_contiguous_mask(mh)
-    idx, cu, mx = get_unpad_data(m.bool())
-    # literal values: flattened positions of the ones of the three rows, their running counts, the longest row
-    assert idx.tolist() == [0, 1, 2, 7, 8, 9, 10, 11, 12, 13, 14] and cu.tolist() == [0, 3, 6, 11] and int(mx) == 5
+    # the oracle's unpad bookkeeping (what the reference's packed branch derives from a mask, padding.py:79-88),
+    # by literal values: flattened positions of the ones of the three rows, their running counts, the longest row
     ref_idx, ref_cu, ref_mx = O.unpad_data(m.numpy())
     assert ref_idx.tolist() == [0, 1, 2, 7, 8, 9, 10, 11, 12, 13, 14] and ref_cu.tolist() == [0, 3, 6, 11] and ref_mx == 5
-    x = torch.arange(15.0).view(3, 5, 1)
-    assert torch.equal(pad_input(unpad_input(x, idx), idx, 3, 5), x * m[:, :, None])
 
 
 def test_no_alloc_entry_point_refuses_what_does_not_fit():
@@ -383,14 +386,46 @@ def test_bench_contract_without_a_gpu():
     assert t is None or t > 2e8
 
 
-def test_delta_table_is_monotone_with_unit_steps():
-    """The backward keeps a sliding window of table rows per tensor row, which rests on delta(r + 1) - delta(r)
-    being 0 or 1 for every table the host builds."""
-    for pb, mr in [(256, 512), (32, 128), (0, 512), (0, 64), (8, 64), (16, 32), (256, 1024), (64, 256), (4, 16), (0, 15), (128, 4096)]:
+def _window_by_brute_force(lut):
+    """Largest delta(r + 31) - delta(r) over every r, from the table itself (constant beyond its ends)."""
+    x = np.concatenate([np.full(31, lut[0]), lut.astype(np.int64), np.full(31, lut[-1])])
+    return int((x[31:] - x[:-31]).max())
+
+
+def test_backward_window_of_every_accepted_table():
+    """The backward keeps a 64-entry sliding window of table rows per tensor row.  It holds the rows one 32-row
+    step reaches (delta(r + 31) - delta(r) + 1) plus a partly stored group of four, so fdb_attn_bwd refuses tables
+    whose window exceeds FDB_BWD_MAX_WINDOW = 60.  Sweep of every configuration the host accepts on a grid:
+    the table is monotone, fdb_delta_lut_window equals the brute-force figure, tables with unit steps have a
+    window of at most 31, every unbucketed table and every bucketed one with max_position >= position_buckets
+    fits, and some configurations below that do not (they are refused before anything is launched)."""
+    refused = accepted = 0
+    grid = [(pb, mr) for pb in (0, 4, 8, 16, 32, 64, 100, 128, 256, 512, 1024) for mr in
+            (3, 8, 15, 16, 24, 40, 64, 100, 128, 200, 256, 300, 512, 513, 600, 1024, 2048, 4096)]
+    for pb, mr in grid:
+        if lib.fdb_delta_lut_radius(pb, mr) < 1:
+            assert lib.fdb_delta_lut_window(pb, mr) == -9
+            continue
         lut, radius = ops.delta_lut_host(pb, mr)
         steps = np.diff(lut.astype(np.int64))
-        assert steps.min() >= 0 and steps.max() <= 1, (pb, mr)
+        assert steps.min() >= 0, (pb, mr)
         assert lut[0] >= 0 and lut[-1] <= 2 * ops.att_span(pb, mr) - 1
+        w = ops.delta_lut_window(pb, mr)
+        assert w == _window_by_brute_force(lut), (pb, mr)
+        if steps.max() <= 1:
+            assert w <= 31, (pb, mr)
+        if pb == 0 or mr >= 2 * pb:
+            assert steps.max() <= 1, (pb, mr)
+        if pb == 0 or mr >= pb:   # steps of 2 occur up to max_position ~ 1.36 position_buckets; the window still fits
+            assert w <= _lib.FDB_BWD_MAX_WINDOW, (pb, mr)
+        if w > _lib.FDB_BWD_MAX_WINDOW:
+            refused += 1
+        else:
+            accepted += 1
+    assert refused > 0 and accepted > 100
+    # the two configurations a review found: worst windows 67 and 192 by its count, i.e. beyond the 60 the ring holds
+    assert ops.delta_lut_window(256, 200) > _lib.FDB_BWD_MAX_WINDOW and ops.delta_lut_window(512, 300) > _lib.FDB_BWD_MAX_WINDOW
+    assert ops.delta_lut_window(256, 512) <= 31
 
 
 def _header_struct_fields(name):
@@ -441,6 +476,7 @@ def _good_bwd_args():
     a.bias_stride_b, a.bias_stride_t, a.bias_stride_h = 512 * 512, 512, 2 * 512 * 512
     a.batch, a.heads, a.head_dim, a.seqlen = 2, 12, 64, 512
     a.att_span, a.lut_radius, a.dtype, a.sm_scale = 256, 512, _lib.FDB_BF16, 0.0721
+    a.lut_window = 24
     return a
 
 
@@ -462,3 +498,5 @@ def test_backward_argument_validation_codes():
     a = _good_bwd_args(); a.seqlen, a.bias_stride_t = 1 << 20, 1 << 12; assert call(a) == -5  # 32-bit offsets
     a = _good_bwd_args(); a.delta_lut = None; assert call(a) == -6
     a = _good_bwd_args(); a.lut_radius = 0; assert call(a) == -6
+    a = _good_bwd_args(); a.lut_window = 61; assert call(a) == -6           # more table rows per step than the ring holds
+    a = _good_bwd_args(); a.lut_window = -1; assert call(a) == -6

@@ -86,8 +86,6 @@ CASES = [
 @pytest.mark.parametrize("scale", [0.02, 1.0], ids=["n002", "unit"])
 def test_operator_matches_oracle(case, dtype, scale):
     B, L, H, D, pb, mr, c2p, p2c = case
-    if scale == 0.02 and D != 64:
-        pytest.skip("small-scale inputs only at the model's head_dim")
     q, k, v, pk, pq = _inputs(B, L, H, D, pb, mr, dtype, 1000 + L, scale, c2p, p2c)
     ref, ref_lse = _oracle_blhd(q, k, v, pk, pq, pb, mr, return_lse=True)
     out, lse = ops.disentangled_attention_fwd(_dev(q), _dev(k), _dev(v), _dev(pk), _dev(pq), position_buckets=pb,
@@ -358,6 +356,89 @@ def test_delta_indices_bit_exact(pb, mr, L, term):
     assert (got == want[i - j + L]).all()
 
 
+def _digit_run(term, dtype, D, L, pb, mr, layout, n_heads_per_call=3, **kw):
+    """delta(i, j) as the attention kernels of `dtype` use it, for every (i, j) of one sequence of length L laid out
+    as `layout` says.  16-bit types cannot carry delta itself (bf16 holds integers up to 256 only), so delta travels
+    as three base-8 digits, one per head: the position table of head h holds digit_h(row) in channel 0, the other
+    factor of the term holds 4 there, sm_scale is 1/8, so a score is digit / 2 exactly; probabilities are read
+    through a one-hot V, 64 keys (head_dim of them) per call, and digit = 2 * (log P_ij + lse_i) to within 0.02."""
+    S = ops.att_span(pb, mr)
+    rows = torch.arange(2 * S)
+    table = torch.zeros(3, 2 * S, D)
+    for h in range(3):
+        table[h, :, 0] = (rows >> (3 * h)) & 7
+    four = torch.zeros(L, 3, D)
+    four[..., 0] = 4.0
+    zero = torch.zeros(L, 3, D)
+    q1, k1 = (four, zero) if term == "c2p" else (zero, four)
+    table = table.to(dtype).cuda()
+
+    def lay(x):  # one sequence [L, 3, D] -> the call's layout; returns (tensor, where the sequence sits)
+        x = x.to(dtype)
+        if layout == "packed":      # a second sequence in front of it and a third behind
+            t = torch.cat([torch.zeros(200, 3, D, dtype=dtype), x, torch.zeros(77, 3, D, dtype=dtype)])
+            return t.cuda(), slice(200, 200 + L)
+        if layout == "left":        # batch row 1 of two, padded on the left
+            t = torch.zeros(2, L + 100, 3, D, dtype=dtype)
+            t[1, 100:] = x
+            t[0, :L] = x
+            return t.cuda(), (1, slice(100, 100 + L))
+        return x[None].cuda(), (0, slice(0, L))
+
+    q, where = lay(q1)
+    k, _ = lay(k1)
+    call = dict(kw, position_buckets=pb, max_relative_positions=mr, sm_scale=0.125, return_lse=True)
+    if layout == "packed":
+        call.update(cu_seqlens=torch.tensor([0, 200, 200 + L, 277 + L], dtype=torch.int32).cuda(), max_seqlen=L)
+    if layout == "left":
+        call.update(seq_start=torch.tensor([0, 100], dtype=torch.int32).cuda(), seq_len=torch.tensor([L, L], dtype=torch.int32).cuda())
+    got = np.zeros((L, L), dtype=np.int64)
+    for j0 in range(0, L, D):
+        n = min(D, L - j0)
+        v1 = torch.zeros(L, 3, D)
+        v1[j0:j0 + n, :, :n] = torch.eye(n)[:, None, :]
+        v, _ = lay(v1)
+        out, lse = ops.disentangled_attention_fwd(q, k, v, table, table, **call)  # both terms compiled in; one of them is zero
+        if layout == "packed":
+            o, l = out[where], lse[where]
+        else:
+            o, l = out[where[0], where[1]], lse.view(out.shape[0], out.shape[1], 3)[where[0], where[1]]
+        p = o[:, :, :n].double().cpu().numpy()                       # [L, 3, n]
+        x = 2.0 * (np.log(p) + l.double().cpu().numpy()[:, :, None])
+        d = np.rint(x)
+        assert np.abs(x - d).max() < 0.1, "digit off the grid by %.3f" % np.abs(x - d).max()
+        d = d.astype(np.int64)
+        got[:, j0:j0 + n] = d[:, 0] + 8 * d[:, 1] + 64 * d[:, 2]
+    return got
+
+
+@pytest.mark.parametrize("variant", ["plain", "packed", "left", "shared", "d32", "short_table"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("term", ["c2p", "p2c"])
+def test_delta_indices_bit_exact_on_the_16_bit_kernels(term, dtype, variant):
+    """The bucketed relative position of every (i, j) as the far-only launch, the near kernel (its ring slots,
+    clamped table rows, block picks and rotations) and the head_dim-32 ring mode use it, recovered exactly:
+    L = 1300 with 256 buckets over 512 positions has far tiles on both sides, both zone edges and the linear,
+    logarithmic and saturated parts of the table.  Variants: the plain fixed layout, a packed batch, a batch
+    padded on the left, far keys shared by three and near steps by two workgroups, head_dim 32, and a short
+    table (32 buckets over 64 positions, L = 300) whose zones all fall inside one query tile."""
+    D, L, pb, mr, layout, kw = 64, 1300, 256, 512, "plain", {}
+    if variant in ("packed", "left"):
+        layout = variant
+    if variant == "shared":
+        kw = dict(far_splits=3, near_splits=2)
+    if variant == "d32":
+        D = 32
+    if variant == "short_table":
+        L, pb, mr = 300, 32, 64
+    got = _digit_run(term, dtype, D, L, pb, mr, layout, **kw)
+    want = O.delta_table(pb, mr, L)  # index r + L
+    i, j = np.meshgrid(np.arange(L), np.arange(L), indexing="ij")
+    bad = np.argwhere(got != want[i - j + L])
+    assert len(bad) == 0, "%d of %d indices differ, first at (i, j) = %s: kernel %d, table %d" % (
+        len(bad), L * L, tuple(bad[0]), got[tuple(bad[0])], want[bad[0][0] - bad[0][1] + L])
+
+
 # ---- packed varlen and padded batches ------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_varlen_matches_per_sequence_oracle(dtype):
@@ -438,7 +519,7 @@ def test_padded_batch_matches_packed(side):
     lens = [200, 77, 130]
     q, k, v, pk, pq = _inputs(B, L, H, D, pb, mr, torch.bfloat16, 21, 1.0)
     start = [0, 0, 0] if side == "right" else [L - n for n in lens]
-    out = torch.zeros(B, L, H, D, dtype=torch.bfloat16, device="cuda")
+    out = torch.full((B, L, H, D), 7.0, dtype=torch.bfloat16, device="cuda")  # the kernels write the padded rows too: zeros
     ops.disentangled_attention_fwd(q.cuda(), k.cuda(), v.cuda(), pk.cuda(), pq.cuda(), position_buckets=pb,
                                    max_relative_positions=mr, out=out,
                                    seq_start=torch.tensor(start, dtype=torch.int32, device="cuda"),
@@ -455,7 +536,7 @@ def test_padded_batch_matches_packed(side):
 @pytest.mark.parametrize("near", [1, 2])
 def test_empty_rows_and_empty_sequences(near):
     """A padded batch with a row of no real tokens and a packed batch with an empty sequence in the middle:
-    nothing is written for them, the other sequences are unaffected (also through the merge kernel)."""
+    the padded rows come back as zeros, the other sequences are unaffected (also through the merge kernel)."""
     pb, mr, H, D = 32, 64, 2, 64
     lens = [300, 0, 77]
     q, k, v, pk, pq = _inputs(3, 300, H, D, pb, mr, torch.bfloat16, 41, 1.0)
@@ -463,7 +544,7 @@ def test_empty_rows_and_empty_sequences(near):
     out = torch.full((3, 300, H, D), 7.0, dtype=torch.bfloat16, device="cuda")
     ops.disentangled_attention_fwd(_dev(q), _dev(k), _dev(v), _dev(pk), _dev(pq), out=out,
                                    seq_len=torch.tensor(lens, dtype=torch.int32).cuda(), **kw)
-    assert (out[1] == 7).all() and (out[2, 77:] == 7).all()
+    assert (out[1] == 0).all() and (out[2, 77:] == 0).all()
     cu = torch.tensor([0, 300, 300, 377], dtype=torch.int32)
     packed = torch.cat([q[0], q[2, :77]]), torch.cat([k[0], k[2, :77]]), torch.cat([v[0], v[2, :77]])
     outp = ops.disentangled_attention_fwd(*[_dev(x) for x in packed], _dev(pk), _dev(pq), cu_seqlens=cu.cuda(),
@@ -543,6 +624,14 @@ def test_fp8_attention(L, pb, mr, single):
                                          pos_query_scale=pqs, single_kernel=single)
     ref_dq = _oracle_blhd(dq(q8, qs), dq(k8, ks), v, dq(pk8, pks).transpose(0, 1), dq(pq8, pqs).transpose(0, 1), pb, mr)
     _check(out, ref_dq, TOL[torch.bfloat16], "unit scale vs de-quantised oracle")
+    # ... and against the UNQUANTISED oracle where the stated bound means something (on the 0.02-scale inputs above
+    # 6e-2 absolute is vacuous): unit-scale inputs, outputs up to 0.26.  The stated bound, 6e-2 max-abs, holds with
+    # room (measured 1.9e-2 at L = 1100); relative to the largest reference entry the error of e4m3 operands (three
+    # mantissa bits on every factor of three score terms) is 7.3 %, held here to 10 %.
+    ref = _oracle_blhd(q, k, v, pk, pq, pb, mr)
+    err = np.abs(out.float().cpu().numpy() - ref).max()
+    assert err <= FP8_TOL, "unit scale vs unquantised oracle: max-abs %.3e" % err
+    assert err <= 0.10 * np.abs(ref).max(), "unit scale vs unquantised oracle: %.3e of max|ref| %.3e" % (err, np.abs(ref).max())
 
 
 def test_fp8_full_length_one_head():
@@ -915,6 +1004,15 @@ def test_module_mask_with_holes_and_backward():
     holed[2, 7] = 0
     out = att(x, holed, rel_embeddings=rel)[0]
     assert torch.isnan(out[2]).all() and torch.equal(out[:2], good[:2]) and not torch.isnan(good).any()
+    assert (good[1, 30:] == 0).all()  # padded rows: zeros, written by the kernels themselves
+    # the same at the operator: a negative seq_len marks the row, fp32 and the one-kernel path included
+    for dtype, D in ((torch.float32, 128), (torch.float16, 32), (torch.bfloat16, 64)):
+        q, k, v, pk, pq = [t.cuda() for t in _inputs(3, 150, 2, D, 32, 64, dtype, 77, 1.0)]
+        sl = torch.tensor([150, -1, 60], dtype=torch.int32).cuda()
+        o = ops.disentangled_attention_fwd(q, k, v, pk, pq, position_buckets=32, max_relative_positions=64, seq_len=sl,
+                                           out=torch.full_like(v, 3.0))
+        assert torch.isnan(o[1]).all() and (o[2, 60:] == 0).all() and not torch.isnan(o[0]).any() and not torch.isnan(o[2]).any()
+        _check(o[2:, :60], _oracle_blhd(*[t.cpu() for t in (q[2:, :60], k[2:, :60], v[2:, :60], pk, pq)], 32, 64), TOL[dtype])
     # FP8 operands have no backward: under autograd the forward runs, the backward raises instead of returning nothing
     att8 = FlashDisentangledSelfAttention(Cfg(), fp8_qk=True).eval().cuda().to(torch.bfloat16)
     att8.load_state_dict(att.state_dict())
@@ -1063,6 +1161,101 @@ def test_backward_is_reproducible_and_takes_a_given_delta(dtype):
     for n, a, b in zip(("dq", "dk", "dv", "dK_r", "dQ_r"), first, given):
         scale = a.float().abs().max().item()
         assert (a.float() - b.float()).abs().max().item() <= (1e-5 if dtype == torch.float32 else 2e-2) * scale, n
+
+
+def test_backward_refuses_tables_its_window_cannot_hold():
+    """position_buckets 256 over 200 positions maps 32 consecutive relative positions onto up to 68 table rows;
+    the score-gradient window of the backward holds 61: the call is refused before anything is launched (the
+    forward takes the table as it is)."""
+    B, L, H, D, pb, mr = 1, 300, 1, 64, 256, 200
+    q, k, v, pk, pq = [x.cuda() for x in _inputs(B, L, H, D, pb, mr, torch.float32, 4300, 1.0, True, True)]
+    out, lse = ops.disentangled_attention_fwd(q, k, v, pk, pq, return_lse=True, position_buckets=pb, max_relative_positions=mr)
+    _check(out, _oracle_blhd(*[x.cpu() for x in (q, k, v, pk, pq)], pb, mr), TOL[torch.float32], "forward with a wide-step table")
+    with pytest.raises(ValueError, match="score-gradient window"):
+        ops.disentangled_attention_bwd(q, k, v, out, lse, torch.ones_like(out), pk, pq, position_buckets=pb, max_relative_positions=mr)
+    # a table with steps of two that still fits (256 buckets over 256 positions: window 44)
+    pb, mr = 256, 256
+    assert 31 < ops.delta_lut_window(pb, mr) <= 60
+    q, k, v, pk, pq = _inputs(B, L, H, D, pb, mr, torch.float32, 4301, 1.0, True, True)
+    dout = torch.randn(B, L, H, D, generator=torch.Generator().manual_seed(4302))
+    t = lambda x: _np(x).transpose(0, 2, 1, 3)
+    ref = O.disentangled_attention_backward(t(q), t(k), t(v), t(dout), _np(pk), _np(pq), pb, mr)
+    leaves = [x.cuda().requires_grad_(True) for x in (q, k, v, pk, pq)]
+    ops.disentangled_attention(*leaves, position_buckets=pb, max_relative_positions=mr).backward(dout.cuda())
+    for n, leaf, r in zip(("dq", "dk", "dv", "dK_r", "dQ_r"), leaves, ref):
+        r = r.transpose(0, 2, 1, 3) if r.ndim == 4 else r
+        err = np.abs(leaf.grad.cpu().numpy() - r).max()
+        assert err <= 2e-4 * max(np.abs(r).max(), 1e-3), "%s: err %.3e" % (n, err)
+
+
+def test_reference_shaped_operators_under_autograd():
+    """flash_attention_with_disentangled takes [B, H, L, D] like the reference's op and is differentiable like it
+    (flash_attention.py:1066-1086): all five gradients against the oracle, one position tensor handed in as
+    [1, H, 2S, D].  The packed operator is forward-only like the reference's (flash_attention_varlen.py:480-483):
+    its backward raises instead of dropping the gradients."""
+    B, L, H, D, pb, mr = 2, 200, 2, 64, 32, 64
+    q, k, v, pk, pq = _inputs(B, L, H, D, pb, mr, torch.float32, 4400, 1.0)
+    dout = torch.randn(B, L, H, D, generator=torch.Generator().manual_seed(4401))
+    t = lambda x: _np(x).transpose(0, 2, 1, 3)
+    c = 1.0 / np.sqrt(3 * D)  # the module's scale with both terms, which is the oracle's (the op's own default is 1/sqrt(D))
+    ref = O.disentangled_attention_backward(t(q), t(k), t(v), t(dout), _np(pk), _np(pq), pb, mr)
+    bh = lambda x: x.cuda().permute(0, 2, 1, 3).contiguous().requires_grad_(True)
+    leaves = [bh(q), bh(k), bh(v), pk.cuda()[None].requires_grad_(True), pq.cuda().requires_grad_(True)]
+    out = ops.flash_attention_with_disentangled(*leaves, False, c, pb, mr)
+    assert out.shape == (B, H, L, D) and out.grad_fn is not None
+    _check(out.detach().permute(0, 2, 1, 3), _oracle_blhd(q, k, v, pk, pq, pb, mr), TOL[torch.float32])
+    out.backward(dout.cuda().permute(0, 2, 1, 3))
+    assert leaves[3].grad.shape == (1, H, 2 * pb, D)
+    for n, leaf, r in zip(("dq", "dk", "dv", "dK_r", "dQ_r"), leaves, ref):
+        got = leaf.grad.cpu().numpy().reshape(r.shape)
+        err = np.abs(got - r).max()
+        assert err <= 2e-4 * max(np.abs(r).max(), 1e-3), "%s: err %.3e, ref max %.3e" % (n, err, np.abs(r).max())
+    # packed: a node whose backward raises
+    lens = [120, 80]
+    cu = torch.tensor([0, 120, 200], dtype=torch.int32).cuda()
+    qp = q[0].cuda().requires_grad_(True)
+    outp = ops.flash_attention_with_disentangled_varlen(qp, k[0].cuda(), v[0].cuda(), pk.cuda(), pq.cuda(), cu, cu, 120, 120,
+                                                        False, c, pb, mr)
+    assert outp.grad_fn is not None
+    t0 = 0
+    for n in lens:
+        sl = slice(t0, t0 + n)
+        _check(outp.detach()[None, sl], _oracle_blhd(q[:1, sl], k[:1, sl], v[:1, sl], pk, pq, pb, mr), TOL[torch.float32])
+        t0 += n
+    with pytest.raises(RuntimeError, match="forward-only"):
+        outp.sum().backward()
+
+
+def test_backward_at_the_benchmark_length():
+    """The backward at the sizes its figures are quoted on.  B = 1, L = 4096 with twelve heads: two of them against
+    the oracle's gradients (bf16); sixteen heads: one of them; B = 8 x L = 4096 x 12 heads: two runs give the same
+    bits (no atomics, nothing depends on the order workgroups run in)."""
+    L, D, pb, mr = 4096, 64, 256, 512
+    t = lambda x: _np(x).transpose(0, 2, 1, 3)
+    for H, heads in ((12, (0, 7)), (16, (13,))):
+        q, k, v, pk, pq = _inputs(1, L, H, D, pb, mr, torch.bfloat16, 4500 + H, 1.0)
+        dout = torch.randn(1, L, H, D, generator=torch.Generator().manual_seed(4501 + H)).to(torch.bfloat16)
+        leaves = [x.cuda().requires_grad_(True) for x in (q, k, v, pk, pq)]
+        ops.disentangled_attention(*leaves, position_buckets=pb, max_relative_positions=mr).backward(dout.cuda())
+        for h in heads:
+            hs = slice(h, h + 1)
+            ref = O.disentangled_attention_backward(t(q[:, :, hs]), t(k[:, :, hs]), t(v[:, :, hs]), t(dout[:, :, hs]), _np(pk[hs]),
+                                                    _np(pq[hs]), pb, mr)
+            got = [leaves[0].grad[:, :, hs], leaves[1].grad[:, :, hs], leaves[2].grad[:, :, hs], leaves[3].grad[hs], leaves[4].grad[hs]]
+            for n, g_, r in zip(("dq", "dk", "dv", "dK_r", "dQ_r"), got, ref):
+                r = r.transpose(0, 2, 1, 3) if r.ndim == 4 else r
+                err = np.abs(g_.float().cpu().numpy() - r).max()
+                assert err <= 3e-2 * max(np.abs(r).max(), 1e-3), "H=%d head %d %s: err %.3e, ref max %.3e" % (H, h, n, err, np.abs(r).max())
+        del leaves
+    B, H = 8, 12
+    g = torch.Generator(device="cuda").manual_seed(4600)
+    rnd = lambda *s: (torch.randn(*s, device="cuda", generator=g) * 0.5).to(torch.bfloat16)
+    q, k, v, dout = [rnd(B, L, H, D) for _ in range(4)]
+    pk, pq = rnd(H, 2 * pb, D), rnd(H, 2 * pb, D)
+    out, lse = ops.disentangled_attention_fwd(q, k, v, pk, pq, return_lse=True, position_buckets=pb, max_relative_positions=mr)
+    runs = [ops.disentangled_attention_bwd(q, k, v, out, lse, dout, pk, pq, position_buckets=pb, max_relative_positions=mr) for _ in range(2)]
+    for n, a, b in zip(("dq", "dk", "dv", "dK_r", "dQ_r"), *runs):
+        assert not torch.isnan(a).any() and torch.equal(a, b), n
 
 
 def test_backward_refuses_an_odd_span():
