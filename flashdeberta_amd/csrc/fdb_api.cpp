@@ -89,6 +89,11 @@ int64_t query_tiles(const fdb_attn_args* a) {
                        : (int64_t)a->batch * ((a->max_seqlen + FDB_BM - 1) / FDB_BM);
 }
 
+// The far / near pair of launches exists for the 16-bit types at head_dim 32 / 64 and for e4m3 operands at head_dim 64;
+// its near launch walks 32-key steps (and can share them among workgroups) at head_dim 64.
+bool pair_supported(int dtype, int head_dim) { return fdb_near_supported(dtype, head_dim) || fdb_fp8_pair_supported(dtype, head_dim); }
+bool steps32_supported(int dtype, int head_dim) { return fdb_near32_supported(dtype, head_dim) || fdb_fp8_pair_supported(dtype, head_dim); }
+
 // Does the call take the far / near pair of launches with a far launch in it?
 // A packed call's max_seqlen is the caller's word; the one bound the library can trust there is the
 // token count (no sequence is longer), so an under-estimate cannot make the far keys disappear: a far
@@ -96,7 +101,7 @@ int64_t query_tiles(const fdb_attn_args* a) {
 bool has_far_launch(const fdb_attn_args* a) {
   const int32_t radius = a->lut_radius > 0 ? a->lut_radius : 1;
   const int32_t longest = a->cu_seqlens ? a->total_tokens : a->max_seqlen;
-  return (a->pos_key || a->pos_query) && a->lse && fdb_near_supported(a->dtype, a->head_dim) &&
+  return (a->pos_key || a->pos_query) && a->lse && pair_supported(a->dtype, a->head_dim) &&
          longest > radius + FDB_BN - 1;
 }
 
@@ -106,7 +111,7 @@ bool has_far_launch(const fdb_attn_args* a) {
 // tiles on 768 slots gain 9 % of the whole call from two shares; shares that need a second round of
 // workgroups, e.g. three for 512 query tiles, gain nothing.)
 int far_parts_wanted(const fdb_attn_args* a) {
-  if (!has_far_launch(a) || !fdb_near32_supported(a->dtype, a->head_dim)) return 1;
+  if (!has_far_launch(a) || !steps32_supported(a->dtype, a->head_dim)) return 1;
   if (a->far_splits > 0) return a->far_splits;
   // A packed batch has its lengths on the device: the host goes by the mean length (the kernel divides each query
   // tile's own far tiles among the shares, whatever they are), and only shares when that mean leaves far tiles at all.
@@ -133,7 +138,7 @@ int far_parts_wanted(const fdb_attn_args* a) {
 // long as the query tiles alone fill at most 70 % of the slots (288 to 352 tiles: 5 to 8 % of the call;
 // 384: between +2 and -4 %).
 int near_parts_wanted(const fdb_attn_args* a) {
-  if (!(a->pos_key || a->pos_query) || !a->lse || !fdb_near32_supported(a->dtype, a->head_dim)) return 1;
+  if (!(a->pos_key || a->pos_query) || !a->lse || !steps32_supported(a->dtype, a->head_dim)) return 1;
   if (a->near_splits > 0) return a->near_splits;
   if (a->cu_seqlens) return 1;
   const int64_t wgs = query_tiles(a) * a->heads, slots = 2 * (int64_t)cu_count();
@@ -200,7 +205,7 @@ int check_noalloc(const fdb_attn_args* a) {
   const int rc = fdb_attn_check(&b);
   if (rc != FDB_OK) return rc;
   int64_t need = 0;
-  if (!b.lse && (b.pos_key || b.pos_query) && fdb_near_supported(b.dtype, b.head_dim)) need += align256(lse_rows(&b) * b.heads * 4);
+  if (!b.lse && (b.pos_key || b.pos_query) && pair_supported(b.dtype, b.head_dim)) need += align256(lse_rows(&b) * b.heads * 4);
   if (b.cu_seqlens) need += align256(fdb_worklist_ints(b.total_tokens, b.batch) * 4);
   return need > FDB_NOALLOC_SCRATCH_BYTES ? FDB_ERR_SCRATCH : FDB_OK;
 }
@@ -333,7 +338,8 @@ int attn_fwd_impl(const fdb_attn_args* a, int launch_mask, void* stream) {
   // Split path: the far tiles in a far-only run of the kernel (three workgroups per CU), the near
   // tiles in a second launch, which merges the two.  It needs the log-sum-exp buffer as the
   // hand-over between the two launches.
-  if ((a->pos_key || a->pos_query) && a->lse && fdb_near_supported(a->dtype, a->head_dim)) {
+  if ((a->pos_key || a->pos_query) && a->lse && pair_supported(a->dtype, a->head_dim)) {
+    const bool fp8 = fdb_fp8_pair_supported(a->dtype, a->head_dim);
     const bool need_far = has_far_launch(a);  // otherwise no tile of any query tile is far
     // as many workgroups per query tile as wanted and as the workspace holds partial results for
     p.far_parts = need_far ? far_parts_wanted(a) : 1;
@@ -345,17 +351,18 @@ int attn_fwd_impl(const fdb_attn_args* a, int launch_mask, void* stream) {
     p.ws = (char*)a->workspace;
     p.ws_rows = lse_rows(a);
     if (need_far && launch_mask != 2) {
-      const int rc_far = fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, FDB_MODE_FAR_ONLY, stream);
+      const int rc_far = fp8 ? fdb_launch_far8(p, (int)grid_x, stream)
+                             : fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, FDB_MODE_FAR_ONLY, stream);
       if (rc_far != 0) return rc_far;
       p.fill_pad = 0;
     }
     if (launch_mask == 1) return FDB_OK;
     p.far_done = need_far ? 1 : 0;
     // head_dim 64: the near kernel (32-key steps, two workgroups per CU); head_dim 32: the fused kernel's ring mode
-    if (fdb_near32_supported(a->dtype, a->head_dim)) {
-      const int rc_near = fdb_launch_near32(p, a->dtype, (int)grid_x, stream);
+    if (steps32_supported(a->dtype, a->head_dim)) {
+      const int rc_near = fp8 ? fdb_launch_near8(p, (int)grid_x, stream) : fdb_launch_near32(p, a->dtype, (int)grid_x, stream);
       if (rc_near != 0 || p.near_parts <= 1) return rc_near;
-      return fdb_launch_merge(p, a->dtype, stream);
+      return fdb_launch_merge(p, fp8 ? (int)FDB_BF16 : a->dtype, stream);  // partial results have v's element type
     }
     return fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, FDB_MODE_NEAR_RING, stream);
   }
@@ -384,7 +391,7 @@ int fdb_attn_fwd_noalloc(const fdb_attn_args* a, void* stream) {
   // [log-sum-exp hand-over][work-list][partial results], each part 256-byte aligned
   int64_t off = 0;
   const bool has_pos = b.pos_key || b.pos_query;
-  if (!b.lse && has_pos && fdb_near_supported(b.dtype, b.head_dim)) {
+  if (!b.lse && has_pos && pair_supported(b.dtype, b.head_dim)) {
     b.lse = (float*)(base + off);
     off += align256(lse_rows(&b) * b.heads * 4);
   }

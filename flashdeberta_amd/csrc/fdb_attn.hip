@@ -217,84 +217,6 @@ __device__ __forceinline__ void softmax_pv_pre(f32x16 (&sacc)[2], f32x16 (&o_acc
   }
 }
 
-// The same without a row maximum on the common path.  The probabilities of the tile are formed
-// against the row's current reference point straight away; their sum bounds their maximum, so a
-// row whose half-sum stays under 2^kLazyTau needs no new reference point (the same guarantee the
-// maximum gives above).  Only when a row fails that test, overflows, or sees its first tile does
-// the wave fall back: it recomputes the scores (requery), finds the maximum and moves the
-// reference points of those rows onto it.
-template <class VT, int D, bool MASK, class VL, class RQ>
-__device__ __forceinline__ void softmax_pv_pre2(f32x16 (&sacc)[2], f32x16 (&o_acc)[D / 32], float& m_run, float& l_run,
-                                                float row_add, f32x16& negm, const VL& vload, const RQ& requery, int lane,
-                                                int j0, int i, int Lb, bool causal) {
-  using vfrag = typename VT::frag;
-  const int g = lane >> 5;
-  auto mask = [&]() __attribute__((always_inline)) {
-    if constexpr (MASK) {
-#pragma unroll
-      for (int jb = 0; jb < 2; ++jb)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int j = j0 + 32 * jb + 8 * (v >> 2) + 4 * g + (v & 3);
-          if (j >= Lb || (causal && j > i)) sacc[jb][v] = -INFINITY;
-        }
-    }
-  };
-  vfrag pf[4];
-  float l_tile = 0.f;
-  auto probs = [&]() __attribute__((always_inline)) {
-    l_tile = 0.f;
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      f32x8 pv;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) pv[e] = __builtin_amdgcn_exp2f(sacc[c >> 1][8 * (c & 1) + e]);
-      pf[c] = VT::from_f32(pv);
-      l_tile = sum8(pv, l_tile);
-    }
-  };
-  const bool first = m_run == -INFINITY;
-  bool slow = __any(first);
-  if (!slow) {
-    mask();
-    probs();
-    slow = __any(!(l_tile <= 256.f));  // 2^kLazyTau; also true for an overflow
-  }
-  if (slow) {
-    // both lanes of a row (its two key halves) must move together
-    const bool mv = first || wave_half_max(l_tile <= 256.f ? 0.f : 1.f) > 0.f;
-    requery(sacc);
-    mask();
-    float mx = sacc[0][0];
-#pragma unroll
-    for (int jb = 0; jb < 2; ++jb)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) mx = fmaxf(mx, sacc[jb][v]);
-    mx = wave_half_max(mx);
-    const float shift = mv ? mx : 0.f;
-    const float alpha = mv ? (first ? 0.f : __builtin_amdgcn_exp2f(-shift)) : 1.f;
-    if (mv) m_run = (first ? 0.f : m_run) + shift;
-    l_run *= alpha;
-#pragma unroll
-    for (int d = 0; d < D / 32; ++d)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) o_acc[d][v] *= alpha;
-#pragma unroll
-    for (int jb = 0; jb < 2; ++jb)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) sacc[jb][v] -= shift;
-    const float nm = row_add - m_run;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) negm[v] = nm;
-    probs();
-  }
-  l_run += l_tile;
-#pragma unroll
-  for (int c = 0; c < 4; ++c)
-#pragma unroll
-    for (int d = 0; d < D / 32; ++d) o_acc[d] = VT::mma(vload(c, d), pf[c], o_acc[d]);
-}
-
 // Two workgroups share a CU (and its 512 registers per lane) when the LDS footprint allows it.
 template <class QT, class VT, int D, bool C2P, bool P2C, int MODE>
 constexpr int min_blocks() {

@@ -137,6 +137,11 @@ bool fdb_near_supported(int dtype, int head_dim);
 // (16-bit element types, head_dim 64); merges the far partial like the ring mode.
 bool fdb_near32_supported(int dtype, int head_dim);
 int fdb_launch_near32(const FdbKParams& p, int dtype, int grid_x, void* stream);
+// The same pair of launches for OCP e4m3 q / k / K_r / Q_r with bf16 v (head_dim 64): e4m3 MFMA contractions over
+// the whole head_dim for the three score products (fdb_fp8.hip).
+bool fdb_fp8_pair_supported(int dtype, int head_dim);
+int fdb_launch_far8(const FdbKParams& p, int grid_x, void* stream);
+int fdb_launch_near8(const FdbKParams& p, int grid_x, void* stream);
 // fdb_launch_merge: after a near launch with near_parts > 1: out / lse from the far partial results (when
 // p.far_done) and the near ones (16-bit element types, head_dim 64).
 int fdb_launch_merge(const FdbKParams& p, int dtype, void* stream);

@@ -99,7 +99,10 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
        padded batches (fixed layout only): seq_start / seq_len int32 [B] GPU tensors give each row's real
        tokens [seq_start, seq_start+seq_len); only those rows of `out` are written, so pass a zeroed `out`
        (or ignore the padded rows).  Either may be None (0 / L).
-       fp8: q/k/pos_* are torch.float8_e4m3fn with float32 per-head scales; v is bfloat16.
+       fp8: q/k/pos_* are torch.float8_e4m3fn with float32 per-head scales; v is bfloat16.  At head_dim 64 the
+       three score products are e4m3 MFMA contractions over the whole head_dim (far / near pair of launches; the
+       far tiles fold Q_r[delta] into the query and round that sum to e4m3 once more); other head_dims and
+       single_kernel=True take the one-kernel e4m3 path.
        single_kernel=True withholds the log-sum-exp buffer, which makes the library walk all key tiles in
        one kernel instead of the far-tile / near-tile pair of launches (same result; for comparison).
        far_splits, near_splits: workgroups that share the far / the near keys of a query tile (0: the library
@@ -109,8 +112,8 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
        library then shares less.
        no_alloc=True goes through fdb_attn_fwd_noalloc: the log-sum-exp hand-over, the work-list of a packed
        call and the partial results come from the scratch built into the library (one per GPU; calls on one
-       GPU must not overlap), so with `out` given nothing is allocated on the way; the fp8 expansion and
-       single_kernel are not available there.
+       GPU must not overlap), so with `out` given nothing is allocated on the way; single_kernel is not
+       available there.
     """
     if not q.is_cuda:
         raise RuntimeError("disentangled_attention_fwd runs on the GPU only; got device %s" % q.device)
@@ -138,20 +141,6 @@ def disentangled_attention_fwd(q, k, v, pos_key=None, pos_query=None, *, cu_seql
         if q_scale is None or k_scale is None or (pos_key is not None and pos_key_scale is None) or (
                 pos_query is not None and pos_query_scale is None):
             raise ValueError("fp8 path: q_scale, k_scale and a scale for each position tensor are required")
-        if D <= 64 and not single_kernel and not no_alloc:
-            # At head_dim <= 64 a key tile is bound by its soft-max and LDS work, not by the MFMA rate, and the
-            # 16-bit kernels (direct-to-LDS staging, far / near pair of launches) are about three times faster
-            # than the fp8-MFMA kernel: FP8 operands are expanded to bf16 (scale applied, one rounding to eight
-            # bits) and take that route.  single_kernel=True keeps the fp8 MFMA contraction.
-            deq = lambda x, s: None if x is None else dequantize_e4m3_per_head(x, s)
-            return disentangled_attention_fwd(
-                deq(q, q_scale), deq(k, k_scale), v,
-                None if pos_key is None else deq(pos_key.transpose(0, 1), pos_key_scale).transpose(0, 1),
-                None if pos_query is None else deq(pos_query.transpose(0, 1), pos_query_scale).transpose(0, 1),
-                cu_seqlens=cu_seqlens, max_seqlen=max_seqlen, sm_scale=sm_scale, position_buckets=position_buckets,
-                max_relative_positions=max_relative_positions, causal=causal, return_lse=return_lse,
-                seq_start=seq_start, seq_len=seq_len, out=out, far_splits=far_splits, near_splits=near_splits,
-                workspace=workspace, _part=_part)
         dt = _lib.FDB_FP8_E4M3
     else:
         if q.dtype not in _DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
