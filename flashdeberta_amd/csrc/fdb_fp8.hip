@@ -375,8 +375,11 @@ __device__ __forceinline__ void rotate16(const float (&xs)[16], float (&px)[16],
    ...);
 }
 
-template <bool C2P, bool P2C>
-__global__ __launch_bounds__(kThreads, 2) void fdb_near8_kernel(const FdbKParams p) {
+// KEEP: block 1 of a step is block 0 of the step before, so C's accumulator and P's A operands of that block are kept
+// from step to step (two workgroups per CU).  Without KEEP both blocks are fetched and contracted in every step -- one
+// more MFMA and two more LDS reads -- and the kernel fits the 168 registers of three workgroups per CU.
+template <bool C2P, bool P2C, bool KEEP>
+__global__ __launch_bounds__(kThreads, (C2P && P2C && KEEP) ? 2 : 3) void fdb_near8_kernel(const FdbKParams p) {
   constexpr int D = 64, DBLKS = 2;
   using VT = Bf16Tr;
   using vfrag = typename VT::frag;
@@ -514,12 +517,17 @@ __global__ __launch_bounds__(kThreads, 2) void fdb_near8_kernel(const FdbKParams
   for (int q = 0; q < 4; ++q)
     c_rd[q] = (LDS_AS const volatile uint16_t*)(scr + li * kScrW + ((li + 28 - 8 * q - 4 * g) & 31));
 
-  i32x8 ac = {0, 0, 0, 0, 0, 0, 0, 0}, aq[2] = {ac, ac};
+  i32x8 ac = {0, 0, 0, 0, 0, 0, 0, 0}, ac1 = ac, aq[2] = {ac, ac};
   f32x16 ckeep[2];
   const uint32_t ek0 = lds0 + (uint32_t)(EK - smem), eq0 = lds0 + (uint32_t)(EQ - smem);
   auto ring_read = [&](int buf, int slot) __attribute__((always_inline)) {
     if constexpr (C2P) ac = lds_frag8(ek0 + slot * kRow8 + rx0, ek0 + slot * kRow8 + rx1);
     if constexpr (P2C) aq[buf] = lds_frag8(eq0 + slot * kRow8 + rx0, eq0 + slot * kRow8 + rx1);
+  };
+  auto ring_read_block1 = [&](int buf, int slot) __attribute__((always_inline)) {  // the rows 32 relative positions up
+    const int s1 = slot >= 32 ? slot - 32 : slot + (kRingRows - 32);
+    if constexpr (C2P) ac1 = lds_frag8(ek0 + s1 * kRow8 + rx0, ek0 + s1 * kRow8 + rx1);
+    if constexpr (P2C) aq[buf] = lds_frag8(eq0 + s1 * kRow8 + rx0, eq0 + s1 * kRow8 + rx1);
   };
   f32x16 zero;
 #pragma unroll
@@ -538,8 +546,10 @@ __global__ __launch_bounds__(kThreads, 2) void fdb_near8_kernel(const FdbKParams
     dnext = d0[5];
     wait_vmcnt<0>();
     __syncthreads();
-    ring_read(1, slot0 >= 32 ? slot0 - 32 : slot0 + (kRingRows - 32));  // block 1 of step 0
-    if constexpr (C2P) ckeep[1] = mma8_sa<127 - kCShift>(ac, qf, zero);
+    if constexpr (KEEP) {
+      ring_read(1, slot0 >= 32 ? slot0 - 32 : slot0 + (kRingRows - 32));  // block 1 of step 0
+      if constexpr (C2P) ckeep[1] = mma8_sa<127 - kCShift>(ac, qf, zero);
+    }
   }
 
   auto step = [&](auto mask_tag, auto par_tag, int k) __attribute__((always_inline)) {
@@ -557,9 +567,11 @@ __global__ __launch_bounds__(kThreads, 2) void fdb_near8_kernel(const FdbKParams
     dnext = batch_delta(k + 6);
     const i32x8 kf = lds_frag8(kx0 + PAR * N8::K_BYTES, kx1 + PAR * N8::K_BYTES);
     ring_read(PAR, slot0);
+    if constexpr (!KEEP) ring_read_block1(PAR ^ 1, slot0);
     f32x16 sacc = zero;
     if constexpr (C2P) {
       ckeep[PAR] = mma8_sa<127 - kCShift>(ac, qf, zero);
+      if constexpr (!KEEP) ckeep[PAR ^ 1] = mma8_sa<127 - kCShift>(ac1, qf, zero);
       const f32x16(&cacc)[2] = ckeep;
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
@@ -752,9 +764,10 @@ __global__ __launch_bounds__(kThreads, 2) void fdb_near8_kernel(const FdbKParams
 
 template <bool C2P, bool P2C>
 int launch_near8_one(const FdbKParams& p, int grid_x, hipStream_t stream) {
-  auto kern = fdb_near8_kernel<C2P, P2C>;
+  constexpr bool kKeep = !(C2P && P2C);   // with both terms: three workgroups per CU
+  auto kern = fdb_near8_kernel<C2P, P2C, kKeep>;
   constexpr int lds = N8::lds_bytes(C2P, P2C);
-  static_assert(lds <= 80 * 1024, "two workgroups per CU");
+  static_assert(lds <= 53 * 1024, "three workgroups per CU (a single term keeps its operands and still fits the registers)");
   static std::atomic<uint64_t> lds_set{0};
   hipError_t e = fdb_set_lds_once((const void*)kern, lds, lds_set);
   if (e != hipSuccess) return (int)e;
