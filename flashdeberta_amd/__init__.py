@@ -5,7 +5,7 @@ shared library exists; touching any operator or model name loads libfdb_hip.so a
 is missing (there is no fallback path).
 """
 _OPS = ("disentangled_attention_fwd", "flash_attention_with_disentangled",
-        "flash_attention_with_disentangled_varlen", "quantize_e4m3_per_head", "dequantize_e4m3_per_head")
+        "flash_attention_with_disentangled_varlen", "quantize_e4m3_per_head", "quantize_e4m3_per_head_pair", "dequantize_e4m3_per_head")
 _MODEL = ("FlashDisentangledSelfAttention", "DEBERTA_SELF_ATTENTION_CLASSES", "FlashDebertaV2Model",
           "patch_model", "DebertaV2Config")
 __all__ = list(_OPS + _MODEL)

@@ -48,7 +48,7 @@ EXPORTS = (
     "fdb_version", "fdb_attn_args_size", "fdb_strerror", "fdb_attn_check", "fdb_attn_fwd", "fdb_attn_fwd_part", "fdb_attn_fwd_noalloc", "fdb_attn_bwd", "fdb_attn_bwd_args_size", "fdb_attn_workspace_bytes",
     "fdb_worklist_ints",
     "fdb_worklist_max_tiles", "fdb_tile_rows", "fdb_build_worklist", "fdb_delta_lut_radius", "fdb_delta_lut", "fdb_delta_lut_window",
-    "fdb_quant_e4m3_per_head", "fdb_dequant_e4m3_per_head",
+    "fdb_quant_e4m3_per_head", "fdb_quant_e4m3_per_head_pair", "fdb_dequant_e4m3_per_head",
 )
 
 
@@ -100,6 +100,8 @@ def _load():
     lib.fdb_delta_lut.argtypes = [i32, i32, i32, vp]
     lib.fdb_quant_e4m3_per_head.restype = ctypes.c_int
     lib.fdb_quant_e4m3_per_head.argtypes = [vp, i64, i64, vp, i64, i64, vp, vp, i32, i32, i32, vp]
+    lib.fdb_quant_e4m3_per_head_pair.restype = ctypes.c_int
+    lib.fdb_quant_e4m3_per_head_pair.argtypes = [vp, vp, i64, i64, vp, vp, i64, i64, vp, vp, vp, i32, i32, i32, vp]
     lib.fdb_dequant_e4m3_per_head.restype = ctypes.c_int
     lib.fdb_dequant_e4m3_per_head.argtypes = [vp, i64, i64, vp, vp, i64, i64, i32, i32, i32, vp]
     return lib

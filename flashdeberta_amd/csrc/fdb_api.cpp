@@ -513,7 +513,20 @@ int fdb_quant_e4m3_per_head(const void* x, int64_t x_stride_t, int64_t x_stride_
   if (!aligned16(x) || (reinterpret_cast<uintptr_t>(y) & 7u) || (x_stride_t * 2) % 16 || (x_stride_h * 2) % 16 ||
       y_stride_t % 8 || y_stride_h % 8)
     return FDB_ERR_ALIGN;
-  return fdb_launch_quant(x, x_stride_t, x_stride_h, y, y_stride_t, y_stride_h, scale, absmax_ws, tokens, heads,
+  return fdb_launch_quant(x, nullptr, x_stride_t, x_stride_h, y, nullptr, y_stride_t, y_stride_h, scale, nullptr, absmax_ws, tokens,
+                          heads, head_dim, stream);
+}
+
+int fdb_quant_e4m3_per_head_pair(const void* x0, const void* x1, int64_t x_stride_t, int64_t x_stride_h, void* y0, void* y1,
+                                 int64_t y_stride_t, int64_t y_stride_h, float* scale0, float* scale1, uint32_t* absmax_ws,
+                                 int32_t tokens, int32_t heads, int32_t head_dim, void* stream) {
+  if (!x0 || !x1 || !y0 || !y1 || !scale0 || !scale1 || !absmax_ws) return FDB_ERR_NULL;
+  if (head_dim != 32 && head_dim != 64 && head_dim != 128) return FDB_ERR_HEAD_DIM;
+  if (tokens < 1 || heads < 1 || heads > 65535) return FDB_ERR_SHAPE;
+  if (!aligned16(x0) || !aligned16(x1) || ((reinterpret_cast<uintptr_t>(y0) | reinterpret_cast<uintptr_t>(y1)) & 7u) ||
+      (x_stride_t * 2) % 16 || (x_stride_h * 2) % 16 || y_stride_t % 8 || y_stride_h % 8)
+    return FDB_ERR_ALIGN;
+  return fdb_launch_quant(x0, x1, x_stride_t, x_stride_h, y0, y1, y_stride_t, y_stride_h, scale0, scale1, absmax_ws, tokens, heads,
                           head_dim, stream);
 }
 

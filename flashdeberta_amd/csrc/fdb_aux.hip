@@ -85,11 +85,21 @@ __device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __builtin
 // grid (token blocks, heads); each thread owns 8 consecutive d of one token.  One atomic per
 // workgroup: all of a head's atomics hit one address and are served one after the other (one per wave
 // from 1024 workgroups per head took 560 us for 50 MB), so the launch also keeps the workgroups few.
+// One or two tensors of one shape and one set of strides per launch (blockIdx.z picks the tensor; its absmax words
+// follow the first tensor's).
+struct QuantPair {
+  const uint16_t* x[2];
+  uint8_t* y[2];
+  float* scale[2];
+};
+
 template <int D>
-__global__ __launch_bounds__(256) void fdb_absmax_kernel(const uint16_t* __restrict__ x, int64_t st, int64_t sh,
-                                                         uint32_t* __restrict__ absmax, int32_t tokens) {
+__global__ __launch_bounds__(256) void fdb_absmax_kernel(const QuantPair pr, int64_t st, int64_t sh,
+                                                         uint32_t* __restrict__ absmax_all, int32_t tokens) {
   constexpr int CPT = D / 8;  // 16-byte chunks per token row
   const int h = blockIdx.y;
+  const uint16_t* __restrict__ x = pr.x[blockIdx.z];
+  uint32_t* __restrict__ absmax = absmax_all + blockIdx.z * gridDim.y;
   float m = 0.f;
   for (int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; c < (int64_t)tokens * CPT;
        c += (int64_t)gridDim.x * blockDim.x) {
@@ -114,12 +124,14 @@ __global__ __launch_bounds__(256) void fdb_absmax_kernel(const uint16_t* __restr
 }
 
 template <int D>
-__global__ __launch_bounds__(256) void fdb_quant_kernel(const uint16_t* __restrict__ x, int64_t st, int64_t sh,
-                                                        uint8_t* __restrict__ y, int64_t yst, int64_t ysh,
-                                                        const uint32_t* __restrict__ absmax, float* __restrict__ scale,
-                                                        int32_t tokens) {
+__global__ __launch_bounds__(256) void fdb_quant_kernel(const QuantPair pr, int64_t st, int64_t sh, int64_t yst, int64_t ysh,
+                                                        const uint32_t* __restrict__ absmax_all, int32_t tokens) {
   constexpr int CPT = D / 8;
   const int h = blockIdx.y;
+  const uint16_t* __restrict__ x = pr.x[blockIdx.z];
+  uint8_t* __restrict__ y = pr.y[blockIdx.z];
+  float* __restrict__ scale = pr.scale[blockIdx.z];
+  const uint32_t* __restrict__ absmax = absmax_all + blockIdx.z * gridDim.y;
   const float amax = fmaxf(__builtin_bit_cast(float, absmax[h]), 1e-12f);
   const float sc = amax / 448.0f;
   if (blockIdx.x == 0 && threadIdx.x == 0) scale[h] = sc;
@@ -283,21 +295,27 @@ int fdb_launch_merge(const FdbKParams& p, int dtype, void* stream) {
   return (int)hipGetLastError();
 }
 
-int fdb_launch_quant(const void* x, int64_t x_st, int64_t x_sh, void* y, int64_t y_st, int64_t y_sh, float* scale,
-                     uint32_t* absmax_ws, int32_t tokens, int32_t heads, int32_t head_dim, void* stream_) {
+int fdb_launch_quant(const void* x0, const void* x1, int64_t x_st, int64_t x_sh, void* y0, void* y1, int64_t y_st, int64_t y_sh,
+                     float* scale0, float* scale1, uint32_t* absmax_ws, int32_t tokens, int32_t heads, int32_t head_dim,
+                     void* stream_) {
   hipStream_t stream = (hipStream_t)stream_;
-  hipLaunchKernelGGL(fdb_fill_u32, dim3((heads + 255) / 256), dim3(256), 0, stream, absmax_ws, heads, 0u);
+  const unsigned n = x1 ? 2u : 1u;
+  QuantPair pr;
+  pr.x[0] = (const uint16_t*)x0; pr.x[1] = (const uint16_t*)x1;
+  pr.y[0] = (uint8_t*)y0; pr.y[1] = (uint8_t*)y1;
+  pr.scale[0] = scale0; pr.scale[1] = scale1;
+  hipLaunchKernelGGL(fdb_fill_u32, dim3((n * heads + 255) / 256), dim3(256), 0, stream, absmax_ws, (int)(n * heads), 0u);
   const int64_t chunks = (int64_t)tokens * head_dim / 8;
   int gx = (int)((chunks + 255) / 256);
   if (gx > 1024) gx = 1024;
   if (gx < 1) gx = 1;
-  int gx_max = 2048 / heads > 1 ? 2048 / heads : 1;  // about 2048 workgroups, i.e. atomics, in all
+  int gx_max = 2048 / heads > 1 ? 2048 / heads : 1;  // about 2048 workgroups, i.e. atomics, per tensor
   if (gx_max > gx) gx_max = gx;
-#define FDB_Q(DD)                                                                                              \
-  hipLaunchKernelGGL(fdb_absmax_kernel<DD>, dim3(gx_max, heads), dim3(256), 0, stream, (const uint16_t*)x, x_st, \
-                     x_sh, absmax_ws, tokens);                                                                 \
-  hipLaunchKernelGGL(fdb_quant_kernel<DD>, dim3(gx, heads), dim3(256), 0, stream, (const uint16_t*)x, x_st,    \
-                     x_sh, (uint8_t*)y, y_st, y_sh, absmax_ws, scale, tokens);
+#define FDB_Q(DD)                                                                                                    \
+  hipLaunchKernelGGL(fdb_absmax_kernel<DD>, dim3(gx_max, heads, n), dim3(256), 0, stream, pr, x_st, x_sh, absmax_ws, \
+                     tokens);                                                                                        \
+  hipLaunchKernelGGL(fdb_quant_kernel<DD>, dim3(gx, heads, n), dim3(256), 0, stream, pr, x_st, x_sh, y_st, y_sh,     \
+                     absmax_ws, tokens);
   switch (head_dim) {
     case 32: FDB_Q(32) break;
     case 64: FDB_Q(64) break;

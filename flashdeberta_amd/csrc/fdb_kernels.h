@@ -146,8 +146,9 @@ int fdb_launch_near8(const FdbKParams& p, int grid_x, void* stream);
 // p.far_done) and the near ones (16-bit element types, head_dim 64).
 int fdb_launch_merge(const FdbKParams& p, int dtype, void* stream);
 int fdb_launch_worklist(const int32_t* cu, int32_t batch, int32_t* wl, int32_t max_tiles, void* stream);
-int fdb_launch_quant(const void* x, int64_t x_st, int64_t x_sh, void* y, int64_t y_st, int64_t y_sh,
-                     float* scale, uint32_t* absmax_ws, int32_t tokens, int32_t heads, int32_t head_dim,
+// one tensor (x1 == NULL) or two of one shape and one set of strides: fill, absmax and quantise in three launches
+int fdb_launch_quant(const void* x0, const void* x1, int64_t x_st, int64_t x_sh, void* y0, void* y1, int64_t y_st, int64_t y_sh,
+                     float* scale0, float* scale1, uint32_t* absmax_ws, int32_t tokens, int32_t heads, int32_t head_dim,
                      void* stream);
 int fdb_launch_dequant(const void* y, int64_t y_st, int64_t y_sh, const float* scale, void* x, int64_t x_st, int64_t x_sh,
                        int32_t tokens, int32_t heads, int32_t head_dim, void* stream);

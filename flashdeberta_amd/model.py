@@ -84,7 +84,7 @@ class FlashDisentangledSelfAttention(DisentangledSelfAttention):
     def __init__(self, config, fp8_qk=None):
         super().__init__(config)
         self.fp8_qk = bool(getattr(config, "fp8_qk", False)) if fp8_qk is None else bool(fp8_qk)
-        self._qkv_memo, self._pos_memo, self._mask_memo = _Memo(), _Memo(), _Memo()
+        self._qkv_memo, self._pos_memo, self._mask_memo, self._pos8_memo = _Memo(), _Memo(), _Memo(), _Memo()
 
     def _fused_qkv(self):
         """Concatenated [3*H*D, hidden] weight and bias of the query, key and value projections."""
@@ -178,14 +178,26 @@ class FlashDisentangledSelfAttention(DisentangledSelfAttention):
         if self.fp8_qk:
             if q.dtype != torch.bfloat16:
                 raise ValueError("fp8_qk needs bfloat16 activations")
-            q, kw["q_scale"] = ops.quantize_e4m3_per_head(q)
-            k, kw["k_scale"] = ops.quantize_e4m3_per_head(k)
-            if pos_key is not None:
-                pos_key, kw["pos_key_scale"] = ops.quantize_e4m3_per_head(pos_key.transpose(0, 1))
-                pos_key = pos_key.transpose(0, 1)
-            if pos_query is not None:
-                pos_query, kw["pos_query_scale"] = ops.quantize_e4m3_per_head(pos_query.transpose(0, 1))
-                pos_query = pos_query.transpose(0, 1)
+            # q and k of the layer in one set of launches; K_r / Q_r likewise, and remembered for as long as the
+            # projected relative embeddings are the same tensors (outside training they are, see _pos_layers)
+            q, kw["q_scale"], k, kw["k_scale"] = ops.quantize_e4m3_per_head_pair(q, k)
+            pos = tuple(x for x in (pos_key, pos_query) if x is not None)
+            hit = self._pos8_memo.get(pos) if pos else None
+            if hit is None and pos:
+                if len(pos) == 2:
+                    k8, ks, q8, qs = ops.quantize_e4m3_per_head_pair(pos_key.transpose(0, 1), pos_query.transpose(0, 1))
+                    hit = (k8.transpose(0, 1), ks, q8.transpose(0, 1), qs)
+                else:
+                    y, sc = ops.quantize_e4m3_per_head(pos[0].transpose(0, 1))
+                    hit = (y.transpose(0, 1), sc, None, None) if pos_key is not None else (None, None, y.transpose(0, 1), sc)
+                if not (torch.is_grad_enabled() and any(x.requires_grad for x in pos)):
+                    self._pos8_memo.put(pos, hit)
+            if pos:
+                pos_key, pos_key_scale, pos_query, pos_query_scale = hit
+                if pos_key is not None:
+                    kw["pos_key_scale"] = pos_key_scale
+                if pos_query is not None:
+                    kw["pos_query_scale"] = pos_query_scale
 
         ctx = ops.disentangled_attention(
             q, k, v, pos_key, pos_query, sm_scale=sm_scale,

@@ -497,6 +497,28 @@ def quantize_e4m3_per_head(x):
     return y.view(_FP8).reshape(x.shape), scale
 
 
+def quantize_e4m3_per_head_pair(x0, x1):
+    """quantize_e4m3_per_head for two bf16 tensors of one shape and one set of strides (q and k of a layer, K_r and
+    Q_r) in the same three launches -> (y0, scale0, y1, scale1).  Tensors whose layouts differ are made contiguous."""
+    for x in (x0, x1):
+        if not x.is_cuda or x.dtype != torch.bfloat16:
+            raise ValueError("quantize_e4m3_per_head_pair expects bfloat16 GPU tensors")
+    if x0.shape != x1.shape:
+        raise ValueError("quantize_e4m3_per_head_pair: shapes differ: %s %s" % (tuple(x0.shape), tuple(x1.shape)))
+    H, D = x0.shape[-2], x0.shape[-1]
+    a, b = x0.reshape(-1, H, D), x1.reshape(-1, H, D)
+    if a.stride() != b.stride() or a.stride(2) != 1:
+        a, b = a.contiguous(), b.contiguous()
+    y = torch.empty((2,) + tuple(a.shape), dtype=torch.uint8, device=a.device)
+    scale = torch.empty((2, H), dtype=torch.float32, device=a.device)
+    ws = torch.empty(2 * H, dtype=torch.int32, device=a.device)
+    with torch.cuda.device(a.device):
+        check(lib.fdb_quant_e4m3_per_head_pair(_ptr(a), _ptr(b), a.stride(0), a.stride(1), _ptr(y[0]), _ptr(y[1]), y.stride(1), y.stride(2),
+                                               _ptr(scale[0]), _ptr(scale[1]), _ptr(ws), a.shape[0], H, D, _stream_ptr(a.device)),
+              "fdb_quant_e4m3_per_head_pair")
+    return y[0].view(_FP8).reshape(x0.shape), scale[0], y[1].view(_FP8).reshape(x1.shape), scale[1]
+
+
 def dequantize_e4m3_per_head(y, scale):
     """y: float8_e4m3fn [..., H, D] on the GPU, scale float32 [H] -> bfloat16 tensor of the same shape,
     x = bf16_rne(y * scale[h])."""

@@ -24,7 +24,8 @@
  *                             followed by clamp(. + S, 0, 2S-1) (:318, :336); host-side, integers out.
  *   fdb_attn_bwd           <- flash_attn_v2_bwd_dise (flash_attention.py:942-1030) with _bwd_preprocess,
  *                             _bwd_kv_dise_kernel and _bwd_q_dise_kernel (:62-141, :581-941).
- *   fdb_quant_e4m3_per_head, fdb_dequant_e4m3_per_head   no reference counterpart (FP8 Q/K variant).
+ *   fdb_quant_e4m3_per_head, fdb_quant_e4m3_per_head_pair, fdb_dequant_e4m3_per_head   no reference counterpart
+ *                             (FP8 Q/K variant).
  */
 #ifndef FDB_H_
 #define FDB_H_
@@ -290,10 +291,19 @@ int fdb_quant_e4m3_per_head(const void* x, int64_t x_stride_t, int64_t x_stride_
                             int32_t tokens, int32_t heads, int32_t head_dim, void* stream);
 
 /*
+ * The same for two tensors of one shape and one set of strides in the same three launches (fill, absmax,
+ * quantise) -- q and k of a layer, or K_r and Q_r.  absmax_ws: device uint32[2 * heads].  Each tensor gets its own
+ * scales.  No reference counterpart (FP8 Q/K variant).
+ */
+int fdb_quant_e4m3_per_head_pair(const void* x0, const void* x1, int64_t x_stride_t, int64_t x_stride_h,
+                                 void* y0, void* y1, int64_t y_stride_t, int64_t y_stride_h,
+                                 float* scale0, float* scale1, uint32_t* absmax_ws,
+                                 int32_t tokens, int32_t heads, int32_t head_dim, void* stream);
+
+/*
  * The inverse map to bf16, x = bf16_rne(e4m3(y) * scale[h]), same indexing as above (y: one byte per
  * element, 8-byte aligned rows; x: bf16, 16-byte aligned rows).  No reference counterpart (FP8 Q/K
- * variant): the host side uses it to run FP8 operands through the 16-bit kernels where those are the
- * faster ones (head_dim <= 64).
+ * variant); a utility for callers and tests, not used by fdb_attn_fwd.
  */
 int fdb_dequant_e4m3_per_head(const void* y, int64_t y_stride_t, int64_t y_stride_h, const float* scale,
                               void* x, int64_t x_stride_t, int64_t x_stride_h,

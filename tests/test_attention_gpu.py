@@ -647,6 +647,59 @@ def test_fp8_quantisation_bit_exact():
     wide[..., :64] = x
     y2, s2 = ops.quantize_e4m3_per_head(wide.cuda()[..., :64])
     assert torch.equal(y2.view(torch.uint8), y.view(torch.uint8)) and torch.equal(s2, s)
+    # two tensors in one set of launches: the same bytes and scales as one at a time -- q and k as the module hands them
+    # over (views of one fused projection output, equal strides) and two tensors whose layouts differ
+    x1 = _outliers(torch.randn(700, 12, 64, generator=g) * 0.5, g).to(torch.bfloat16)
+    y1, s1 = ops.quantize_e4m3_per_head(x1.cuda())
+    qkv = torch.stack([x, x1, x], dim=1).cuda()  # [T, 3, H, D]
+    for a, b in ((qkv[:, 0], qkv[:, 1]), (x.cuda(), qkv[:, 1])):
+        ya, sa, yb, sb = ops.quantize_e4m3_per_head_pair(a, b)
+        assert torch.equal(ya.view(torch.uint8), y.view(torch.uint8)) and torch.equal(sa, s)
+        assert torch.equal(yb.view(torch.uint8), y1.view(torch.uint8)) and torch.equal(sb, s1)
+
+
+def test_module_with_fp8_operands_matches_the_operator():
+    """fp8_qk=True: the module quantises q and k in one set of launches and remembers the quantised K_r / Q_r while the
+    projected relative embeddings are unchanged; its output equals the operator's on operands quantised one by one, and
+    stays within the fp8 bound of the 16-bit module."""
+    from flashdeberta_amd import FlashDisentangledSelfAttention
+
+    class Cfg:
+        hidden_size, num_attention_heads = 256, 4
+        attention_probs_dropout_prob = hidden_dropout_prob = 0.0
+        pos_att_type = ["c2p", "p2c"]
+        relative_attention, position_buckets, max_relative_positions = True, 32, 64
+        max_position_embeddings, share_att_key = 512, True
+
+    torch.manual_seed(7)
+    att = FlashDisentangledSelfAttention(Cfg()).eval().cuda().to(torch.bfloat16)
+    att8 = FlashDisentangledSelfAttention(Cfg(), fp8_qk=True).eval().cuda().to(torch.bfloat16)
+    att8.load_state_dict(att.state_dict())
+    x = torch.randn(2, 300, 256, device="cuda", dtype=torch.bfloat16)
+    rel = torch.randn(64, 256, device="cuda", dtype=torch.bfloat16)
+    with torch.no_grad():
+        ref16 = att(x, None, rel_embeddings=rel)[0]
+        out = att8(x, None, rel_embeddings=rel)[0]
+        again = att8(x, None, rel_embeddings=rel)[0]          # K_r / Q_r come from the memo now
+        q, k, v = att8._qkv(x, x)
+        pk, pq = att8._pos_layers(rel)
+        q8, qs = ops.quantize_e4m3_per_head(q)
+        k8, ks = ops.quantize_e4m3_per_head(k)
+        pk8, pks = ops.quantize_e4m3_per_head(pk.transpose(0, 1))
+        pq8, pqs = ops.quantize_e4m3_per_head(pq.transpose(0, 1))
+        want = ops.disentangled_attention_fwd(q8, k8, v, pk8.transpose(0, 1), pq8.transpose(0, 1), position_buckets=32,
+                                              max_relative_positions=64, q_scale=qs, k_scale=ks, pos_key_scale=pks,
+                                              pos_query_scale=pqs).view(2, 300, 256)
+    assert torch.equal(out, want) and torch.equal(again, out)
+    assert att8._pos8_memo.get((pk, pq)) is not None
+    err = (out.float() - ref16.float()).abs().max().item()
+    assert err <= FP8_TOL * max(1.0, ref16.float().abs().max().item()), err
+    rel2 = rel * 2                                             # another embedding tensor: nothing stale is reused
+    with torch.no_grad():
+        out2 = att8(x, None, rel_embeddings=rel2)[0]
+        ref2 = att(x, None, rel_embeddings=rel2)[0]
+    assert not torch.equal(out2, out)
+    assert (out2.float() - ref2.float()).abs().max().item() <= FP8_TOL * max(1.0, ref2.float().abs().max().item())
 
 
 def test_fp8_dequantisation_exact():
