@@ -284,6 +284,12 @@ int fdb_attn_check(const fdb_attn_args* a) {
   // the kernels walk K and V with 32-bit row strides (in bytes)
   if (a->k_stride_t < 0 || a->v_stride_t < 0 || a->k_stride_t * qsz > INT32_MAX || a->v_stride_t * vsz > INT32_MAX)
     return FDB_ERR_SHAPE;
+  // ... and the rows of K_r / Q_r with 32-bit byte offsets from a head's first row (24-bit row strides)
+  const int64_t table_rows = 2 * (int64_t)a->att_span;
+  if (a->pos_key && (a->pk_stride_r < 0 || a->pk_stride_r * qsz >= (1 << 24) || table_rows * a->pk_stride_r * qsz > INT32_MAX))
+    return FDB_ERR_SHAPE;
+  if (a->pos_query && (a->pq_stride_r < 0 || a->pq_stride_r * qsz >= (1 << 24) || table_rows * a->pq_stride_r * qsz > INT32_MAX))
+    return FDB_ERR_SHAPE;
   const int64_t v_strides[] = {a->v_stride_b, a->v_stride_t, a->v_stride_h, a->o_stride_b, a->o_stride_t, a->o_stride_h};
   for (int64_t s : v_strides)
     if ((s * vsz) % 16 != 0) return FDB_ERR_ALIGN;

@@ -163,15 +163,28 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
   const uint32_t wave_kb = (uint32_t)wave * 1024u;                  // this wave's 1 KB of a 32-row tile
   const uint32_t chunk_off = (uint32_t)((scc ^ ring_f(srow)) * 16);
   int dnext = 0;
+  // A step inside the sequence: its first row travels as the scalar base of the load, this thread's place in the
+  // tile as a 32-bit offset computed once.  Only a step that reaches past the end clamps its rows one by one.
+  const uint32_t k_lane = (uint32_t)(srow ^ 3) * k_rsb + chunk_off, v_lane = (uint32_t)srow * v_rsb + chunk_off;
   auto k_dma = [&](int s, int buf) __attribute__((always_inline)) {
     // LDS row srow holds key srow ^ 3 of the step (see the scratch reads below); rows past the end
     // re-read the last one, their scores are masked
-    const int row = min(s * kStep + (srow ^ 3), Lb - 1);
-    dma16(kb + (uint64_t)(uint32_t)row * k_rsb + chunk_off, lds0 + buf * NCfg::K_BYTES + wave_kb);
+    const uint32_t dst = lds0 + buf * NCfg::K_BYTES + wave_kb;
+    if ((s + 1) * kStep <= Lb) {
+      dma16s(kb + (uint64_t)(uint32_t)(s * kStep) * k_rsb, k_lane, dst);
+    } else {
+      const int row = min(s * kStep + (srow ^ 3), Lb - 1);
+      dma16(kb + (uint64_t)(uint32_t)row * k_rsb + chunk_off, dst);
+    }
   };
   auto v_dma = [&](int s, int buf) __attribute__((always_inline)) {
-    const int row = min(s * kStep + srow, Lb - 1);
-    dma16(vb + (uint64_t)(uint32_t)row * v_rsb + chunk_off, lds0 + 2 * NCfg::K_BYTES + buf * NCfg::V_BYTES + wave_kb);
+    const uint32_t dst = lds0 + 2 * NCfg::K_BYTES + buf * NCfg::V_BYTES + wave_kb;
+    if ((s + 1) * kStep <= Lb) {
+      dma16s(vb + (uint64_t)(uint32_t)(s * kStep) * v_rsb, v_lane, dst);
+    } else {
+      const int row = min(s * kStep + srow, Lb - 1);
+      dma16(vb + (uint64_t)(uint32_t)row * v_rsb + chunk_off, dst);
+    }
   };
   auto batch_delta = [&](int batch) __attribute__((always_inline)) {  // table row of this thread's ring row
     const int r = r_hi0 - (batch * 32 + srow);
@@ -180,10 +193,13 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
     return (int)((const uint16_t*)p.lut)[max(-p.R, min(p.R, r)) + p.R];
   };
   const uint32_t ek_lds = lds0 + (uint32_t)(EK - smem) + wave_kb, eq_lds = lds0 + (uint32_t)(EQ - smem) + wave_kb;
+  // table rows are addressed with 32-bit byte offsets from the head's first row (the host checks that a row stride
+  // stays under 2^24 bytes and the whole table under 2^31)
+  const uint32_t pk_rowb = (uint32_t)(p.pk_sr * 2), pq_rowb = (uint32_t)(p.pq_sr * 2);
   auto batch_dma = [&](int delta, int batch) __attribute__((always_inline)) {
     const uint32_t seg = (uint32_t)(batch % kRingBatches) * (32 * kRowBytes);
-    if constexpr (C2P) dma16(pkb + (int64_t)delta * p.pk_sr * 2 + chunk_off, ek_lds + seg);
-    if constexpr (P2C) dma16(pqb + (int64_t)delta * p.pq_sr * 2 + chunk_off, eq_lds + seg);
+    if constexpr (C2P) dma16s(pkb, __umul24((uint32_t)delta, pk_rowb) + chunk_off, ek_lds + seg);
+    if constexpr (P2C) dma16s(pqb, __umul24((uint32_t)delta, pq_rowb) + chunk_off, eq_lds + seg);
   };
 
   f32x16 o_acc[DBLKS];
@@ -308,9 +324,23 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
 #pragma unroll
     for (int v = 0; v < 16; ++v) sacc[v] = 0.f;
     const f32x16 zero = sacc;
-    if constexpr (C2P) {
+    f32x16 pacc[2];
+    // The sixteen MFMAs of the four score products first, in two pairs of chains that alternate (no MFMA waits for
+    // its own previous link): C with P's block 1 (whose operands are this step's keys and the rows kept from the
+    // step before), then P's block 0 with the content product.  What follows C -- the pick, the scratch round trip --
+    // runs under the second pair.
 #pragma unroll
-      for (int x = 0; x < KS; ++x) ckeep[PAR] = QT::mma(ac[x], qf[x], x == 0 ? zero : ckeep[PAR]);
+    for (int x = 0; x < KS; ++x) {
+      if constexpr (C2P) ckeep[PAR] = QT::mma(ac[x], qf[x], x == 0 ? zero : ckeep[PAR]);
+      if constexpr (P2C) pacc[1] = QT::mma(kf[x], aq[PAR ^ 1][x], x == 0 ? zero : pacc[1]);
+    }
+#pragma unroll
+    for (int x = 0; x < KS; ++x) {
+      if constexpr (P2C) pacc[0] = QT::mma(kf[x], aq[PAR][x], x == 0 ? zero : pacc[0]);
+      sacc = QT::mma(kf[x], qf[x], sacc);
+    }
+    uint16_t craw[16];
+    if constexpr (C2P) {
       const f32x16(&cacc)[2] = ckeep;  // block bk of this step sits in ckeep[PAR ^ bk]
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {  // C[i = li][(32*bk) + 8*q4 + 4*g + 0..3], block 0 where that column is >= li
@@ -327,25 +357,14 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
       }
       wave_lds_fence();
 #pragma unroll
-      for (int v = 0; v < 16; ++v)
-        sacc[v] = QT::scratch_to_f32(c_rd[v >> 2][v & 3]);
+      for (int v = 0; v < 16; ++v) craw[v] = c_rd[v >> 2][v & 3];
       wave_lds_fence();
-      __builtin_amdgcn_sched_barrier(0);
     }
     // P with the keys as MFMA rows, like the content product: register v of lane (g, n) holds
     // P[jj(v, g)][32 bk + n], and element (jj, i = li) wants column li + 31 - jj of that row, i.e. the same
     // register of another lane of its own half.  Each source lane is read by exactly one lane, which
     // wants block 1 from it if n + jj < 31 and block 0 otherwise: the source picks, one lane permutation
     // per register moves it.
-    f32x16 pacc[2];
-    if constexpr (P2C) {
-#pragma unroll
-      for (int bk = 0; bk < 2; ++bk)
-#pragma unroll
-        for (int x = 0; x < KS; ++x) pacc[bk] = QT::mma(kf[x], aq[PAR ^ bk][x], x == 0 ? zero : pacc[bk]);
-    }
-#pragma unroll
-    for (int x = 0; x < KS; ++x) sacc = QT::mma(kf[x], qf[x], sacc);
     float px[16];
     if constexpr (P2C) {
       // Source lane (g, n) of register v (key jj = 4g + c) is read by lane (g, (n - rot) mod 32), which wants
@@ -366,10 +385,22 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
       else
         rotate16<27>(xs, px, std::make_integer_sequence<int, 16>{});
     }
-    if constexpr (P2C) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) sacc[v] += px[v];
+    for (int v = 0; v < 16; ++v) {
+      if constexpr (C2P) sacc[v] += QT::scratch_to_f32(craw[v]);
+      if constexpr (P2C) sacc[v] += px[v];
     }
+    // V^T operands requested here, ahead of the soft-max, so that the four MFMAs at the end of the step find them
+    vfrag vfr[2][DBLKS];
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int d = 0; d < DBLKS; ++d) {
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(Vs + PAR * NCfg::V_BYTES + vlx[2 * d] + 2048 * c));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(Vs + PAR * NCfg::V_BYTES + vlx[2 * d + 1] + 2048 * c + 1024));
+        vfr[c][d] = __builtin_bit_cast(vfrag, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      }
+    __builtin_amdgcn_sched_barrier(0);
     // ---- mask, online soft-max in base 2, O^T += V^T P^T ---------------------------------------------------
     if constexpr (MASK) {
 #pragma unroll
@@ -422,12 +453,7 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
 #pragma unroll
     for (int c = 0; c < 2; ++c)
 #pragma unroll
-      for (int d = 0; d < DBLKS; ++d) {
-        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(Vs + PAR * NCfg::V_BYTES + vlx[2 * d] + 2048 * c));
-        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(Vs + PAR * NCfg::V_BYTES + vlx[2 * d + 1] + 2048 * c + 1024));
-        const vfrag vf = __builtin_bit_cast(vfrag, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-        o_acc[d] = VT::mma(vf, pf[c], o_acc[d]);
-      }
+      for (int d = 0; d < DBLKS; ++d) o_acc[d] = VT::mma(vfr[c][d], pf[c], o_acc[d]);
     slot0 = slot0 + 32 >= kRingRows ? slot0 + 32 - kRingRows : slot0 + 32;
   };
   {

@@ -83,7 +83,9 @@ enum fdb_status {
  *   score(i,j) = sm_scale * ( q_i.k_j + q_i.K_r[delta(i-j)] + k_j.Q_r[delta(i-j)] ),
  *   delta(r) = delta_lut[clamp(r, -lut_radius, lut_radius) + lut_radius]; a NULL pos pointer
  *   drops that term.  out_i = sum_j softmax_j(score(i,.)) v_j ; lse_i = log sum_j exp(score(i,j)).
- * Strides are in elements.  The last dimension has unit stride.
+ * Strides are in elements.  The last dimension has unit stride.  Token strides of k and v below 2^31 bytes;
+ * row strides of pos_key / pos_query non-negative and below 2^24 bytes, a head's 2S rows within 2^31 bytes
+ * (FDB_ERR_SHAPE otherwise).
  */
 typedef struct fdb_attn_args {
   const void* q;
