@@ -4,27 +4,33 @@
 // (rows normalised over the far keys in out, their log-sum-exp in lse) is merged in the epilogue.
 //
 // The position products need the rows E_K[r] = K_r[delta(r)] and E_Q[r] = Q_r[delta(r)] for the
-// contiguous range of relative positions r of a tile.  They are staged in LDS rings with coalesced
+// contiguous range of relative positions r of a tile.  They are staged in LDS rings with direct
 // loads, so the MFMA A operands are plain LDS reads.
 //
-// What shapes this kernel is LDS: a wave alone on its SIMD issues a dependent instruction only
-// every eight to nine cycles, and nothing else hides that but a second wave.  Two workgroups share
-// a CU when each stays under 80 KB, which the rings allow only with 32-key steps:
+// What shapes this kernel is the issue rate of a wave: with two waves on a SIMD a wave issues one
+// instruction of any kind -- vector, scalar, LDS, wait -- about every five clocks, and a step's time is its
+// instruction count times that plus the MFMAs' own 32 clocks each; so the step is written for the fewest
+// instructions, not for the fewest of one kind.  Two workgroups share a CU when each stays under 80 KB of
+// LDS, which the rings allow only with 32-key steps:
 //   workgroup = 4 waves x 32 query rows, one step = 32 keys;
-//   a step sees 159 relative positions (5 batches of 32); the rings hold a sixth batch, the one being
-//   filled for the next step: 192 rows of 128 bytes, unpadded and XOR-swizzled;
+//   a step sees 160 relative positions, five batches of 32, one per (wave, block); each ring holds exactly
+//   these five (160 rows of 128 bytes, unpadded and XOR-swizzled): the batch a step's loads bring in for the
+//   next step takes the place of the one no wave reads any more;
 //   a wave's 32 x 32 sub-tile sees 63 relative positions, so both position products are 2 MFMA
-//   blocks, private to the wave: C[i][r] = q_i . E_K[r] and P[j][r] = k_j . E_Q[r], of which element
-//   (i, j) wants index r = i - j.  C goes through a per-wave 16-bit LDS scratch (only the one of its
-//   two blocks a lane needs, picked before the write) and comes back as the initial value of the
-//   content product's accumulator; P is computed with the keys as MFMA rows, so its skew is a rotation
+//   blocks, private to the wave: C[r][i] = q_i . E_K[r] and P[j][r] = k_j . E_Q[r], of which element
+//   (i, j) wants index r = i - j.  C goes through a per-wave 16-bit LDS scratch that holds both blocks: a
+//   step contracts and writes only the block that is new to it (the other one is the block the step before
+//   wrote), and reads its skewed band back with sixteen 2-byte loads that land in the upper half of a
+//   register, i.e. as fp32 values; P is computed with the keys as MFMA rows, so its skew is a rotation
 //   of the lanes of a half-wave by a constant of the register (ds_swizzle) and needs no scratch.
-// LDS: K 2 x 4 KB + V 2 x 4 KB + rings 2 x 24 KB + scratch 11 KB = 75 KB.
+//   The query operand carries the soft-max scale and the content product starts from minus the row's
+//   reference point, so the sum leaves for the exponential as it is.
+// LDS: K 2 x 4 KB + V 2 x 4 KB + rings 2 x 20 KB + scratch 17 KB = 73 KB.
 //
 // Staging goes global -> LDS directly (global_load_lds_dwordx4: no staging registers, no LDS write
 // instructions of the waves' own) and runs one step ahead: right after the one barrier of step s (every
 // wave is done with step s-1) a wave issues its share of K(s+1) and V(s+1) into the buffers step s does not
-// read and of the 32 rows per table that step s+1 reads for the first time into the ring's sixth batch;
+// read and of the 32 rows per table that step s+1 reads for the first time;
 // it waits for these loads at the top of step s+1, before that step's barrier, behind which everybody's
 // have landed.  The loads have a whole step to arrive.
 #include <hip/hip_runtime.h>
@@ -42,11 +48,11 @@ namespace {
 
 constexpr int kNThreads = 256;
 constexpr int kStep = 32;        // keys per step
-constexpr int kRingBatches = 6;  // 5 batches of 32 relative positions in use by a step + the one being filled for the next
+constexpr int kRingBatches = 5;  // batches of 32 relative positions in a ring: the five a step reads
 constexpr int kRingRows = 32 * kRingBatches;
-constexpr int kScrW = 44;        // 16-bit elements between the rows of a wave's bias scratch: 36 in use; rows 8-byte aligned, and
-                                 // 22 words apart, so that the 32 rows of a write land in 64 different banks
-constexpr int kScrElems = 32 * kScrW;
+constexpr int kScrPitch = 68;    // 16-bit elements per row of a wave's C scratch: two blocks of 32 columns + columns 0..3 once
+                                 // more (a run of four never wraps); 34 words, so the 32 rows of a write land in 32 different bank pairs
+constexpr int kScrElems = 32 * kScrPitch;
 constexpr int kRowBytes = 128;   // head_dim 64, 16-bit
 
 struct NCfg {
@@ -64,12 +70,45 @@ struct NCfg {
 __device__ __forceinline__ int ring_f(int row) { return 4 * ((row >> 1) & 1) | ((row >> 2) & 3); }
 
 // px[v] = xs[v] of the lane (ROT0 - c(v)) places further up in this lane's half-wave (mod 32), c(v) = 8*(v/4) + 3 - v%4:
-// ds_swizzle in rotate mode, the amount in the instruction's offset field (0xC000 | amount << 5).
+// ds_swizzle in rotate mode, the amount in the instruction's offset field (0xC000 | amount << 5).  Issued as asm, so
+// that the compiler keeps no account of it: the step waits once for all its LDS traffic (lds_wait_all) instead
+// of once per value.
+template <int OFFSET>
+__device__ __forceinline__ float swizzle_asm(float x) {
+  float r;
+  asm volatile("ds_swizzle_b32 %0, %1 offset:%2" : "=v"(r) : "v"(x), "n"(OFFSET));
+  return r;
+}
 template <int ROT0, int... V>
 __device__ __forceinline__ void rotate16(const float (&xs)[16], float (&px)[16], std::integer_sequence<int, V...>) {
-  ((px[V] = __builtin_bit_cast(
-        float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, xs[V]), 0xC000 | ((ROT0 - (8 * (V >> 2) + 3 - (V & 3))) << 5)))),
-   ...);
+  ((px[V] = swizzle_asm<(0xC000 | (((ROT0 - (8 * (V >> 2) + 3 - (V & 3))) & 31) << 5))>(xs[V])), ...);
+}
+
+// A 16-bit LDS element as fp32.  bf16: the load that fills the upper half of the register clears the lower half on
+// this hardware, so the register is the value; issued as asm, the caller waits (lds_wait_all) before it uses the value.
+template <class QT, int OFF>
+__device__ __forceinline__ float lds_elem_f32(uint32_t addr) {
+  if constexpr (std::is_same<QT, Bf16Tr>::value) {
+    float r;
+    asm volatile("ds_read_u16_d16_hi %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
+    return r;
+  } else {
+    return (float)*(LDS_AS const _Float16*)(uintptr_t)(addr + OFF);
+  }
+}
+__device__ __forceinline__ void lds_wait_all() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+
+// The direct loads of this kernel: M0 is set and left (nothing else in the kernel reads it).
+__device__ __forceinline__ void dma16n(const void* g, uint32_t lds_base) {
+  const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(base) : "memory");
+}
+__device__ __forceinline__ void dma16sn(const void* base, uint32_t lane_off, uint32_t lds_base) {
+  const uint32_t lb = __builtin_amdgcn_readfirstlane(lds_base);
+  const uint64_t b64 = (uint64_t)(uintptr_t)base;
+  const uint32_t blo = __builtin_amdgcn_readfirstlane((uint32_t)b64), bhi = __builtin_amdgcn_readfirstlane((uint32_t)(b64 >> 32));
+  const uint64_t sb = ((uint64_t)bhi << 32) | blo;
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(lane_off), "s"(sb), "s"(lb) : "memory");
 }
 
 template <class QT, class VT, bool C2P, bool P2C>
@@ -90,7 +129,6 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
   const int lane = tid & 63, li = lane & 31, g = lane >> 5;
   int xq, h;
   block_map((int)blockIdx.x, p.grid_x, p.H, p.tiles_per_seq, p.cu == nullptr, kMiddleFirst, xq, h);
-  uint16_t* scr = (uint16_t*)scr_raw + wave * kScrElems;
 
   int b, m0, tok0, Lb;
   int64_t qo, ko, vo, oo;
@@ -133,6 +171,10 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
   // compiler wait for every outstanding vector-memory load at the top of each step.
 #pragma unroll
   for (int s = 0; s < KS; ++s) asm volatile("" ::"v"(qf[s]));
+  // the query operand carries the soft-max scale (in base 2): the content product and C leave the MFMA in the
+  // exponent's unit; P, which the keys make, is scaled where it is added
+#pragma unroll
+  for (int s = 0; s < KS; ++s) qf[s] = QT::from_f32(QT::to_f32(qf[s]) * x_scale);
 
   // ---- the near range: the 64-key tiles the far-only run skips, walked 32 keys at a time -----------
   int j_end = Lb;
@@ -151,8 +193,9 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
   const int n_steps = s1 - s0;
   const int n_full = p.causal ? 0 : max(0, min(n_steps, Lb / kStep - s0));  // steps k < n_full need no mask
 
-  // relative positions of the workgroup at step k = s - s0: r in [r_hi0 - 32k - 158, r_hi0 - 32k];
-  // u = r_hi0 - r counts downwards from the first step's largest r; ring slot = u mod 192; batch = u / 32.
+  // relative positions of the workgroup at step k = s - s0: r in [r_hi0 - 32k - 159, r_hi0 - 32k];
+  // u = r_hi0 - r counts downwards from the first step's largest r; batch = u / 32, ring slot = batch mod 5.
+  // Wave w's block bk at step k is batch k + 4 - w - bk, MFMA row m its row 31 - m: r = iw0 - 32s - 32 + 32bk + m.
   const int r_hi0 = m0 + FDB_BM - 1 - s0 * kStep;
 
   // ---- staging: one 16-byte chunk per thread of K, of V and of one batch of each ring ----------------
@@ -171,35 +214,38 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
     // re-read the last one, their scores are masked
     const uint32_t dst = lds0 + buf * NCfg::K_BYTES + wave_kb;
     if ((s + 1) * kStep <= Lb) {
-      dma16s(kb + (uint64_t)(uint32_t)(s * kStep) * k_rsb, k_lane, dst);
+      dma16sn(kb + (uint64_t)(uint32_t)(s * kStep) * k_rsb, k_lane, dst);
     } else {
       const int row = min(s * kStep + (srow ^ 3), Lb - 1);
-      dma16(kb + (uint64_t)(uint32_t)row * k_rsb + chunk_off, dst);
+      dma16n(kb + (uint64_t)(uint32_t)row * k_rsb + chunk_off, dst);
     }
   };
   auto v_dma = [&](int s, int buf) __attribute__((always_inline)) {
     const uint32_t dst = lds0 + 2 * NCfg::K_BYTES + buf * NCfg::V_BYTES + wave_kb;
     if ((s + 1) * kStep <= Lb) {
-      dma16s(vb + (uint64_t)(uint32_t)(s * kStep) * v_rsb, v_lane, dst);
+      dma16sn(vb + (uint64_t)(uint32_t)(s * kStep) * v_rsb, v_lane, dst);
     } else {
       const int row = min(s * kStep + srow, Lb - 1);
-      dma16(vb + (uint64_t)(uint32_t)row * v_rsb + chunk_off, dst);
+      dma16n(vb + (uint64_t)(uint32_t)row * v_rsb + chunk_off, dst);
     }
   };
-  auto batch_delta = [&](int batch) __attribute__((always_inline)) {  // table row of this thread's ring row
-    const int r = r_hi0 - (batch * 32 + srow);
+  // table row of this thread's row of a batch; the relative position runs down by 32 per batch
+  int r_tab = r_hi0 - srow;
+  auto batch_delta = [&]() __attribute__((always_inline)) {
     // table rows are indices >= 0: read unsigned, so that the loaded register is the value and nothing
     // has to wait for the load before the next step uses it
-    return (int)((const uint16_t*)p.lut)[max(-p.R, min(p.R, r)) + p.R];
+    const int d = (int)((const uint16_t*)p.lut)[max(-p.R, min(p.R, r_tab)) + p.R];
+    r_tab -= 32;
+    return d;
   };
   const uint32_t ek_lds = lds0 + (uint32_t)(EK - smem) + wave_kb, eq_lds = lds0 + (uint32_t)(EQ - smem) + wave_kb;
   // table rows are addressed with 32-bit byte offsets from the head's first row (the host checks that a row stride
   // stays under 2^24 bytes and the whole table under 2^31)
   const uint32_t pk_rowb = (uint32_t)(p.pk_sr * 2), pq_rowb = (uint32_t)(p.pq_sr * 2);
-  auto batch_dma = [&](int delta, int batch) __attribute__((always_inline)) {
-    const uint32_t seg = (uint32_t)(batch % kRingBatches) * (32 * kRowBytes);
-    if constexpr (C2P) dma16s(pkb, __umul24((uint32_t)delta, pk_rowb) + chunk_off, ek_lds + seg);
-    if constexpr (P2C) dma16s(pqb, __umul24((uint32_t)delta, pq_rowb) + chunk_off, eq_lds + seg);
+  auto batch_dma = [&](int delta, int slot) __attribute__((always_inline)) {
+    const uint32_t seg = (uint32_t)slot * (32 * kRowBytes);
+    if constexpr (C2P) dma16sn(pkb, __umul24((uint32_t)delta, pk_rowb) + chunk_off, ek_lds + seg);
+    if constexpr (P2C) dma16sn(pqb, __umul24((uint32_t)delta, pq_rowb) + chunk_off, eq_lds + seg);
   };
 
   f32x16 o_acc[DBLKS];
@@ -208,15 +254,18 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
 #pragma unroll
     for (int v = 0; v < 16; ++v) o_acc[d][v] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
+  // the content product's accumulator starts from minus the row's reference point (0 before the row has one)
+  f32x16 negm;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) negm[v] = 0.f;
 
   // ---- per-lane constants ------------------------------------------------------------------------------
-  // A row (block bk, lane li) of the wave's sub-tile at step k: r = iw0 - 32s - 31 + 32bk + li, i.e.
-  // u = 158 + 32k - 32*(wave + bk) - li; its slot keeps the low five bits of 158 - li for ever.
-  const int fr = ring_f(158 - li);
-  uint32_t rlx[KS];  // chunk 2s + g of the row sits in slot (2s) ^ g ^ f
+  // MFMA row m = li of a position product is row 31 - li of its batch; chunk 2x + g of that row sits in
+  // slot (2x) ^ g ^ f(row).
+  const int arow = 31 - li, fr = ring_f(arow);
+  uint32_t ra[KS];
 #pragma unroll
-  for (int s = 0; s < KS; ++s) rlx[s] = ((g ^ fr) * 16) ^ (32 * s);
-  int slot0 = 158 - li - 32 * wave;  // block 0 at step 0: u = 158 - li - 32*wave >= 31
+  for (int x = 0; x < KS; ++x) ra[x] = (uint32_t)(arow * kRowBytes) + (uint32_t)((((g ^ fr) * 16)) ^ (32 * x));
   uint32_t klx[KS], vlx[4];  // K fragment rows li; V^T operand (c, d-block db, half h): row 16c + 8h + 4*(grp/2) + s16/4,
                              // 8-byte unit 8db + 4*(grp%2) + s16%4, i.e. chunk ^ f = lane part ^ (4db) ^ (2h)
   {
@@ -229,37 +278,50 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
       vlx[x] = vlane ^ (64 * (x >> 1) ^ 32 * (x & 1));
     }
   }
-  // scratch: C[i = li][rr] with rr = r - r_lo in 0..63; element (jj, i = li) wants C[li][li + 31 - jj], i.e. only the
-  // band rr in [li, li + 31] of row li is ever read.  Of the two columns rr = c and c + 32 (the same accumulator
-  // register of block 0 and of block 1) a lane therefore needs exactly one, c if c >= li: it picks that one
-  // (the lanes that pick block 0 are a constant of the register: a scalar mask), rounds to the 16-bit type and
-  // writes 32 columns, position rr mod 32, as four 8-byte groups instead of 64 columns in fp32 -- LDS writes are
-  // what a step pays most for.  Positions 32..35 repeat 0..3, so that a run of four positions never wraps.
-  // K's rows sit in LDS with the low two bits of the row index inverted, so MFMA row m = 8q + 4g + e of
-  // the content product is key jj = 8q + 4g + 3 - e: the four C elements a lane adds to consecutive
-  // accumulator registers are the run of positions that starts at (li + 28 - 8q - 4g) mod 32.
-  uint16_t* c_wrp = scr + li * kScrW + 4 * g;  // row = this lane's MFMA column; group q4 at + 8 q4
-  // (read through volatile pointers: four neighbouring 16-bit reads must stay four instructions -- fused into
-  // one 8-byte read at an address aligned to two bytes only, they would be served lane by lane)
-  LDS_AS const volatile uint16_t* c_rd[4];
+  // scratch: row li = this lane's query, 64 columns in two halves: the block a step contracts (its block 0, columns
+  // rr = 0..31 of the step) goes to half PAR = step parity, and the other half still holds the block the step before
+  // wrote there, which is this step's block 1 (rr = 32..63).  Element (jj, i = li) wants rr = li + 32 - jj, i.e. column
+  // (32 PAR + li + 32 - jj) mod 64.  K's rows sit in LDS with the low two bits of the row index inverted, so MFMA
+  // row m = 8q + 4g + e of the content product is key jj = 8q + 4g + 3 - e: the four C elements a lane adds to
+  // consecutive accumulator registers are the run of columns that starts at (32 PAR + li + 29 - 8q - 4g) mod 64; columns
+  // 64..67 repeat 0..3, so that a run never wraps.
+  const uint32_t scr0 = lds0 + (uint32_t)(scr_raw - smem) + (uint32_t)wave * (kScrElems * 2) + (uint32_t)li * (kScrPitch * 2);
+  uint16_t* c_wr = (uint16_t*)scr_raw + wave * kScrElems + li * kScrPitch + 4 * g;  // group q4 of half h at + 32 h + 8 q4
+  uint16_t* c_dup = g == 0 ? c_wr + 64 : c_wr;  // where columns 0..3 go once more (the lanes that hold 4..7 write those again)
+  uint32_t c_rd[2][4];
 #pragma unroll
-  for (int q = 0; q < 4; ++q)
-    c_rd[q] = (LDS_AS const volatile uint16_t*)(scr + li * kScrW + ((li + 28 - 8 * q - 4 * g) & 31));
+  for (int par = 0; par < 2; ++par)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) c_rd[par][q] = scr0 + 2u * (uint32_t)((32 * par + li + 29 - 8 * q - 4 * g) & 63);
+  const int xl = li + 4 * g;  // P: a source lane (n = li) of register v hands out block 1 where n + jj < 32
 
   // Block 1 of a step holds the rows that were block 0 of the step before, and a step reads only its
   // new block 0 from the rings.  C[r][i] does not depend on the keys, so C's block 1 IS the block 0 the
-  // step before computed: its accumulator is kept (two that swap roles; the loop is unrolled over the
-  // parity) and only block 0 is contracted.  P depends on the step's keys: there the A operands are
-  // kept instead, in two buffers that swap roles the same way.
+  // step before contracted: it is still in the scratch.  P depends on the step's keys: there the A operands
+  // are kept, in two buffers that swap roles with the step's parity.
   qfrag ac[C2P ? KS : 1], aq[2][P2C ? KS : 1];
-  f32x16 ckeep[2];
   auto ring_read = [&](int buf, int slot) __attribute__((always_inline)) {
+    const uint32_t boff = (uint32_t)slot * (32 * kRowBytes);
 #pragma unroll
     for (int x = 0; x < KS; ++x) {
-      if constexpr (C2P) ac[x] = QT::load(EK + slot * kRowBytes + rlx[x]);
-      if constexpr (P2C) aq[buf][x] = QT::load(EQ + slot * kRowBytes + rlx[x]);
+      if constexpr (C2P) ac[x] = QT::load(EK + boff + ra[x]);
+      if constexpr (P2C) aq[buf][x] = QT::load(EQ + boff + ra[x]);
     }
   };
+  f32x16 zero;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) zero[v] = 0.f;
+  // the block in cacc, rounded, to half `half` of the scratch
+  auto c_store = [&](const f32x16& cacc, int half) __attribute__((always_inline)) {
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {  // C[i = li][8*q4 + 4*g + 0..3]
+      const typename QT::scratch4 packed = QT::pack4(f32x4{cacc[4 * q4], cacc[4 * q4 + 1], cacc[4 * q4 + 2], cacc[4 * q4 + 3]});
+      *(typename QT::scratch4*)(c_wr + 32 * half + 8 * q4) = packed;
+      if (half == 0 && q4 == 0) *(typename QT::scratch4*)c_dup = packed;
+    }
+  };
+  int slot_rd = 4 - wave;  // ring slot of this wave's block 0
+  int slot_dma = 0;        // ring slot the step's loads fill
   // ---- prologue: step 0's K and ring batches 0..4 on their way to LDS -------------------------------------
   // All table values first, then all rows: the loads of one kind are in flight together.
   if (n_steps > 0) {
@@ -267,7 +329,7 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
     v_dma(s0, 0);
     int d0[6];
 #pragma unroll
-    for (int bt = 0; bt < 6; ++bt) d0[bt] = batch_delta(bt);
+    for (int bt = 0; bt < 6; ++bt) d0[bt] = batch_delta();
     // (taken here, all at once: the compiler, which does not count the direct loads, would otherwise wait for
     // each value at its use, behind all the direct loads issued before it)
 #pragma unroll
@@ -277,22 +339,18 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
     dnext = d0[5];
     wait_vmcnt<0>();
     __syncthreads();  // the prologue's ring rows
-    ring_read(1, slot0 >= 32 ? slot0 - 32 : slot0 + (kRingRows - 32));  // block 1 of step 0
+    ring_read(1, 3 - wave);  // block 1 of step 0
     if constexpr (C2P) {
+      f32x16 c1;
 #pragma unroll
-      for (int x = 0; x < KS; ++x) {
-        if (x == 0) {
-#pragma unroll
-          for (int v = 0; v < 16; ++v) ckeep[1][v] = 0.f;
-        }
-        ckeep[1] = QT::mma(ac[x], qf[x], ckeep[1]);
-      }
+      for (int x = 0; x < KS; ++x) c1 = QT::mma(ac[x], qf[x], x == 0 ? zero : c1);
+      c_store(c1, 1);
     }
   }
 
   auto step = [&](auto mask_tag, auto par_tag, int k) __attribute__((always_inline)) {
     constexpr bool MASK = decltype(mask_tag)::value;
-    constexpr int PAR = decltype(par_tag)::value;  // buffer of this step's block 0
+    constexpr int PAR = decltype(par_tag)::value;  // parity of the step: its K / V buffers, its half of the scratch
     const int s = s0 + k;
     const int j0 = s * kStep;
     // This wave's direct loads of the step before -- K, V and the new ring batch of this step -- have landed;
@@ -307,88 +365,61 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
     // what the last steps fetch), so every step issues the same loads and the one wait above covers them.
     k_dma(s + 1, PAR ^ 1);
     v_dma(s + 1, PAR ^ 1);
-    batch_dma(dnext, k + 5);
-    __builtin_amdgcn_sched_barrier(0);  // the table load stays behind the direct loads
-    dnext = batch_delta(k + 6);         // used a step from now
+    batch_dma(dnext, slot_dma);          // batch k + 5 in place of batch k
+    __builtin_amdgcn_sched_barrier(0);   // the table load stays behind the direct loads
+    dnext = batch_delta();               // of batch k + 6, used a step from now
     // ---- operands of the step out of LDS ------------------------------------------------------------------
     qfrag kf[KS];
 #pragma unroll
     for (int x = 0; x < KS; ++x) kf[x] = QT::load(Ks + PAR * NCfg::K_BYTES + klx[x]);
-    ring_read(PAR, slot0);
-    // ---- the five products -------------------------------------------------------------------------------
-    // C, C to the scratch and its skewed diagonal back as the initial value of the content product's
-    // accumulator; P runs while those reads are in flight (the scheduling fence keeps it behind them).
-    // The LDS unit runs one wave's operations in order, so the reads of C are served before the writes
-    // of the next step; only the compiler needs the fences.
-    f32x16 sacc;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) sacc[v] = 0.f;
-    const f32x16 zero = sacc;
-    f32x16 pacc[2];
-    // The sixteen MFMAs of the four score products first, in two pairs of chains that alternate (no MFMA waits for
-    // its own previous link): C with P's block 1 (whose operands are this step's keys and the rows kept from the
-    // step before), then P's block 0 with the content product.  What follows C -- the pick, the scratch round trip --
-    // runs under the second pair.
+    ring_read(PAR, slot_rd);
+    // ---- the sixteen MFMAs of the four score products, in two pairs of chains that alternate (no MFMA waits for
+    // its own previous link): C's new block with P's block 1 (whose operands are this step's keys and the rows
+    // kept from the step before), then P's block 0 with the content product.  What follows C -- the write to the
+    // scratch and the reads of the skewed band -- runs under the second pair.
+    f32x16 sacc, cnew, pacc[2];
 #pragma unroll
     for (int x = 0; x < KS; ++x) {
-      if constexpr (C2P) ckeep[PAR] = QT::mma(ac[x], qf[x], x == 0 ? zero : ckeep[PAR]);
+      if constexpr (C2P) cnew = QT::mma(ac[x], qf[x], x == 0 ? zero : cnew);
       if constexpr (P2C) pacc[1] = QT::mma(kf[x], aq[PAR ^ 1][x], x == 0 ? zero : pacc[1]);
     }
 #pragma unroll
     for (int x = 0; x < KS; ++x) {
       if constexpr (P2C) pacc[0] = QT::mma(kf[x], aq[PAR][x], x == 0 ? zero : pacc[0]);
-      sacc = QT::mma(kf[x], qf[x], sacc);
+      sacc = QT::mma(kf[x], qf[x], x == 0 ? negm : sacc);
     }
-    uint16_t craw[16];
+    float cband[16];
     if constexpr (C2P) {
-      const f32x16(&cacc)[2] = ckeep;  // block bk of this step sits in ckeep[PAR ^ bk]
+      c_store(cnew, PAR);
+      wave_lds_fence();  // the LDS unit runs one wave's operations in order; this keeps the compiler from moving them
 #pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {  // C[i = li][(32*bk) + 8*q4 + 4*g + 0..3], block 0 where that column is >= li
-        f32x4 pick;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int c0 = 8 * q4 + e, c1 = c0 + 4;  // the column in the lanes g = 0 / g = 1
-          const uint64_t mask = ((2ull << c0) - 1ull) | ((c1 >= 31 ? 0xffffffffull : (2ull << c1) - 1ull) << 32);
-          pick[e] = __builtin_amdgcn_inverse_ballot_w64(mask) ? cacc[PAR][4 * q4 + e] : cacc[PAR ^ 1][4 * q4 + e];
-        }
-        const typename QT::scratch4 packed = QT::pack4(pick);
-        *(typename QT::scratch4*)(c_wrp + 8 * q4) = packed;
-        if (q4 == 0) *(typename QT::scratch4*)(c_wrp + 32) = packed;
+      for (int q = 0; q < 4; ++q) {
+        cband[4 * q + 0] = lds_elem_f32<QT, 0>(c_rd[PAR][q]);
+        cband[4 * q + 1] = lds_elem_f32<QT, 2>(c_rd[PAR][q]);
+        cband[4 * q + 2] = lds_elem_f32<QT, 4>(c_rd[PAR][q]);
+        cband[4 * q + 3] = lds_elem_f32<QT, 6>(c_rd[PAR][q]);
       }
-      wave_lds_fence();
-#pragma unroll
-      for (int v = 0; v < 16; ++v) craw[v] = c_rd[v >> 2][v & 3];
       wave_lds_fence();
     }
     // P with the keys as MFMA rows, like the content product: register v of lane (g, n) holds
-    // P[jj(v, g)][32 bk + n], and element (jj, i = li) wants column li + 31 - jj of that row, i.e. the same
-    // register of another lane of its own half.  Each source lane is read by exactly one lane, which
-    // wants block 1 from it if n + jj < 31 and block 0 otherwise: the source picks, one lane permutation
-    // per register moves it.
+    // P[jj(v, g)][32 bk + n], and element (jj, i = li) wants column li + 32 - jj of that row, i.e. the same
+    // register of another lane of its own half: lane (li - jj) mod 32, block 1 if li >= jj.  Each source lane is
+    // read by exactly one lane, which wants block 1 from it if n + jj < 32 and block 0 otherwise: the source
+    // picks (a compare of its lane constant with a constant of the register), and a rotation of each half-wave
+    // by 32 - jj moves it: ds_swizzle in rotate mode, no address registers; the halves differ by 4 in jj, so each
+    // half runs its own sixteen under its half of the execution mask.
     float px[16];
     if constexpr (P2C) {
-      // Source lane (g, n) of register v (key jj = 4g + c) is read by lane (g, (n - rot) mod 32), which wants
-      // block 1 from it if n + jj < 31 and block 0 otherwise: which lanes pick block 1 is a constant of the
-      // register, so the select takes its mask from a scalar pair.  The move itself is a rotation of each
-      // half-wave by a constant, rot = 31 - jj: ds_swizzle in rotate mode (offset 0xC000 | rot << 5), no
-      // address registers; the halves differ by 4 in jj, so each half runs its own sixteen under its
-      // half of the execution mask.
       float xs[16];
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int c = 8 * (v >> 2) + 3 - (v & 3);  // jj - 4g
-        const uint64_t mask = (uint64_t)((1u << (31 - c)) - 1u) | ((uint64_t)(c < 27 ? (1u << (27 - c)) - 1u : 0u) << 32);
-        xs[v] = __builtin_amdgcn_inverse_ballot_w64(mask) ? pacc[1][v] : pacc[0][v];
+        xs[v] = (xl < 32 - c) ? pacc[1][v] : pacc[0][v];
       }
       if (g == 0)
-        rotate16<31>(xs, px, std::make_integer_sequence<int, 16>{});
+        rotate16<32>(xs, px, std::make_integer_sequence<int, 16>{});
       else
-        rotate16<27>(xs, px, std::make_integer_sequence<int, 16>{});
-    }
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      if constexpr (C2P) sacc[v] += QT::scratch_to_f32(craw[v]);
-      if constexpr (P2C) sacc[v] += px[v];
+        rotate16<28>(xs, px, std::make_integer_sequence<int, 16>{});
     }
     // V^T operands requested here, ahead of the soft-max, so that the four MFMAs at the end of the step find them
     vfrag vfr[2][DBLKS];
@@ -401,6 +432,20 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
         vfr[c][d] = __builtin_bit_cast(vfrag, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
       }
     __builtin_amdgcn_sched_barrier(0);
+    // one wait for the band of C and the rotated P (issued as asm: the compiler keeps no count of them)
+    if constexpr (C2P || P2C) {
+      lds_wait_all();
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        if constexpr (C2P && std::is_same<QT, Bf16Tr>::value) asm volatile("" : "+v"(cband[v]));
+        if constexpr (P2C) asm volatile("" : "+v"(px[v]));
+      }
+    }
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      if constexpr (C2P) sacc[v] += cband[v];
+      if constexpr (P2C) sacc[v] = __builtin_fmaf(px[v], x_scale, sacc[v]);
+    }
     // ---- mask, online soft-max in base 2, O^T += V^T P^T ---------------------------------------------------
     if constexpr (MASK) {
 #pragma unroll
@@ -409,52 +454,59 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
         if (j >= Lb || (p.causal && j > i)) sacc[v] = -INFINITY;
       }
     }
-    // The probabilities are formed against the row's current reference point first; the half-row sum of a
-    // step bounds its largest one, so while it stays under 2^kLazyTau nothing has to move and no maximum is
-    // taken.  Otherwise (or before a row has a reference point) the wave takes the maximum, moves the
-    // reference points of the rows that need it and forms the probabilities again.
+    // sacc = score - reference point.  The probabilities are formed first; the half-row sum of a step bounds its
+    // largest one, so while it stays under 2^kLazyTau nothing has to move and no maximum is taken.  Otherwise (or
+    // before a row has a reference point) the wave takes the maximum, moves the reference points of the rows that
+    // need it, shifts the step's scores and forms the probabilities again.
     vfrag pf[2];
     float l_blk = 0.f;
-    auto probs = [&](float off) __attribute__((always_inline)) {
+    auto probs = [&]() __attribute__((always_inline)) {
       l_blk = 0.f;
 #pragma unroll
       for (int c = 0; c < 2; ++c) {
         f32x8 pv;
 #pragma unroll
-        for (int e = 0; e < 8; ++e)  // the V^T operand takes the keys in ascending order
-          pv[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[8 * c + (e ^ 3)], x_scale, off));
+        for (int e = 0; e < 8; ++e) pv[e] = __builtin_amdgcn_exp2f(sacc[8 * c + (e ^ 3)]);  // the V^T operand takes the keys in ascending order
         pf[c] = VT::from_f32(pv);
         l_blk = sum8(pv, l_blk);
       }
     };
-    bool slow = __any(m_run == -INFINITY);
+    const bool first = m_run == -INFINITY;
+    bool slow = __any(first);
     if (!slow) {
-      probs(-m_run);
+      probs();
       slow = __any(!(l_blk <= 256.f));  // 2^kLazyTau; also true for an overflow
     }
     if (slow) {
       float mx = sacc[0];
 #pragma unroll
       for (int v = 1; v < 16; ++v) mx = fmaxf(mx, sacc[v]);
-      mx = wave_half_max(mx) * x_scale;  // x_scale > 0
-      if (__any(mx > m_run + kLazyTau)) {
-        const float m_new = (mx > m_run + kLazyTau) ? mx : m_run;
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // m_run = -inf before the first visible key: 0
+      mx = wave_half_max(mx);  // relative to the reference point (to 0 while the row has none)
+      const bool mv = first ? mx > -INFINITY : mx > kLazyTau;
+      if (__any(mv)) {
+        const float shift = mv ? mx : 0.f;
+        const float alpha = first ? 0.f : __builtin_amdgcn_exp2f(-shift);  // 1 where nothing moves
+        if (mv) m_run = (first ? 0.f : m_run) + shift;
         l_run *= alpha;
-        m_run = m_new;
 #pragma unroll
         for (int d = 0; d < DBLKS; ++d)
 #pragma unroll
           for (int v = 0; v < 16; ++v) o_acc[d][v] *= alpha;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) sacc[v] -= shift;
+        const float nm = m_run == -INFINITY ? 0.f : -m_run;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) negm[v] = nm;
       }
-      probs((MASK && m_run == -INFINITY) ? 0.f : -m_run);  // a row that has seen no visible key yet
+      probs();
     }
     l_run += l_blk;
 #pragma unroll
     for (int c = 0; c < 2; ++c)
 #pragma unroll
       for (int d = 0; d < DBLKS; ++d) o_acc[d] = VT::mma(vfr[c][d], pf[c], o_acc[d]);
-    slot0 = slot0 + 32 >= kRingRows ? slot0 + 32 - kRingRows : slot0 + 32;
+    slot_rd = slot_rd == kRingBatches - 1 ? 0 : slot_rd + 1;
+    slot_dma = slot_dma == kRingBatches - 1 ? 0 : slot_dma + 1;
   };
   {
     using T0 = std::integral_constant<int, 0>;
