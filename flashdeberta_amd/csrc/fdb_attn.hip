@@ -430,8 +430,8 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
 #pragma unroll
       for (int q2 = 0; q2 < 2; ++q2) {  // this wave's two 8-row groups of K and of V
         const uint32_t dst = lds0 + bufoff + (2 * wave + q2) * 1024;
-        dma16s(kt, dma_koff[q2], dst);
-        dma16s(vt, dma_voff[q2], dst + C::DMA_TILE);
+        dma16sn(kt, dma_koff[q2], dst);
+        dma16sn(vt, dma_voff[q2], dst + C::DMA_TILE);
       }
     } else {
 #pragma unroll
@@ -439,8 +439,8 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
         const uint32_t row = (uint32_t)min(16 * wave + 8 * q2 + (lane >> 3), last);
         const uint32_t c16 = ((lane & 7) ^ (4 * ((lane >> 4) & 1)) ^ (lane >> 5) ^ (2 * q2)) * 16;  // slot ^ f(row), unclamped row
         const uint32_t dst = lds0 + bufoff + (2 * wave + q2) * 1024;
-        dma16s(kt, row * k_rsb + c16, dst);
-        dma16s(vt, row * v_rsb + c16, dst + C::DMA_TILE);
+        dma16sn(kt, row * k_rsb + c16, dst);
+        dma16sn(vt, row * v_rsb + c16, dst + C::DMA_TILE);
       }
     }
   };

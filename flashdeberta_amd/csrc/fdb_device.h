@@ -311,6 +311,21 @@ __device__ __forceinline__ void dma16s(const void* base, uint32_t lane_off, uint
   asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\ts_mov_b32 m0, %0"
                : "=&s"(keep) : "v"(lane_off), "s"(sb), "s"(lb) : "memory");
 }
+// The same two loads with M0 set and left as it is: for kernels in which nothing else reads M0 (no other direct
+// load variant, no LDS-direct or message instructions), where saving and restoring it is two more scalar
+// instructions per load.
+__device__ __forceinline__ void dma16n(const void* g, uint32_t lds_base) {
+  const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(base) : "memory");
+}
+__device__ __forceinline__ void dma16sn(const void* base, uint32_t lane_off, uint32_t lds_base) {
+  const uint32_t lb = __builtin_amdgcn_readfirstlane(lds_base);
+  const uint64_t b64 = (uint64_t)(uintptr_t)base;
+  const uint32_t blo = __builtin_amdgcn_readfirstlane((uint32_t)b64), bhi = __builtin_amdgcn_readfirstlane((uint32_t)(b64 >> 32));
+  const uint64_t sb = ((uint64_t)bhi << 32) | blo;
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(lane_off), "s"(sb), "s"(lb) : "memory");
+}
+
 // Wait until at most N vector-memory loads of this wave are outstanding (loads complete in issue
 // order).  Issued through the builtin rather than asm, so that the compiler's own count of its
 // outstanding loads takes the wait into account and it does not wait a second time for a value

@@ -98,19 +98,6 @@ __device__ __forceinline__ float lds_elem_f32(uint32_t addr) {
 }
 __device__ __forceinline__ void lds_wait_all() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
-// The direct loads of this kernel: M0 is set and left (nothing else in the kernel reads it).
-__device__ __forceinline__ void dma16n(const void* g, uint32_t lds_base) {
-  const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(base) : "memory");
-}
-__device__ __forceinline__ void dma16sn(const void* base, uint32_t lane_off, uint32_t lds_base) {
-  const uint32_t lb = __builtin_amdgcn_readfirstlane(lds_base);
-  const uint64_t b64 = (uint64_t)(uintptr_t)base;
-  const uint32_t blo = __builtin_amdgcn_readfirstlane((uint32_t)b64), bhi = __builtin_amdgcn_readfirstlane((uint32_t)(b64 >> 32));
-  const uint64_t sb = ((uint64_t)bhi << 32) | blo;
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(lane_off), "s"(sb), "s"(lb) : "memory");
-}
-
 template <class QT, class VT, bool C2P, bool P2C>
 __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams p) {
   constexpr int D = 64, KS = 4, DBLKS = 2;
@@ -209,20 +196,20 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
   // A step inside the sequence: its first row travels as the scalar base of the load, this thread's place in the
   // tile as a 32-bit offset computed once.  Only a step that reaches past the end clamps its rows one by one.
   const uint32_t k_lane = (uint32_t)(srow ^ 3) * k_rsb + chunk_off, v_lane = (uint32_t)srow * v_rsb + chunk_off;
-  auto k_dma = [&](int s, int buf) __attribute__((always_inline)) {
+  auto k_dma = [&](int s, int buf, bool inside) __attribute__((always_inline)) {
     // LDS row srow holds key srow ^ 3 of the step (see the scratch reads below); rows past the end
     // re-read the last one, their scores are masked
     const uint32_t dst = lds0 + buf * NCfg::K_BYTES + wave_kb;
-    if ((s + 1) * kStep <= Lb) {
+    if (inside || (s + 1) * kStep <= Lb) {
       dma16sn(kb + (uint64_t)(uint32_t)(s * kStep) * k_rsb, k_lane, dst);
     } else {
       const int row = min(s * kStep + (srow ^ 3), Lb - 1);
       dma16n(kb + (uint64_t)(uint32_t)row * k_rsb + chunk_off, dst);
     }
   };
-  auto v_dma = [&](int s, int buf) __attribute__((always_inline)) {
+  auto v_dma = [&](int s, int buf, bool inside) __attribute__((always_inline)) {
     const uint32_t dst = lds0 + 2 * NCfg::K_BYTES + buf * NCfg::V_BYTES + wave_kb;
-    if ((s + 1) * kStep <= Lb) {
+    if (inside || (s + 1) * kStep <= Lb) {
       dma16sn(vb + (uint64_t)(uint32_t)(s * kStep) * v_rsb, v_lane, dst);
     } else {
       const int row = min(s * kStep + srow, Lb - 1);
@@ -265,7 +252,8 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
   const int arow = 31 - li, fr = ring_f(arow);
   uint32_t ra[KS];
 #pragma unroll
-  for (int x = 0; x < KS; ++x) ra[x] = (uint32_t)(arow * kRowBytes) + (uint32_t)((((g ^ fr) * 16)) ^ (32 * x));
+  for (int x = 0; x < KS; ++x)
+    ra[x] = lds0 + (uint32_t)((C2P ? EK : EQ) - smem) + (uint32_t)(arow * kRowBytes) + (uint32_t)((((g ^ fr) * 16)) ^ (32 * x));
   uint32_t klx[KS], vlx[4];  // K fragment rows li; V^T operand (c, d-block db, half h): row 16c + 8h + 4*(grp/2) + s16/4,
                              // 8-byte unit 8db + 4*(grp%2) + s16%4, i.e. chunk ^ f = lane part ^ (4db) ^ (2h)
   {
@@ -274,8 +262,8 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
     const uint32_t vlane = (4 * (grp >> 1) + (s16 >> 2)) * kRowBytes + slotl * 16 + (s16 & 1) * 8;
 #pragma unroll
     for (int x = 0; x < 4; ++x) {
-      klx[x] = (li * kRowBytes + ((g ^ ring_f(li)) * 16)) ^ (32 * x);
-      vlx[x] = vlane ^ (64 * (x >> 1) ^ 32 * (x & 1));
+      klx[x] = lds0 + (uint32_t)(Ks - smem) + ((li * kRowBytes + ((g ^ ring_f(li)) * 16)) ^ (32 * x));  // absolute LDS addresses:
+      vlx[x] = lds0 + (uint32_t)(Vs - smem) + (vlane ^ (64 * (x >> 1) ^ 32 * (x & 1)));                  // buffer and block are immediates
     }
   }
   // scratch: row li = this lane's query, 64 columns in two halves: the block a step contracts (its block 0, columns
@@ -304,8 +292,8 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
     const uint32_t boff = (uint32_t)slot * (32 * kRowBytes);
 #pragma unroll
     for (int x = 0; x < KS; ++x) {
-      if constexpr (C2P) ac[x] = QT::load(EK + boff + ra[x]);
-      if constexpr (P2C) aq[buf][x] = QT::load(EQ + boff + ra[x]);
+      if constexpr (C2P) ac[x] = *(LDS_AS const qfrag*)(uintptr_t)(ra[x] + boff);
+      if constexpr (P2C) aq[buf][x] = *(LDS_AS const qfrag*)(uintptr_t)(ra[x] + boff + (C2P ? NCfg::RING_BYTES : 0));
     }
   };
   f32x16 zero;
@@ -325,8 +313,8 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
   // ---- prologue: step 0's K and ring batches 0..4 on their way to LDS -------------------------------------
   // All table values first, then all rows: the loads of one kind are in flight together.
   if (n_steps > 0) {
-    k_dma(s0, 0);  // K and V need no table value: on their way while the table is read
-    v_dma(s0, 0);
+    k_dma(s0, 0, false);  // K and V need no table value: on their way while the table is read
+    v_dma(s0, 0, false);
     int d0[6];
 #pragma unroll
     for (int bt = 0; bt < 6; ++bt) d0[bt] = batch_delta();
@@ -348,9 +336,10 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
     }
   }
 
-  auto step = [&](auto mask_tag, auto par_tag, int k) __attribute__((always_inline)) {
+  auto step = [&](auto mask_tag, auto par_tag, auto next_tag, int k) __attribute__((always_inline)) {
     constexpr bool MASK = decltype(mask_tag)::value;
     constexpr int PAR = decltype(par_tag)::value;  // parity of the step: its K / V buffers, its half of the scratch
+    constexpr bool NEXT_INSIDE = decltype(next_tag)::value;  // the next step's keys all lie inside the sequence
     const int s = s0 + k;
     const int j0 = s * kStep;
     // This wave's direct loads of the step before -- K, V and the new ring batch of this step -- have landed;
@@ -363,15 +352,15 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
     // ---- staging for the next step, straight into LDS ----------------------------------------------------------
     // It runs unconditionally, past the last step too (row and table indices are clamped, and nobody reads
     // what the last steps fetch), so every step issues the same loads and the one wait above covers them.
-    k_dma(s + 1, PAR ^ 1);
-    v_dma(s + 1, PAR ^ 1);
+    k_dma(s + 1, PAR ^ 1, NEXT_INSIDE);
+    v_dma(s + 1, PAR ^ 1, NEXT_INSIDE);
     batch_dma(dnext, slot_dma);          // batch k + 5 in place of batch k
     __builtin_amdgcn_sched_barrier(0);   // the table load stays behind the direct loads
     dnext = batch_delta();               // of batch k + 6, used a step from now
     // ---- operands of the step out of LDS ------------------------------------------------------------------
     qfrag kf[KS];
 #pragma unroll
-    for (int x = 0; x < KS; ++x) kf[x] = QT::load(Ks + PAR * NCfg::K_BYTES + klx[x]);
+    for (int x = 0; x < KS; ++x) kf[x] = *(LDS_AS const qfrag*)(uintptr_t)(klx[x] + PAR * NCfg::K_BYTES);
     ring_read(PAR, slot_rd);
     // ---- the sixteen MFMAs of the four score products, in two pairs of chains that alternate (no MFMA waits for
     // its own previous link): C's new block with P's block 1 (whose operands are this step's keys and the rows
@@ -427,8 +416,8 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
     for (int c = 0; c < 2; ++c)
 #pragma unroll
       for (int d = 0; d < DBLKS; ++d) {
-        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(Vs + PAR * NCfg::V_BYTES + vlx[2 * d] + 2048 * c));
-        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(Vs + PAR * NCfg::V_BYTES + vlx[2 * d + 1] + 2048 * c + 1024));
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(uintptr_t)(vlx[2 * d] + PAR * NCfg::V_BYTES + 2048 * c));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(uintptr_t)(vlx[2 * d + 1] + PAR * NCfg::V_BYTES + 2048 * c + 1024));
         vfr[c][d] = __builtin_bit_cast(vfrag, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
       }
     __builtin_amdgcn_sched_barrier(0);
@@ -511,26 +500,34 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
   {
     using T0 = std::integral_constant<int, 0>;
     using T1 = std::integral_constant<int, 1>;
+    using Y = std::true_type;
+    using N = std::false_type;
     int k = 0;
+    // the bulk: unmasked steps whose successor is unmasked too (its rows need no clamping)
+#pragma unroll 1
+    for (; k + 2 < n_full; k += 2) {
+      step(N{}, T0{}, Y{}, k);
+      step(N{}, T1{}, Y{}, k + 1);
+    }
 #pragma unroll 1
     for (; k + 1 < n_full; k += 2) {
-      step(std::false_type{}, T0{}, k);
-      step(std::false_type{}, T1{}, k + 1);
+      step(N{}, T0{}, N{}, k);
+      step(N{}, T1{}, N{}, k + 1);
     }
     if (k < n_full) {
-      step(std::false_type{}, T0{}, k);
+      step(N{}, T0{}, N{}, k);
       ++k;
     }
     if ((k & 1) && k < n_steps) {
-      step(std::true_type{}, T1{}, k);
+      step(Y{}, T1{}, N{}, k);
       ++k;
     }
 #pragma unroll 1
     for (; k + 1 < n_steps; k += 2) {
-      step(std::true_type{}, T0{}, k);
-      step(std::true_type{}, T1{}, k + 1);
+      step(Y{}, T0{}, N{}, k);
+      step(Y{}, T1{}, N{}, k + 1);
     }
-    if (k < n_steps) step(std::true_type{}, T0{}, k);
+    if (k < n_steps) step(Y{}, T0{}, N{}, k);
   }
   wait_vmcnt<0>();  // the last step's direct loads: none may still be writing LDS when the workgroup ends
 
