@@ -152,6 +152,29 @@ int near_parts_wanted(const fdb_attn_args* a) {
   return best;
 }
 
+// Does the call take the far / near pair of launches (otherwise one kernel walks every key tile)?
+bool takes_pair(const fdb_attn_args* a) {
+  return (a->pos_key || a->pos_query) && a->lse && pair_supported(a->dtype, a->head_dim);
+}
+
+// One-kernel mode: workgroups per query tile.  When the query tiles leave most of the GPU idle (one workgroup per CU
+// is what the larger instantiations of that kernel reach), the key tiles of a query tile are shared out among up to
+// FDB_MAX_FAR_PARTS workgroups, each keeping at least two; a merge launch follows.  far_splits overrides it.
+int key_parts_wanted(const fdb_attn_args* a) {
+  if (takes_pair(a)) return 1;
+  const int32_t typical = a->cu_seqlens ? a->total_tokens / a->batch : a->max_seqlen;
+  const int n64 = (typical + FDB_BN - 1) / FDB_BN;
+  // a causal query tile's keys end at its own rows: a share could hold no visible key for some of them, a case the
+  // tiles' soft-max does not meet otherwise (a row's first tile always shows it a key) and is not written for
+  if (a->causal) return 1;
+  if (a->far_splits > 0) return a->far_splits;
+  const int64_t wgs = query_tiles(a) * a->heads, slots = cu_count();
+  int n = (int)(slots / wgs);
+  if (n > FDB_MAX_FAR_PARTS) n = FDB_MAX_FAR_PARTS;
+  while (n > 1 && n64 / n < 2) --n;
+  return n > 1 ? n : 1;
+}
+
 int64_t lse_rows(const fdb_attn_args* a) {
   return a->cu_seqlens ? (int64_t)a->total_tokens : (int64_t)a->batch * a->max_seqlen;
 }
@@ -298,6 +321,10 @@ int fdb_attn_check(const fdb_attn_args* a) {
 
 int64_t fdb_attn_workspace_bytes(const fdb_attn_args* a) {
   if (fdb_attn_check(a) != FDB_OK) return 0;
+  if (!takes_pair(a)) {
+    const int parts = key_parts_wanted(a);
+    return parts > 1 ? parts * far_part_bytes(a) : 0;
+  }
   const int near = near_parts_wanted(a);
   return (far_parts_wanted(a) - 1 + (near > 1 ? near : 0)) * far_part_bytes(a);
 }
@@ -373,7 +400,20 @@ int attn_fwd_impl(const fdb_attn_args* a, int launch_mask, void* stream) {
     return fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, FDB_MODE_NEAR_RING, stream);
   }
   if (launch_mask != 0) return FDB_ERR_UNSUPPORTED;  // a single kernel has no parts
-  return fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, FDB_MODE_FUSED, stream);
+  // as many shares of the keys as wanted and as the workspace holds partial results for
+  p.key_parts = key_parts_wanted(a);
+  const int64_t slots_have = a->workspace ? a->workspace_bytes / far_part_bytes(a) : 0;
+  if (p.key_parts > slots_have) p.key_parts = slots_have >= 2 ? (int)slots_have : 1;
+  if (p.key_parts <= 1) {
+    p.key_parts = 1;
+    return fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, FDB_MODE_FUSED, stream);
+  }
+  p.ws_slots = p.key_parts;
+  p.ws = (char*)a->workspace;
+  p.ws_rows = lse_rows(a);
+  const int rc_attn = fdb_launch_attn(p, a->dtype, a->head_dim, (int)grid_x, FDB_MODE_FUSED, stream);
+  if (rc_attn != 0) return rc_attn;
+  return fdb_launch_merge_parts(p, a->dtype, a->head_dim, stream);
 }
 
 }  // namespace

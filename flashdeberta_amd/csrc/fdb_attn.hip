@@ -223,7 +223,10 @@ constexpr int min_blocks() {
   const int lds = Cfg<QT, VT, D>::lds_bytes_mode(MODE, C2P, P2C);
   if (MODE == kFarOnly) return 3;  // the far zones need the shifted query and the per-row constants on top of the plain kernel
   if (MODE == kNearRing) return 2;  // one workgroup fits a CU; the bound keeps every value in the 256 registers VALU code can read
-  return lds <= 40 * 1024 ? 3 : lds <= 80 * 1024 ? 2 : 1;  // three: 170 registers, the plain loop's working set without spills
+  // three: 170 registers, the plain loop's working set at head_dim <= 64; head_dim 128 doubles the output accumulators
+  // and the query fragments: two workgroups (256 registers) for the 16-bit types, one (512) for fp32
+  if (D >= 128) return QT::SZ == 4 ? 1 : (lds <= 80 * 1024 ? 2 : 1);
+  return (lds <= 40 * 1024 && QT::SZ < 4) ? 3 : lds <= 80 * 1024 ? 2 : 1;  // fp32 fragments are twice the registers
 }
 
 template <class QT, class VT, int D, bool FP8, bool C2P, bool P2C, int MODE>
@@ -367,8 +370,18 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
   // The far tiles of this workgroup: [zl0, zl1) left of the near range and [zr0, zr1) right of it.  A
   // far-only run may be split over p.far_parts workgroups per query tile (blockIdx.y), each taking an equal
   // share of the far tiles in walking order and leaving a partial result of its own.
-  int zl0 = 0, zl1 = t_near0, zr0 = t_near1, zr1 = n_tiles;
-  const int part = FAR_ONLY ? (int)blockIdx.y : 0;
+  // One-kernel mode with p.key_parts > 1: this workgroup walks its share [t_lo, t_hi) of the key tiles only, and the
+  // three ranges are cut to it.
+  const int part = (FAR_ONLY || (MODE == kFused && p.key_parts > 1)) ? (int)blockIdx.y : 0;
+  int t_lo = 0, t_hi = n_tiles;
+  if (MODE == kFused && p.key_parts > 1) {
+    t_lo = (int)((int64_t)n_tiles * part / p.key_parts);
+    t_hi = (int)((int64_t)n_tiles * (part + 1) / p.key_parts);
+    const int n0 = t_near0, n1 = t_near1;
+    t_near0 = min(max(n0, t_lo), t_hi);
+    t_near1 = min(max(n1, t_lo), t_hi);
+  }
+  int zl0 = t_lo, zl1 = t_near0, zr0 = t_near1, zr1 = t_hi;
   if (FAR_ONLY && p.far_parts > 1) {
     const int n_far = t_near0 + (n_tiles - t_near1);
     const int o_lo = (int)((int64_t)n_far * part / p.far_parts), o_hi = (int)((int64_t)n_far * (part + 1) / p.far_parts);
@@ -761,7 +774,11 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
     // Row offsets (bytes) into K_r / Q_r of the A rows this lane feeds to the position products
     // of one tile; looked up through the table one tile ahead so that the row loads of a tile
     // never wait for the table.
-    int64_t off_c[3], off_p[3];
+    // Where the A rows of all six blocks would not fit the registers (fp32; head_dim 128 in a 16-bit type), they are
+    // fetched block by block, one block ahead of the MFMAs that use them, and the offsets of the next tile go to a set
+    // of their own until this tile's last block has been requested.
+    constexpr bool LAZY_A = D >= 128 || C::KSTEPS * (int)(sizeof(qfrag) / 4) >= 32;
+    int64_t off_c[3], off_p[3], offn_c[3], offn_p[3];
     auto lookup = [&](int t) __attribute__((always_inline)) {
       const int j0 = t * FDB_BN;
       if constexpr (C2P) {
@@ -769,7 +786,7 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
 #pragma unroll
         for (int blk = 0; blk < 3; ++blk) {
           const int r = max(-p.R, min(p.R, r_lo + 32 * blk + li));
-          off_c[blk] = (int64_t)p.lut[r + p.R] * p.pk_sr * QT::SZ + 8 * g * QT::SZ;
+          offn_c[blk] = (int64_t)p.lut[r + p.R] * p.pk_sr * QT::SZ + 8 * g * QT::SZ;
         }
       }
       if constexpr (P2C) {
@@ -778,7 +795,7 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
         for (int n = 0; n < 3; ++n) {
           const int wblk = (wave * 3 + n) >> 1;
           const int r = max(-p.R, min(p.R, r_lo + 32 * wblk + li));
-          off_p[n] = (int64_t)p.lut[r + p.R] * p.pq_sr * QT::SZ + 8 * g * QT::SZ;
+          offn_p[n] = (int64_t)p.lut[r + p.R] * p.pq_sr * QT::SZ + 8 * g * QT::SZ;
         }
       }
     };
@@ -787,18 +804,29 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
     constexpr bool MASK = decltype(mask_tag)::value;
     for (int t = t0; t < t1; ++t) {
       const int j0 = t * FDB_BN;
-      qfrag ac[C2P ? 3 : 1][C::KSTEPS], ap[P2C ? 3 : 1][C::KSTEPS];
-      if constexpr (C2P) {
 #pragma unroll
-        for (int blk = 0; blk < 3; ++blk)
-#pragma unroll
-          for (int s = 0; s < C::KSTEPS; ++s) ac[blk][s] = QT::load(pkb + off_c[blk] + 16 * s * QT::SZ);
+      for (int n = 0; n < 3; ++n) {
+        off_c[n] = offn_c[n];
+        off_p[n] = offn_p[n];
       }
-      if constexpr (P2C) {
+      constexpr int nC = C2P ? 3 : 0, nP = P2C ? 3 : 0, NB = nC + nP;
+      qfrag ac[(C2P && !LAZY_A) ? 3 : 1][C::KSTEPS], ap[(P2C && !LAZY_A) ? 3 : 1][C::KSTEPS], abuf[LAZY_A ? 2 : 1][C::KSTEPS];
+      auto load_blk = [&](int b, qfrag (&dst)[C::KSTEPS]) __attribute__((always_inline)) {  // block b of the tile: C's three, then P's
+        const char* base = b < nC ? pkb + off_c[b < nC ? b : 0] : pqb + off_p[b >= nC ? b - nC : 0];
 #pragma unroll
-        for (int n = 0; n < 3; ++n)
+        for (int s = 0; s < C::KSTEPS; ++s) dst[s] = QT::load(base + 16 * s * QT::SZ);
+      };
+      if constexpr (!LAZY_A) {
+        if constexpr (C2P) {
 #pragma unroll
-          for (int s = 0; s < C::KSTEPS; ++s) ap[n][s] = QT::load(pqb + off_p[n] + 16 * s * QT::SZ);
+          for (int blk = 0; blk < 3; ++blk) load_blk(blk, ac[blk]);
+        }
+        if constexpr (P2C) {
+#pragma unroll
+          for (int n = 0; n < 3; ++n) load_blk(nC + n, ap[n]);
+        }
+      } else {
+        load_blk(0, abuf[0]);
       }
       stage(t);
       if (t + 1 < t_near1) lookup(t + 1);
@@ -812,8 +840,11 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
           f32x16 acc;
 #pragma unroll
           for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+          if constexpr (LAZY_A) {
+            if (blk + 1 < NB) load_blk(blk + 1, abuf[(blk + 1) & 1]);
+          }
 #pragma unroll
-          for (int s = 0; s < C::KSTEPS; ++s) acc = QT::mma(ac[blk][s], qf[s], acc);
+          for (int s = 0; s < C::KSTEPS; ++s) acc = QT::mma(LAZY_A ? abuf[blk & 1][s] : ac[LAZY_A ? 0 : blk][s], qf[s], acc);
           if constexpr (FP8) acc *= c2p_mul;
 #pragma unroll
           for (int q4 = 0; q4 < 4; ++q4)
@@ -828,10 +859,13 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
           f32x16 acc;
 #pragma unroll
           for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+          if constexpr (LAZY_A) {
+            if (nC + n + 1 < NB) load_blk(nC + n + 1, abuf[(nC + n + 1) & 1]);
+          }
 #pragma unroll
           for (int s = 0; s < C::KSTEPS; ++s) {
             qfrag kf = QT::load(Ks + (jblk * 32 + li) * C::K_RS + (16 * s + 8 * g) * QT::SZ);
-            acc = QT::mma(ap[n][s], kf, acc);
+            acc = QT::mma(LAZY_A ? abuf[(nC + n) & 1][s] : ap[LAZY_A ? 0 : n][s], kf, acc);
           }
           if constexpr (FP8) acc *= p2c_mul;
           ST* dst0 = p2cS + (jblk * 32 + li) * kP2cStride + 32 * wblk + 4 * g;
@@ -941,6 +975,10 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
       orow = far_part_out(p, part, D * VT::SZ) + (tok * p.H + h) * (D * VT::SZ);
       lse_row = far_part_lse(p, part, D * VT::SZ);
     }
+    if (MODE == kFused && p.key_parts > 1) {  // every share's partial result goes to its workspace slot
+      orow = ws_slot_out(p, part, D * VT::SZ) + (tok * p.H + h) * (D * VT::SZ);
+      lse_row = ws_slot_lse(p, part, D * VT::SZ);
+    }
 #pragma unroll
     for (int d = 0; d < C::DBLKS; ++d)
 #pragma unroll
@@ -962,7 +1000,8 @@ int launch_one(const FdbKParams& p, int grid_x, hipStream_t stream) {
   static std::atomic<uint64_t> lds_set{0};
   hipError_t e = fdb_set_lds_once((const void*)kern, lds, lds_set);
   if (e != hipSuccess) return (int)e;
-  const unsigned parts = MODE == kFarOnly && p.far_parts > 1 ? (unsigned)p.far_parts : 1u;
+  const unsigned parts = MODE == kFarOnly && p.far_parts > 1 ? (unsigned)p.far_parts
+                         : MODE == kFused && p.key_parts > 1 ? (unsigned)p.key_parts : 1u;
   hipLaunchKernelGGL(kern, dim3((unsigned)grid_x * p.H, parts, 1), dim3(kThreads), lds, stream, p);
   return (int)hipGetLastError();
 }

@@ -283,6 +283,74 @@ __global__ __launch_bounds__(256) void fdb_merge_kernel(const FdbKParams p) {
 
 }  // namespace
 
+// The same for the one-kernel mode: p.key_parts partial results, all in the workspace, any element type and head_dim;
+// one thread per four elements.
+template <class VT, int D>
+__global__ __launch_bounds__(256) void fdb_merge_parts_kernel(const FdbKParams p) {
+  constexpr int CPR = D / 4, RB = D * VT::SZ;
+  const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= p.ws_rows * p.H * CPR) return;
+  const int cc = (int)(c % CPR);
+  const int64_t row = c / CPR;  // tok * H + h
+  const int h = (int)(row % p.H);
+  const int64_t tok = row / p.H;
+  char* dst;
+  if (p.cu) {
+    dst = p.out + (tok * p.o_st + (int64_t)h * p.o_sh) * VT::SZ;
+  } else {
+    const int b = (int)(tok / p.L), l = (int)(tok % p.L);
+    const int t0 = p.seq_start ? min(max(p.seq_start[b], 0), p.L) : 0;
+    const int len = p.seq_len ? min(max(p.seq_len[b], 0), p.L - t0) : p.L;
+    if (l < t0 || l >= t0 + len) return;  // rows outside the real tokens were written by the attention launch
+    dst = p.out + ((int64_t)b * p.o_sb + (int64_t)l * p.o_st + (int64_t)h * p.o_sh) * VT::SZ;
+  }
+  dst += cc * 4 * VT::SZ;
+  float w[FDB_MAX_FAR_PARTS], m = -INFINITY;
+#pragma unroll
+  for (int s = 0; s < FDB_MAX_FAR_PARTS; ++s) {
+    w[s] = s < p.key_parts ? ws_slot_lse(p, s, RB)[row] * 1.4426950408889634f : -INFINITY;
+    m = fmaxf(m, w[s]);
+  }
+  float denom = 0.f;
+#pragma unroll
+  for (int s = 0; s < FDB_MAX_FAR_PARTS; ++s) {
+    w[s] = w[s] != -INFINITY ? __builtin_amdgcn_exp2f(w[s] - m) : 0.f;
+    denom += w[s];
+  }
+  const float inv = denom > 0.f ? 1.f / denom : 0.f;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int s = 0; s < FDB_MAX_FAR_PARTS; ++s)
+    if (s < p.key_parts && w[s] > 0.f) {
+      const f32x4 x = VT::load4(ws_slot_out(p, s, RB) + row * RB + cc * 4 * VT::SZ);
+      const float f = w[s] * inv;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[e] = __builtin_fmaf(x[e], f, acc[e]);
+    }
+  VT::store4(dst, acc[0], acc[1], acc[2], acc[3]);
+  if (cc == 0 && p.lse) p.lse[row] = denom > 0.f ? (m + __builtin_amdgcn_logf(denom)) * 0.6931471805599453f : -INFINITY;
+}
+
+template <class VT>
+int launch_merge_parts_d(const FdbKParams& p, int head_dim, hipStream_t stream) {
+  const int64_t threads = p.ws_rows * p.H * (head_dim / 4);
+  const unsigned blocks = (unsigned)((threads + 255) / 256);
+  switch (head_dim) {
+    case 32: hipLaunchKernelGGL((fdb_merge_parts_kernel<VT, 32>), dim3(blocks), dim3(256), 0, stream, p); break;
+    case 64: hipLaunchKernelGGL((fdb_merge_parts_kernel<VT, 64>), dim3(blocks), dim3(256), 0, stream, p); break;
+    case 128: hipLaunchKernelGGL((fdb_merge_parts_kernel<VT, 128>), dim3(blocks), dim3(256), 0, stream, p); break;
+    default: return FDB_ERR_HEAD_DIM;
+  }
+  return (int)hipGetLastError();
+}
+
+int fdb_launch_merge_parts(const FdbKParams& p, int dtype, int head_dim, void* stream) {
+  if (dtype == FDB_F32) return launch_merge_parts_d<fdb::F32Tr>(p, head_dim, (hipStream_t)stream);
+  if (dtype == FDB_F16) return launch_merge_parts_d<fdb::F16Tr>(p, head_dim, (hipStream_t)stream);
+  if (dtype == FDB_BF16 || dtype == FDB_FP8_E4M3) return launch_merge_parts_d<fdb::Bf16Tr>(p, head_dim, (hipStream_t)stream);  // v's type
+  return FDB_ERR_DTYPE;
+}
+
 int fdb_launch_merge(const FdbKParams& p, int dtype, void* stream) {
   const int64_t chunks = p.ws_rows * p.H * 8;
   const unsigned blocks = (unsigned)((chunks + 255) / 256);

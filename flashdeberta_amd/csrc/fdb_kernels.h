@@ -38,7 +38,9 @@ struct FdbKParams {
                      // partial result of its own (the first in out / lse, the others in workspace slots 0 ..)
   int32_t near_parts; // workgroups per query tile of the near launch; above 1 each leaves the partial result of
                       // its share of the steps in workspace slot far_parts-1 + part, and fdb_launch_merge follows
-  int32_t ws_slots;  // partial results in the workspace: far_parts-1, plus near_parts if that is above 1
+  int32_t key_parts; // one-kernel mode: workgroups per query tile, each with an equal share of the key tiles and a
+                     // partial result of its own in workspace slot `part`; fdb_launch_merge_parts follows (1: no sharing)
+  int32_t ws_slots;  // partial results in the workspace: far_parts-1, plus near_parts if that is above 1; key_parts in the one-kernel mode
   char* ws;          // [ws_slots][ws_rows][H][D] elements of v's type (rows normalised over the keys seen), then
   int64_t ws_rows;   // [ws_slots][ws_rows][H] float log-sum-exps (-inf: no key seen); ws_rows = rows of the lse buffer
   int32_t causal;
@@ -145,6 +147,9 @@ int fdb_launch_near8(const FdbKParams& p, int grid_x, void* stream);
 // fdb_launch_merge: after a near launch with near_parts > 1: out / lse from the far partial results (when
 // p.far_done) and the near ones (16-bit element types, head_dim 64).
 int fdb_launch_merge(const FdbKParams& p, int dtype, void* stream);
+// fdb_launch_merge_parts: after a one-kernel launch with key_parts > 1: out (and lse, when given) from the key_parts
+// partial results in the workspace (any element type and head_dim).
+int fdb_launch_merge_parts(const FdbKParams& p, int dtype, int head_dim, void* stream);
 int fdb_launch_worklist(const int32_t* cu, int32_t batch, int32_t* wl, int32_t max_tiles, void* stream);
 // one tensor (x1 == NULL) or two of one shape and one set of strides: fill, absmax and quantise in three launches
 int fdb_launch_quant(const void* x0, const void* x1, int64_t x_st, int64_t x_sh, void* y0, void* y1, int64_t y_st, int64_t y_sh,

@@ -121,7 +121,8 @@ typedef struct fdb_attn_args {
   int32_t lut_radius;
   int32_t dtype;           /* enum fdb_dtype                                                 */
   int32_t causal;          /* nonzero: key j visible to query i only if j <= i               */
-  int32_t far_splits;      /* 0: the library decides; 1 .. FDB_MAX_FAR_SPLITS: workgroups that share the far keys of a query tile */
+  int32_t far_splits;      /* 0: the library decides; 1 .. FDB_MAX_FAR_SPLITS: workgroups that share the far keys of a query tile
+                              (all its keys where one kernel serves the call) */
   int32_t near_splits;     /* the same for the near keys (those whose bucketed relative position varies)                  */
   float sm_scale;
 } fdb_attn_args;
@@ -248,7 +249,10 @@ int fdb_attn_bwd(const fdb_attn_bwd_args* a, void* stream);
  * rows * heads * (head_dim * sizeof(v element) + 4) bytes each (rows: those of the lse buffer): far_splits - 1
  * slots, plus near_splits slots if near_splits > 1 (a small merge kernel then follows the two launches).
  * The workspace is optional: without it (or with a smaller one) the call first gives up the near splits,
- * then uses as many far splits as fit, down to one, with the same result up to rounding.  far_splits and
+ * then uses as many far splits as fit, down to one, with the same result up to rounding.  Calls that one kernel
+ * serves (fp32, head_dim 128, no position term, no lse buffer) share ALL key tiles of a query tile among up to
+ * FDB_MAX_FAR_SPLITS workgroups when the query tiles fill less than half of the compute units (never for causal
+ * calls): far_splits slots (far_splits asks for a number), and a merge kernel follows.  far_splits and
  * near_splits of `a` are read, its workspace fields ignored here.  No counterpart in the reference, whose
  * kernels have one program per query tile (flash_attention.py:465-488).
  */

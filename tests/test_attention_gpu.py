@@ -211,6 +211,53 @@ def test_near_steps_shared_among_workgroups(far, near, L, pb, mr, causal, c2p, p
     assert (out.float() - one.float()).abs().max().item() <= TOL[dtype]
 
 
+@pytest.mark.parametrize("splits", [2, 3, 4])
+@pytest.mark.parametrize("L,D,pb,mr,causal,c2p,p2c,dtype,packed", [
+    (700, 64, 256, 512, False, True, True, torch.float32, False),    # fp32: the one-kernel mode, eleven key tiles
+    (520, 128, 32, 64, False, True, True, torch.bfloat16, False),    # head_dim 128, far tiles on both sides of each share
+    (333, 128, 256, 512, False, True, False, torch.float32, False),  # one term, ragged last tile
+    (450, 64, 32, 64, True, True, True, torch.float32, False),       # causal: never shared, whatever is asked for
+    (300, 64, 0, 64, False, False, False, torch.float16, False),     # no position term: plain tiles
+    (90, 32, 32, 64, False, True, True, torch.float32, False),       # two key tiles: empty shares
+    (400, 64, 32, 64, False, True, True, torch.float32, True),       # packed sequences of unequal length
+])
+def test_one_kernel_mode_shares_the_keys_of_a_query_tile(splits, L, D, pb, mr, causal, c2p, p2c, dtype, packed):
+    """Calls that one kernel serves (fp32, head_dim 128, no position term) with the key tiles of every query tile
+    shared among several workgroups and the merge launch behind them: same result as unshared, both match the
+    oracle (output and log-sum-exp); padded rows stay zero."""
+    H = 2
+    q, k, v, pk, pq = _inputs(2, L, H, D, pb, mr, dtype, 900 + L + splits, 1.0, c2p, p2c)
+    kw = dict(position_buckets=pb, max_relative_positions=mr, causal=causal, return_lse=True)
+    tol = TOL[dtype]
+    if packed:
+        lens = [L, L // 3]
+        qs, ks, vs = [torch.cat([x[b, :n] for b, n in enumerate(lens)]) for x in (q, k, v)]
+        cu = torch.tensor([0, lens[0], sum(lens)], dtype=torch.int32).cuda()
+        args = [_dev(x) for x in (qs, ks, vs, pk, pq)]
+        out, lse = ops.disentangled_attention_fwd(*args, cu_seqlens=cu, max_seqlen=L, far_splits=splits, **kw)
+        one, _ = ops.disentangled_attention_fwd(*args, cu_seqlens=cu, max_seqlen=L, far_splits=1, **kw)
+        off = 0
+        for b, n in enumerate(lens):
+            ref, ref_lse = _oracle_blhd(q[b:b + 1, :n], k[b:b + 1, :n], v[b:b + 1, :n], pk, pq, pb, mr, causal=causal, return_lse=True)
+            _check(out[off:off + n][None], ref, tol, "out of sequence %d" % b)
+            _check(lse[off:off + n][None], ref_lse, 4 * tol, "lse of sequence %d" % b)
+            off += n
+    else:
+        ref, ref_lse = _oracle_blhd(q, k, v, pk, pq, pb, mr, causal=causal, return_lse=True)
+        args = [_dev(x) for x in (q, k, v, pk, pq)]
+        out, lse = ops.disentangled_attention_fwd(*args, far_splits=splits, **kw)
+        one, _ = ops.disentangled_attention_fwd(*args, far_splits=1, **kw)
+        _check(out, ref, tol, "out")
+        _check(lse.view(2, L, H), ref_lse, 4 * tol, "lse")
+        # a padded batch: the rows outside the real tokens are zeros, the others those of the shorter sequence alone
+        n = L - 37
+        pad, _ = ops.disentangled_attention_fwd(*args, far_splits=splits, seq_len=torch.tensor([L, n], dtype=torch.int32).cuda(), **kw)
+        ref_n = _oracle_blhd(q[1:, :n], k[1:, :n], v[1:, :n], pk, pq, pb, mr, causal=causal)
+        _check(pad[1:, :n], ref_n, tol, "padded row")
+        assert (pad[1, n:] == 0).all()
+    assert (out.float() - one.float()).abs().max().item() <= tol
+
+
 @pytest.mark.parametrize("slots", [0, 1, 2, 4, 5])
 def test_caller_owned_workspace_of_any_size(slots):
     """A caller-owned workspace smaller than what three far and three near shares need (five slots): the
