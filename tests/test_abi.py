@@ -145,7 +145,15 @@ def test_far_split_policy_and_workspace_size():
     a = args(8, 4096); a.near_splits = 3; assert ws(a) == 3 * part(8 * 4096, 12)
     a = args(1, 4096); a.far_splits = 1; assert ws(a) == 0
     a = args(1, 2048); a.near_splits = 1; assert ws(a) == 0
-    a = args(1, 4096); a.dtype = _lib.FDB_F32; a.far_splits = a.near_splits = 3; assert ws(a) == 0   # fp32 takes the fused kernel
+    # fp32 takes the one-kernel mode: its shares divide all key tiles of a query tile and every share has a slot
+    part32 = lambda rows, heads: rows * heads * (64 * 4 + 4)
+    a = args(1, 4096); a.dtype = _lib.FDB_F32; a.far_splits = a.near_splits = 3; assert ws(a) == 3 * part32(4096, 12)
+    a = args(1, 4096); a.dtype = _lib.FDB_F32; assert ws(a) == 0                         # 384 workgroups on 256 compute units
+    a = args(1, 1024); a.dtype = _lib.FDB_F32; assert ws(a) == 2 * part32(1024, 12)      # 96: two shares of eight tiles
+    a = args(1, 512); a.dtype = _lib.FDB_F32; assert ws(a) == 4 * part32(512, 12)        # 48: four shares of two tiles
+    a = args(1, 512); a.dtype = _lib.FDB_F32; a.causal = 1; assert ws(a) == 0            # causal calls are never shared
+    a = args(1, 512); a.dtype = _lib.FDB_F32; a.causal = 1; a.far_splits = 3; assert ws(a) == 0
+    a = args(1, 100); a.dtype = _lib.FDB_F32; assert ws(a) == 0                          # two key tiles: nothing to share
     a = args(1, 4096); a.cu_seqlens, a.worklist = 0x6000, 0x7000; assert ws(a) == 0   # lengths unknown to the host
     a.far_splits = 2; assert ws(a) == part(4096, 12)
     a = args(1, 4096); a.far_splits = 5; assert chk(a) == -5 and ws(a) == 0
