@@ -16,7 +16,7 @@
 //      with and without a higher priority for the VALU wave
 //   D  a far tile of the attention kernels (8 MFMAs of scores, 32 exponentials + 16 conversions + 32 adds, 8 MFMAs
 //      of P V): 1 to 4 independent waves per SIMD; two waves per SIMD half a tile apart, with and without workgroup
-//      barriers between the phases
+//      barriers between the phases; three waves per SIMD one phase apart with a barrier after every phase
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -230,9 +230,11 @@ static int run_pair(const char* name, float* d) {
 // MODE 0: 256-thread workgroups, WPS per CU, every wave runs scores -> VALU phase -> P V one after the other;
 // MODE 1: one 512-thread workgroup per CU, the second wave of every SIMD half a tile behind the first, workgroup
 //         barriers between the phases (explicit ping-pong: between two barriers one wave of a SIMD issues only MFMAs,
-//         the other only VALU instructions);  MODE 2: the same offset at the start and no barriers afterwards.
+//         the other only VALU instructions);  MODE 2: the same offset at the start and no barriers afterwards;
+// MODE 3: one 768-thread workgroup per CU, three waves per SIMD one phase apart (scores | VALU phase | P V), a workgroup
+//         barrier after every phase: at any time one wave of a SIMD is in each of the three phases.
 template <int MODE, int WPS>
-__global__ __launch_bounds__(MODE ? 512 : 256, MODE ? 1 : WPS) void tile_kernel(float* out, int iters, float seed) {
+__global__ __launch_bounds__(MODE == 3 ? 768 : MODE ? 512 : 256, MODE ? 1 : WPS) void tile_kernel(float* out, int iters, float seed) {
   __shared__ int cnt[4];
   int role = 0;
   if (MODE) {
@@ -277,6 +279,20 @@ __global__ __launch_bounds__(MODE ? 512 : 256, MODE ? 1 : WPS) void tile_kernel(
       pv();
       __builtin_amdgcn_sched_barrier(0);
     }
+  } else if (MODE == 3) {
+    for (int e = 0; e < role; ++e) __syncthreads();
+    for (int it = 0; it < iters; ++it) {
+      scores();
+      __builtin_amdgcn_sched_barrier(0);
+      __syncthreads();
+      valu_phase(s0, s1, p, l);
+      __builtin_amdgcn_sched_barrier(0);
+      __syncthreads();
+      pv();
+      __builtin_amdgcn_sched_barrier(0);
+      __syncthreads();
+    }
+    for (int e = role; e < 2; ++e) __syncthreads();
   } else {
     scores();
     if (role == 1) {
@@ -306,10 +322,10 @@ static int run_tile(const char* name, float* d) {
   const int iters = 20000;
   float ms;
   CHECK(hipFuncSetAttribute((const void*)tile_kernel<MODE, WPS>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_for(1)));
-  if (timed([&] { tile_kernel<MODE, WPS><<<g_cus * (MODE ? 1 : WPS), MODE ? 512 : 256, lds_for(MODE ? 1 : WPS)>>>(d, iters, 0.001f); }, &ms)) return 1;
+  if (timed([&] { tile_kernel<MODE, WPS><<<g_cus * (MODE ? 1 : WPS), MODE == 3 ? 768 : MODE ? 512 : 256, lds_for(MODE ? 1 : WPS)>>>(d, iters, 0.001f); }, &ms)) return 1;
   static long long clk[8192];
   CHECK(hipMemcpyFromSymbol(clk, HIP_SYMBOL(g_wave_clk), sizeof clk));
-  const int waves_per_simd = MODE ? 2 : WPS, waves = g_cus * 4 * waves_per_simd;
+  const int waves_per_simd = MODE == 3 ? 3 : MODE ? 2 : WPS, waves = g_cus * 4 * waves_per_simd;
   double hi = 0, mean = 0;
   for (int i = 0; i < waves; ++i) {
     hi = clk[i] > hi ? (double)clk[i] : hi;
@@ -344,7 +360,8 @@ int main() {
   if (run_tile<0, 1>("tile loop, one wave per SIMD", d) || run_tile<0, 2>("tile loop, two independent waves per SIMD", d) ||
       run_tile<0, 3>("tile loop, three independent waves per SIMD", d) || run_tile<0, 4>("tile loop, four independent waves per SIMD", d) ||
       run_tile<1, 1>("tile loop, two waves per SIMD half a tile apart, barriers", d) ||
-      run_tile<2, 1>("tile loop, two waves per SIMD half a tile apart, free-running", d))
+      run_tile<2, 1>("tile loop, two waves per SIMD half a tile apart, free-running", d) ||
+      run_tile<3, 1>("tile loop, three waves per SIMD a phase apart, barriers", d))
     return 1;
   return 0;
 }
