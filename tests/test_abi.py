@@ -105,6 +105,11 @@ def test_argument_validation_codes():
     a = _good_args(); a.dtype = _lib.FDB_FP8_E4M3; assert chk(a) == -7   # no scales
     a = _good_args(); a.cu_seqlens = 0x4000; assert chk(a) == -8          # no work-list
     a = _good_args(); a.dtype = _lib.FDB_F32; a.head_dim = 128; assert chk(a) == 0       # every dtype at every head_dim
+    # rows of the position tables are addressed with 32-bit byte offsets: 24-bit row strides, a head's table within 2^31 bytes
+    a = _good_args(); a.pk_stride_r = -64; assert chk(a) == -5
+    a = _good_args(); a.pq_stride_r = 1 << 23; assert chk(a) == -5                       # 2^24 bytes per row in a 16-bit type
+    a = _good_args(); a.pk_stride_r = (1 << 23) - 8; assert chk(a) == -5                 # rows fit, 2 * att_span of them do not
+    a = _good_args(); a.pk_stride_r = 768; a.pq_stride_r = 1536; assert chk(a) == 0      # rows of a [2S, H * D] projection output
     a = _good_args(); a.pos_key = a.pos_query = None; a.delta_lut = None; a.att_span = 0; assert chk(a) == 0
     assert lib.fdb_attn_check(None) == -1
     # launching with bad arguments returns the same code without touching the GPU
