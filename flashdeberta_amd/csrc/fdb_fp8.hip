@@ -16,8 +16,8 @@
 //                     (s_q q + s_qr Q_r[delta]) * sm_scale * log2(e) * s_k is formed in fp32 and rounded to e4m3 once
 //                     per row and side with a power-of-two exponent that the MFMA's scale operand takes back out.
 //   fdb_near8_kernel  the near key tiles in 32-key steps, the scheme of the 16-bit near kernel (expanded table rows
-//                     in two LDS rings, C through a per-wave 16-bit scratch, P by lane rotations) on 64-byte rows:
-//                     4 score MFMAs per step instead of 16.  The three products have the units s_q s_k, s_q s_kr
+//                     in two LDS rings, C through a per-wave fp16 scratch that holds both blocks of a step, P by lane
+//                     rotations) on 64-byte rows: 4 score MFMAs per step instead of 16.  The three products have the units s_q s_k, s_q s_kr
 //                     and s_k s_qr: the content product accumulates on top of C * (s_kr / s_k), P enters as
 //                     fma(P, s_qr / s_q, .), and one factor s_q s_k sm_scale log2(e) converts the sum.
 #include <hip/hip_runtime.h>
@@ -349,53 +349,72 @@ int launch_far8_one(const FdbKParams& p, int grid_x, hipStream_t stream) {
 // near tiles
 // ---------------------------------------------------------------------------------------------------------------
 constexpr int kStep = 32;        // keys per step
-constexpr int kRingBatches = 6;  // 5 batches of 32 relative positions in use by a step + the one being filled for the next
-constexpr int kRingRows = 32 * kRingBatches;
-constexpr int kScrW = 44;        // 16-bit elements between the rows of a wave's C scratch (36 in use; see the 16-bit near kernel)
-constexpr int kScrElems = 32 * kScrW;
+// Batches of 32 relative positions in the rings.  A step reads five batches of E_Q (one per wave and block) while its
+// loads fill a sixth; of E_K it reads only the four batches of the waves' new blocks, so the batch that the loads
+// replace is the one no wave needs any more.
+constexpr int kRingBatchesK = 5, kRingBatchesQ = 6;
+constexpr int kScrPitch = 68;    // 16-bit elements per row of a wave's C scratch: two blocks of 32 columns + columns 0..3 once more
+constexpr int kScrElems = 32 * kScrPitch;
 constexpr int kCShift = 8;       // C leaves its MFMA scaled by 2^-8 so that 64 * 448 * 448 fits the fp16 scratch
 
 struct N8 {
   static constexpr int K_BYTES = kStep * kRow8;       // 2 KB, rows swizzled with f8
   static constexpr int V_BYTES = kStep * kRowV;       // 4 KB, rows swizzled like the 16-bit kernels' (vf)
-  static constexpr int RING_BYTES = kRingRows * kRow8;  // 12 KB
+  static constexpr int RINGK_BYTES = 32 * kRingBatchesK * kRow8;  // 10 KB
+  static constexpr int RINGQ_BYTES = 32 * kRingBatchesQ * kRow8;  // 12 KB
   static constexpr int SCR_BYTES = 4 * kScrElems * 2;
   static constexpr int lds_bytes(bool c2p, bool p2c) {
-    return 2 * K_BYTES + 2 * V_BYTES + (c2p ? RING_BYTES + SCR_BYTES : 0) + (p2c ? RING_BYTES : 0);
+    return 2 * K_BYTES + 2 * V_BYTES + (c2p ? RINGK_BYTES + SCR_BYTES : 0) + (p2c ? RINGQ_BYTES : 0);
   }
 };
 
 // swizzle of the 128-byte V rows: slot (row, s) holds chunk s ^ vf(row)
 __device__ __forceinline__ int vf(int row) { return 4 * ((row >> 1) & 1) | ((row >> 2) & 3); }
 
+// Lane rotations and the reads of C's band are issued as asm, outside the compiler's count of outstanding LDS
+// operations: the step waits for all of them once (lds_wait_all8) instead of once per value.
+template <int OFFSET>
+__device__ __forceinline__ float swizzle_asm8(float x) {
+  float r;
+  asm volatile("ds_swizzle_b32 %0, %1 offset:%2" : "=v"(r) : "v"(x), "n"(OFFSET));
+  return r;
+}
+// px[v] = xs[v] of the lane (ROT0 - c(v)) places further up in this lane's half-wave (mod 32), c(v) = 8*(v/4) + 3 - v%4
 template <int ROT0, int... V>
 __device__ __forceinline__ void rotate16(const float (&xs)[16], float (&px)[16], std::integer_sequence<int, V...>) {
-  ((px[V] = __builtin_bit_cast(
-        float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, xs[V]), 0xC000 | ((ROT0 - (8 * (V >> 2) + 3 - (V & 3))) << 5)))),
-   ...);
+  ((px[V] = swizzle_asm8<(0xC000 | (((ROT0 - (8 * (V >> 2) + 3 - (V & 3))) & 31) << 5))>(xs[V])), ...);
 }
+template <int OFF>
+__device__ __forceinline__ uint32_t lds_u16_asm(uint32_t addr) {
+  uint32_t r;
+  asm volatile("ds_read_u16 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
+  return r;
+}
+__device__ __forceinline__ void lds_wait_all8() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
-// KEEP: block 1 of a step is block 0 of the step before, so C's accumulator and P's A operands of that block are kept
-// from step to step (two workgroups per CU).  Without KEEP both blocks are fetched and contracted in every step -- one
-// more MFMA and two more LDS reads -- and the kernel fits the 168 registers of three workgroups per CU.
-template <bool C2P, bool P2C, bool KEEP>
-__global__ __launch_bounds__(kThreads, (C2P && P2C && KEEP) ? 2 : 3) void fdb_near8_kernel(const FdbKParams p) {
+// The scheme of the 16-bit near kernel (fdb_near.hip) on e4m3 operands: rings of batches aligned to the waves' blocks, C's
+// scratch holding both blocks of a step (only the block that is new to the step is contracted and written; the other one
+// is the block the step before wrote).  P's A operands of block 1 are read again rather than kept from the step before
+// (168 registers per lane at three workgroups per CU do not hold them), which is why the ring of E_Q has a sixth batch: the
+// batch a step's loads overwrite must not be one that a wave still reads in that step.  Per wave and step one e4m3 MFMA
+// each for the content product and C, two for P, four bf16 MFMAs for P V.
+template <bool C2P, bool P2C>
+__global__ __launch_bounds__(kThreads, 3) void fdb_near8_kernel(const FdbKParams p) {
   constexpr int D = 64, DBLKS = 2;
   using VT = Bf16Tr;
   using vfrag = typename VT::frag;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   char* Ks = smem;                    // [2][32][64]: step k reads buffer k & 1
   char* Vs = Ks + 2 * N8::K_BYTES;    // [2][32][128]
-  char* EK = Vs + 2 * N8::V_BYTES;    // [192][64] rows K_r[delta(r)], slot = (r_hi0 - r) mod 192
-  char* EQ = EK + (C2P ? N8::RING_BYTES : 0);
-  char* scr_raw = EQ + (P2C ? N8::RING_BYTES : 0);
+  char* EK = Vs + 2 * N8::V_BYTES;    // [160][64] rows K_r[delta(r)]: batch u / 32 of u = r_hi0 - r in slot batch mod 5; E_Q: [192][64], mod 6
+  char* EQ = EK + (C2P ? N8::RINGK_BYTES : 0);
+  char* scr_raw = EQ + (P2C ? N8::RINGQ_BYTES : 0);
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63, li = lane & 31, g = lane >> 5;
   int xq, h;
   block_map((int)blockIdx.x, p.grid_x, p.H, p.tiles_per_seq, p.cu == nullptr, kMiddleFirst, xq, h);
-  uint16_t* scr = (uint16_t*)scr_raw + wave * kScrElems;
 
   int b, m0, tok0, Lb;
   int64_t qo, ko, vo, oo;
@@ -453,41 +472,57 @@ __global__ __launch_bounds__(kThreads, (C2P && P2C && KEEP) ? 2 : 3) void fdb_ne
   }
   const int n_steps = s1 - s0;
   const int n_full = p.causal ? 0 : max(0, min(n_steps, Lb / kStep - s0));
+  // u = r_hi0 - r counts downwards from the first step's largest r; batch = u / 32, ring slot = batch mod 5 (E_K) or 6 (E_Q).  Wave w's
+  // block bk at step k is batch k + 4 - w - bk, MFMA row m its row 31 - m: r = iw0 - 32 s - 32 + 32 bk + m.
   const int r_hi0 = m0 + FDB_BM - 1 - s0 * kStep;
 
   // ---- staging ---------------------------------------------------------------------------------------------
   // V: one 16-byte chunk per thread (a wave's load fills 8 rows of 128 bytes).  The 64-byte rows of K and of one
   // batch of each ring are 2 KB each, i.e. two waves' loads: waves 0 and 1 fetch K and E_K, waves 2 and 3 E_Q
   // (a load fills 16 rows, lane l slot l % 4 of row l / 4).  LDS row r of K holds key r ^ 3 of the step, as in
-  // the 16-bit kernel.
+  // the 16-bit kernel.  A step inside the sequence travels as a scalar base + this thread's 32-bit offset.
   const uint32_t lds0 = (uint32_t)(uintptr_t)(LDS_AS char*)smem;
   const int vrow = tid >> 3, vcc = tid & 7;
   const uint32_t v_chunk = (uint32_t)((vcc ^ vf(vrow)) * 16);
   const int row8 = (tid & 127) >> 2;                                   // row of a 32-row e4m3 tile this thread fetches a chunk of
   const uint32_t chunk8 = (uint32_t)(((tid & 3) ^ f8(row8)) * 16);
   const uint32_t half_kb = (uint32_t)(wave & 1) * 1024u;
+  const uint32_t k_lane = (uint32_t)(row8 ^ 3) * k_rsb + chunk8, v_lane = (uint32_t)vrow * v_rsb + v_chunk;
   int dnext = 0;
   auto k_dma = [&](int s, int buf) __attribute__((always_inline)) {
     if (wave < 2) {
-      const int row = min(s * kStep + (row8 ^ 3), Lb - 1);
-      dma16(kb + (uint64_t)(uint32_t)row * k_rsb + chunk8, lds0 + buf * N8::K_BYTES + half_kb);
+      const uint32_t dst = lds0 + buf * N8::K_BYTES + half_kb;
+      if ((s + 1) * kStep <= Lb) {
+        dma16sn(kb + (uint64_t)(uint32_t)(s * kStep) * k_rsb, k_lane, dst);
+      } else {
+        const int row = min(s * kStep + (row8 ^ 3), Lb - 1);
+        dma16n(kb + (uint64_t)(uint32_t)row * k_rsb + chunk8, dst);
+      }
     }
   };
   auto v_dma = [&](int s, int buf) __attribute__((always_inline)) {
-    const int row = min(s * kStep + vrow, Lb - 1);
-    dma16(vb + (uint64_t)(uint32_t)row * v_rsb + v_chunk, lds0 + 2 * N8::K_BYTES + buf * N8::V_BYTES + (uint32_t)wave * 1024u);
+    const uint32_t dst = lds0 + 2 * N8::K_BYTES + buf * N8::V_BYTES + (uint32_t)wave * 1024u;
+    if ((s + 1) * kStep <= Lb) {
+      dma16sn(vb + (uint64_t)(uint32_t)(s * kStep) * v_rsb, v_lane, dst);
+    } else {
+      const int row = min(s * kStep + vrow, Lb - 1);
+      dma16n(vb + (uint64_t)(uint32_t)row * v_rsb + v_chunk, dst);
+    }
   };
-  auto batch_delta = [&](int batch) __attribute__((always_inline)) {
-    const int r = r_hi0 - (batch * 32 + row8);
-    return (int)((const uint16_t*)p.lut)[max(-p.R, min(p.R, r)) + p.R];
+  int r_tab = r_hi0 - row8;  // relative position of this thread's row of a batch; runs down by 32 per batch
+  auto batch_delta = [&]() __attribute__((always_inline)) {
+    const int d = (int)((const uint16_t*)p.lut)[max(-p.R, min(p.R, r_tab)) + p.R];
+    r_tab -= 32;
+    return d;
   };
   const uint32_t ek_lds = lds0 + (uint32_t)(EK - smem) + half_kb, eq_lds = lds0 + (uint32_t)(EQ - smem) + half_kb;
-  auto batch_dma = [&](int delta, int batch) __attribute__((always_inline)) {
-    const uint32_t seg = (uint32_t)(batch % kRingBatches) * (32 * kRow8);
+  const uint32_t pk_rowb = (uint32_t)p.pk_sr, pq_rowb = (uint32_t)p.pq_sr;  // the host bounds them (24-bit row strides)
+  auto batch_dma = [&](int delta, int slot) __attribute__((always_inline)) {
+    const uint32_t seg = (uint32_t)slot * (32 * kRow8);
     if (wave < 2) {
-      if constexpr (C2P) dma16(pkb + (int64_t)delta * p.pk_sr + chunk8, ek_lds + seg);
+      if constexpr (C2P) dma16sn(pkb, __umul24((uint32_t)delta, pk_rowb) + chunk8, ek_lds + seg);
     } else {
-      if constexpr (P2C) dma16(pqb + (int64_t)delta * p.pq_sr + chunk8, eq_lds + seg);
+      if constexpr (P2C) dma16sn(pqb, __umul24((uint32_t)delta, pq_rowb) + chunk8, eq_lds + seg);
     }
   };
 
@@ -499,9 +534,8 @@ __global__ __launch_bounds__(kThreads, (C2P && P2C && KEEP) ? 2 : 3) void fdb_ne
   float m_run = -INFINITY, l_run = 0.f;
 
   // ---- per-lane constants (see the 16-bit near kernel for the derivations) --------------------------------------
-  const int fr = f8(158 - li);   // the ring slot of this lane's row keeps the low five bits of 158 - li for ever
-  const uint32_t rx0 = (uint32_t)(((2 * g) ^ fr) * 16), rx1 = (uint32_t)(((2 * g + 1) ^ fr) * 16);
-  int slot0 = 158 - li - 32 * wave;
+  const int arow = 31 - li, fr = f8(arow);  // MFMA row m = li of a position product is row 31 - li of its batch
+  const uint32_t ra0 = (uint32_t)(arow * kRow8) + (uint32_t)(((2 * g) ^ fr) * 16), ra1 = (uint32_t)(arow * kRow8) + (uint32_t)(((2 * g + 1) ^ fr) * 16);
   const uint32_t kx0 = lds0 + (uint32_t)(li * kRow8 + ((2 * g) ^ f8(li)) * 16), kx1 = lds0 + (uint32_t)(li * kRow8 + ((2 * g + 1) ^ f8(li)) * 16);
   uint32_t vlx[4];
   {
@@ -509,36 +543,46 @@ __global__ __launch_bounds__(kThreads, (C2P && P2C && KEEP) ? 2 : 3) void fdb_ne
     const int slotl = (2 * (grp & 1) + ((s16 & 3) >> 1)) ^ (4 * ((s16 >> 3) & 1)) ^ (grp >> 1);
     const uint32_t vlane = (4 * (grp >> 1) + (s16 >> 2)) * kRowV + slotl * 16 + (s16 & 1) * 8;
 #pragma unroll
-    for (int x = 0; x < 4; ++x) vlx[x] = vlane ^ (64 * (x >> 1) ^ 32 * (x & 1));
+    for (int x = 0; x < 4; ++x) vlx[x] = lds0 + (uint32_t)(Vs - smem) + (vlane ^ (64 * (x >> 1) ^ 32 * (x & 1)));
   }
-  uint16_t* c_wrp = scr + li * kScrW + 4 * g;
-  LDS_AS const volatile uint16_t* c_rd[4];
+  // C's scratch: row li, two halves of 32 columns that alternate with the step's parity (+ columns 0..3 once more)
+  const uint32_t scr0 = lds0 + (uint32_t)(scr_raw - smem) + (uint32_t)wave * (kScrElems * 2) + (uint32_t)li * (kScrPitch * 2);
+  uint16_t* c_wr = (uint16_t*)scr_raw + wave * kScrElems + li * kScrPitch + 4 * g;
+  uint16_t* c_dup = g == 0 ? c_wr + 64 : c_wr;
+  uint32_t c_rd[2][4];
 #pragma unroll
-  for (int q = 0; q < 4; ++q)
-    c_rd[q] = (LDS_AS const volatile uint16_t*)(scr + li * kScrW + ((li + 28 - 8 * q - 4 * g) & 31));
+  for (int par = 0; par < 2; ++par)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) c_rd[par][q] = scr0 + 2u * (uint32_t)((32 * par + li + 29 - 8 * q - 4 * g) & 63);
+  const int xl = li + 4 * g;  // P: a source lane (n = li) of register v hands out block 1 where n + jj < 32
 
-  i32x8 ac = {0, 0, 0, 0, 0, 0, 0, 0}, ac1 = ac, aq[2] = {ac, ac};
-  f32x16 ckeep[2];
   const uint32_t ek0 = lds0 + (uint32_t)(EK - smem), eq0 = lds0 + (uint32_t)(EQ - smem);
-  auto ring_read = [&](int buf, int slot) __attribute__((always_inline)) {
-    if constexpr (C2P) ac = lds_frag8(ek0 + slot * kRow8 + rx0, ek0 + slot * kRow8 + rx1);
-    if constexpr (P2C) aq[buf] = lds_frag8(eq0 + slot * kRow8 + rx0, eq0 + slot * kRow8 + rx1);
-  };
-  auto ring_read_block1 = [&](int buf, int slot) __attribute__((always_inline)) {  // the rows 32 relative positions up
-    const int s1 = slot >= 32 ? slot - 32 : slot + (kRingRows - 32);
-    if constexpr (C2P) ac1 = lds_frag8(ek0 + s1 * kRow8 + rx0, ek0 + s1 * kRow8 + rx1);
-    if constexpr (P2C) aq[buf] = lds_frag8(eq0 + s1 * kRow8 + rx0, eq0 + s1 * kRow8 + rx1);
+  auto ring_frag = [&](uint32_t ring, int slot) __attribute__((always_inline)) {
+    const uint32_t boff = (uint32_t)slot * (32 * kRow8);
+    return lds_frag8(ring + boff + ra0, ring + boff + ra1);
   };
   f32x16 zero;
 #pragma unroll
   for (int v = 0; v < 16; ++v) zero[v] = 0.f;
+  auto c_store = [&](const f32x16& cacc, int half) __attribute__((always_inline)) {
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      const u32x2 packed = {__builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(cacc[4 * q4], cacc[4 * q4 + 1])),
+                            __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(cacc[4 * q4 + 2], cacc[4 * q4 + 3]))};
+      *(u32x2*)(c_wr + 32 * half + 8 * q4) = packed;
+      if (half == 0 && q4 == 0) *(u32x2*)c_dup = packed;
+    }
+  };
+  int slot_k = 4 - wave, slot_q = 4 - wave;  // ring slots of this wave's block 0
+  const int ring_n = wave < 2 ? kRingBatchesK : kRingBatchesQ;  // the ring this wave's loads fill
+  int slot_dma = wave < 2 ? 0 : 5;                              // and the slot of it that the step's loads fill
   // ---- prologue -----------------------------------------------------------------------------------------------
   if (n_steps > 0) {
     k_dma(s0, 0);
     v_dma(s0, 0);
     int d0[6];
 #pragma unroll
-    for (int bt = 0; bt < 6; ++bt) d0[bt] = batch_delta(bt);
+    for (int bt = 0; bt < 6; ++bt) d0[bt] = batch_delta();
 #pragma unroll
     for (int bt = 0; bt < 6; ++bt) asm volatile("" : "+v"(d0[bt]));
 #pragma unroll
@@ -546,10 +590,7 @@ __global__ __launch_bounds__(kThreads, (C2P && P2C && KEEP) ? 2 : 3) void fdb_ne
     dnext = d0[5];
     wait_vmcnt<0>();
     __syncthreads();
-    if constexpr (KEEP) {
-      ring_read(1, slot0 >= 32 ? slot0 - 32 : slot0 + (kRingRows - 32));  // block 1 of step 0
-      if constexpr (C2P) ckeep[1] = mma8_sa<127 - kCShift>(ac, qf, zero);
-    }
+    if constexpr (C2P) c_store(mma8_sa<127 - kCShift>(ring_frag(ek0, 3 - wave), qf, zero), 1);  // block 1 of step 0
   }
 
   auto step = [&](auto mask_tag, auto par_tag, int k) __attribute__((always_inline)) {
@@ -562,58 +603,63 @@ __global__ __launch_bounds__(kThreads, (C2P && P2C && KEEP) ? 2 : 3) void fdb_ne
     __syncthreads();
     k_dma(s + 1, PAR ^ 1);
     v_dma(s + 1, PAR ^ 1);
-    batch_dma(dnext, k + 5);
+    batch_dma(dnext, slot_dma);  // batch k + 5 in place of batch k (E_K) or k - 1 (E_Q)
     __builtin_amdgcn_sched_barrier(0);
-    dnext = batch_delta(k + 6);
+    dnext = batch_delta();
     const i32x8 kf = lds_frag8(kx0 + PAR * N8::K_BYTES, kx1 + PAR * N8::K_BYTES);
-    ring_read(PAR, slot0);
-    if constexpr (!KEEP) ring_read_block1(PAR ^ 1, slot0);
-    f32x16 sacc = zero;
+    f32x16 sacc, cnew, pacc[2];
+    if constexpr (C2P) cnew = mma8_sa<127 - kCShift>(ring_frag(ek0, slot_k), qf, zero);
+    if constexpr (P2C) pacc[1] = mma8(kf, ring_frag(eq0, slot_q == 0 ? kRingBatchesQ - 1 : slot_q - 1), zero);
+    if constexpr (P2C) pacc[0] = mma8(kf, ring_frag(eq0, slot_q), zero);
+    sacc = mma8(kf, qf, zero);
+    uint32_t craw[16];
     if constexpr (C2P) {
-      ckeep[PAR] = mma8_sa<127 - kCShift>(ac, qf, zero);
-      if constexpr (!KEEP) ckeep[PAR ^ 1] = mma8_sa<127 - kCShift>(ac1, qf, zero);
-      const f32x16(&cacc)[2] = ckeep;
+      c_store(cnew, PAR);
+      wave_lds_fence();
 #pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        f32x4 pick;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int c0 = 8 * q4 + e, c1 = c0 + 4;
-          const uint64_t mask = ((2ull << c0) - 1ull) | ((c1 >= 31 ? 0xffffffffull : (2ull << c1) - 1ull) << 32);
-          pick[e] = __builtin_amdgcn_inverse_ballot_w64(mask) ? cacc[PAR][4 * q4 + e] : cacc[PAR ^ 1][4 * q4 + e];
-        }
-        const u32x2 packed = {__builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(pick[0], pick[1])),
-                              __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(pick[2], pick[3]))};
-        *(u32x2*)(c_wrp + 8 * q4) = packed;
-        if (q4 == 0) *(u32x2*)(c_wrp + 32) = packed;
+      for (int q = 0; q < 4; ++q) {
+        craw[4 * q + 0] = lds_u16_asm<0>(c_rd[PAR][q]);
+        craw[4 * q + 1] = lds_u16_asm<2>(c_rd[PAR][q]);
+        craw[4 * q + 2] = lds_u16_asm<4>(c_rd[PAR][q]);
+        craw[4 * q + 3] = lds_u16_asm<6>(c_rd[PAR][q]);
       }
       wave_lds_fence();
-#pragma unroll
-      for (int v = 0; v < 16; ++v)
-        sacc[v] = __builtin_fmaf((float)__builtin_bit_cast(_Float16, (uint16_t)c_rd[v >> 2][v & 3]), rho_c, 0.f);
-      wave_lds_fence();
-      __builtin_amdgcn_sched_barrier(0);
     }
-    f32x16 pacc[2];
+    float px[16];
     if constexpr (P2C) {
-#pragma unroll
-      for (int bk = 0; bk < 2; ++bk) pacc[bk] = mma8(kf, aq[PAR ^ bk], zero);
-    }
-    sacc = mma8(kf, qf, sacc);
-    if constexpr (P2C) {
-      float xs[16], px[16];
+      float xs[16];
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int c = 8 * (v >> 2) + 3 - (v & 3);
-        const uint64_t mask = (uint64_t)((1u << (31 - c)) - 1u) | ((uint64_t)(c < 27 ? (1u << (27 - c)) - 1u : 0u) << 32);
-        xs[v] = __builtin_amdgcn_inverse_ballot_w64(mask) ? pacc[1][v] : pacc[0][v];
+        const int c = 8 * (v >> 2) + 3 - (v & 3);  // jj - 4g
+        xs[v] = (xl < 32 - c) ? pacc[1][v] : pacc[0][v];
       }
       if (g == 0)
-        rotate16<31>(xs, px, std::make_integer_sequence<int, 16>{});
+        rotate16<32>(xs, px, std::make_integer_sequence<int, 16>{});
       else
-        rotate16<27>(xs, px, std::make_integer_sequence<int, 16>{});
+        rotate16<28>(xs, px, std::make_integer_sequence<int, 16>{});
+    }
+    vfrag vfr[2][DBLKS];
 #pragma unroll
-      for (int v = 0; v < 16; ++v) sacc[v] = __builtin_fmaf(px[v], rho_p, sacc[v]);
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int d = 0; d < DBLKS; ++d) {
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(uintptr_t)(vlx[2 * d] + PAR * N8::V_BYTES + 2048 * c));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(uintptr_t)(vlx[2 * d + 1] + PAR * N8::V_BYTES + 2048 * c + 1024));
+        vfr[c][d] = __builtin_bit_cast(vfrag, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      }
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (C2P || P2C) {
+      lds_wait_all8();
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        if constexpr (C2P) asm volatile("" : "+v"(craw[v]));
+        if constexpr (P2C) asm volatile("" : "+v"(px[v]));
+      }
+    }
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      if constexpr (C2P) sacc[v] = __builtin_fmaf((float)__builtin_bit_cast(_Float16, (uint16_t)craw[v]), rho_c, sacc[v]);
+      if constexpr (P2C) sacc[v] = __builtin_fmaf(px[v], rho_p, sacc[v]);
     }
     if constexpr (MASK) {
 #pragma unroll
@@ -661,13 +707,10 @@ __global__ __launch_bounds__(kThreads, (C2P && P2C && KEEP) ? 2 : 3) void fdb_ne
 #pragma unroll
     for (int c = 0; c < 2; ++c)
 #pragma unroll
-      for (int d = 0; d < DBLKS; ++d) {
-        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(Vs + PAR * N8::V_BYTES + vlx[2 * d] + 2048 * c));
-        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(Vs + PAR * N8::V_BYTES + vlx[2 * d + 1] + 2048 * c + 1024));
-        const vfrag vfr = __builtin_bit_cast(vfrag, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-        o_acc[d] = VT::mma(vfr, pf[c], o_acc[d]);
-      }
-    slot0 = slot0 + 32 >= kRingRows ? slot0 + 32 - kRingRows : slot0 + 32;
+      for (int d = 0; d < DBLKS; ++d) o_acc[d] = VT::mma(vfr[c][d], pf[c], o_acc[d]);
+    slot_k = slot_k == kRingBatchesK - 1 ? 0 : slot_k + 1;
+    slot_q = slot_q == kRingBatchesQ - 1 ? 0 : slot_q + 1;
+    slot_dma = slot_dma == ring_n - 1 ? 0 : slot_dma + 1;
   };
   {
     using T0 = std::integral_constant<int, 0>;
@@ -764,10 +807,9 @@ __global__ __launch_bounds__(kThreads, (C2P && P2C && KEEP) ? 2 : 3) void fdb_ne
 
 template <bool C2P, bool P2C>
 int launch_near8_one(const FdbKParams& p, int grid_x, hipStream_t stream) {
-  constexpr bool kKeep = !(C2P && P2C);   // with both terms: three workgroups per CU
-  auto kern = fdb_near8_kernel<C2P, P2C, kKeep>;
+  auto kern = fdb_near8_kernel<C2P, P2C>;
   constexpr int lds = N8::lds_bytes(C2P, P2C);
-  static_assert(lds <= 53 * 1024, "three workgroups per CU (a single term keeps its operands and still fits the registers)");
+  static_assert(lds <= 52 * 1024, "three workgroups per CU: with 53 KB a CU was seen to take only two");
   static std::atomic<uint64_t> lds_set{0};
   hipError_t e = fdb_set_lds_once((const void*)kern, lds, lds_set);
   if (e != hipSuccess) return (int)e;
