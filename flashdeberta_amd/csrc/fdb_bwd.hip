@@ -200,13 +200,13 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
     if (!kDQ && tid < C::TROWS) {
       const int row = min(r0 + tid, Lb - 1);
       const int64_t t = ((int64_t)b * p.L + tok0 + row) * p.H + h;
-      st_reg[0] = p.lse[t] * 1.4426950408889634f;
+      st_reg[0] = p.lse[t];   // used (scaled to base 2) only when stored: a use here would wait for the loads at once
       st_reg[1] = p.delta[t];
     }
   };
   auto stats_store = [&](int buf) __attribute__((always_inline)) {
     if (!kDQ && tid < C::TROWS) {
-      stat_s[buf * 2 * C::TROWS + tid] = st_reg[0];
+      stat_s[buf * 2 * C::TROWS + tid] = st_reg[0] * 1.4426950408889634f;
       stat_s[buf * 2 * C::TROWS + C::TROWS + tid] = st_reg[1];
     }
   };

@@ -55,8 +55,21 @@ __global__ __launch_bounds__(256) void issue_kernel(unsigned long long* out, int
                    : "+v"(a), "+v"(b)
                    :
                    : "s40", "scc");
-    } else {  // waits that are already satisfied and nops
+    } else if (KIND == 5) {  // waits that are already satisfied and nops
       asm volatile(REP16("s_waitcnt vmcnt(0)\n\ts_nop 0\n\ts_waitcnt lgkmcnt(0)\n\ts_nop 0\n\t") ::: "memory");
+    } else if (KIND == 6) {  // the exponential of the soft-max (transcendental unit)
+      asm volatile(REP16("v_exp_f32 %0, %0\n\tv_exp_f32 %1, %1\n\tv_exp_f32 %2, %2\n\tv_exp_f32 %3, %3\n\t")
+                   : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+    } else if (KIND == 7) {  // exponentials and plain vector instructions in turn, as in the soft-max of a key tile (2 : 3)
+      asm volatile(REP16("v_exp_f32 %0, %0\n\tv_add_f32 %2, %2, %3\n\tv_exp_f32 %1, %1\n\tv_add_f32 %3, %3, %2\n\t")
+                   : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+    } else if (KIND == 8) {  // conversion of two fp32 values to packed bf16
+      asm volatile(REP16("v_cvt_pk_bf16_f32 %0, %0, %1\n\tv_cvt_pk_bf16_f32 %1, %1, %2\n\tv_cvt_pk_bf16_f32 %2, %2, %3\n\tv_cvt_pk_bf16_f32 %3, %3, %0\n\t")
+                   : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+    } else {  // arbitrary lane permutation through the LDS pipe (address register per lane)
+      asm volatile(REP16("ds_bpermute_b32 %0, %1, %0\n\tds_bpermute_b32 %2, %1, %2\n\tds_bpermute_b32 %3, %1, %3\n\t"
+                         "ds_bpermute_b32 %0, %1, %0\n\t") "s_waitcnt lgkmcnt(0)\n\t"
+                   : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
     }
   }
   asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t1)::"memory");
@@ -97,5 +110,6 @@ int main() {
   CHECK(hipMemset(d, 0, 64));
   return run<0>("v_fma_f32 (independent)", d) || run<1>("s_add_u32 (independent)", d) || run<2>("v_fma_f32 / s_add_u32 alternating", d) ||
          run<3>("ds_swizzle_b32 (lane rotation, LDS pipe)", d) || run<4>("v_fma_f32 / s_add_u32 / ds_swizzle_b32 / satisfied s_waitcnt", d) ||
-         run<5>("satisfied s_waitcnt / s_nop 0", d);
+         run<5>("satisfied s_waitcnt / s_nop 0", d) || run<6>("v_exp_f32 (independent)", d) || run<7>("v_exp_f32 / v_add_f32 alternating", d) ||
+         run<8>("v_cvt_pk_bf16_f32", d) || run<9>("ds_bpermute_b32 (lane permutation, LDS pipe)", d);
 }
