@@ -1687,6 +1687,9 @@ def test_random_fp8_variants(seed):
     # more: its reference is the model of that arithmetic; every other route contracts the de-quantised operands as is
     pair = D == 64 and (c2p or p2c) and not single
     cpu = lambda x: None if x is None else x.cpu()
+    if pair:  # far and near keys of a query tile shared out among workgroups, as the library would for few tiles
+        kw["far_splits"], kw["near_splits"] = int(r.randint(4)), int(r.randint(4))
+        what += " shares %d/%d" % (kw["far_splits"], kw["near_splits"])
 
     def reference(sl, batch):
         if not pair:
