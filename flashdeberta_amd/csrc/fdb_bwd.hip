@@ -59,10 +59,30 @@ struct BCfg {
   static constexpr int TROWS = RS > 272 ? kBwdStep : 2 * kBwdStep;
   static constexpr int TILE = TROWS * RS;                    // a multiple of 1024: RS is a multiple of 16
   static constexpr int REGION = 2 * TILE;                    // [Y1 tile | Y2 tile] of one buffer
-  // two buffers, loop-row statistics, ring windows, far-step scores, groups to store; the table follows
-  static constexpr int fixed_lds_bytes() { return 2 * REGION + 4 * TROWS * 4 + FDB_BM * kRingStrideMax * 4 + FDB_BM * 4 + FDB_BM * 8; }
+  // two buffers, loop-row statistics, ring windows, groups to store; the table follows
+  static constexpr int fixed_lds_bytes() { return 2 * REGION + 4 * TROWS * 4 + FDB_BM * kRingStrideMax * 4 + FDB_BM * 8; }
   static int lds_bytes(int radius) { return fixed_lds_bytes() + (((2 * radius + 1) * 2 + 15) & ~15); }
 };
+
+// acc[m][n] = a_lane(n) + b_loop(m) as one MFMA: the start of S' in a block with a single table row, where the
+// position scores are one value per lane-side row and one per loop-side row.  Loop rows are MFMA rows (operand A,
+// lane = row), lane-side rows MFMA columns (operand B); the two contraction slots used are k = 0, 1.
+template <class QT>
+__device__ __forceinline__ f32x16 rank1_start(float a_lane, float b_loop, int g) {
+  const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  if constexpr (QT::SZ == 4) {
+    // K = 2: lane group g supplies k = g
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(g == 0 ? b_loop : 1.f, g == 0 ? 1.f : a_lane, zero, 0, 0, 0);
+  } else {
+    // K = 16: lane group 0 supplies k = 0..7
+    f32x8 ay = {0, 0, 0, 0, 0, 0, 0, 0}, ax = {0, 0, 0, 0, 0, 0, 0, 0};
+    ay[0] = g == 0 ? b_loop : 0.f;
+    ay[1] = g == 0 ? 1.f : 0.f;
+    ax[0] = g == 0 ? 1.f : 0.f;
+    ax[1] = g == 0 ? a_lane : 0.f;
+    return QT::mma(QT::from_f32(ay), QT::from_f32(ax), zero);
+  }
+}
 
 template <class QT, int D, int ROLE, bool C2P, bool P2C>
 __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_bwd_kernel(const FdbBwdParams p) {
@@ -75,8 +95,7 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
   char* Ys = smem;                                    // two buffers of [K | V] (dQ role) / [Q | dO] (dK/dV role)
   float* stat_s = (float*)(Ys + 2 * C::REGION);       // dK/dV role: per buffer, log-sum-exp (base 2) and Delta of the staged loop rows
   float* ring_s = stat_s + 4 * C::TROWS;              // [128 lane-side rows][kRingStride] score-gradient windows
-  float* vec_s = ring_s + FDB_BM * kRingStrideMax;      // [4 waves][32] loop-side position scores of a far step
-  int2* inf_s = (int2*)(vec_s + FDB_BM);              // [4 waves][32] (first group, groups) to store per row
+  int2* inf_s = (int2*)(ring_s + FDB_BM * kRingStrideMax);  // [4 waves][32] (first group, groups) to store per row
   LDS_AS int16_t* lut_s = (LDS_AS int16_t*)(inf_s + FDB_BM);  // the whole table (the launcher sizes the allocation for it)
 
   const int tid = threadIdx.x;
@@ -147,7 +166,6 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
   constexpr bool kGrad = kDQ ? C2P : P2C;
   float* ring_w = ring_s + wave * 32 * kRingStride;
   float* ring_x = ring_w + li * kRingStride;
-  float* vec_w = vec_s + wave * 32;
   int2* inf_w = inf_s + wave * 32;
   char* gw = nullptr;   // this sequence and head of the gradient tensor (elements of the input type)
   if (kGrad) {
@@ -297,20 +315,7 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
     const int d_far = dfar_n;
     f32x16 sacc, dpacc;   // S' starts from the position scores, dP' from -Delta: the products add on top
     if (kBias && far) {
-      if (kLoopT) {
-        if (g == 0) vec_w[li] = (float)raw_loop[0];
-        wave_lds_fence();
-#pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-          const f32x4 t4 = *(const f32x4*)(vec_w + 8 * q4 + 4 * g);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) sacc[4 * q4 + e] = t4[e] + (float)raw_lane[0];
-        }
-        wave_lds_fence();
-      } else {
-#pragma unroll
-        for (int v = 0; v < 16; ++v) sacc[v] = (float)raw_lane[0];
-      }
+      sacc = rank1_start<QT>(kLaneT ? (float)raw_lane[0] : 0.f, kLoopT ? (float)raw_loop[0] : 0.f, g);
     } else {
 #pragma unroll
       for (int v = 0; v < 16; ++v) sacc[v] = (float)raw_lane[v] + (float)raw_loop[v];
