@@ -30,6 +30,7 @@
 #include <stdint.h>
 
 #include <atomic>
+#include <type_traits>
 
 #include "fdb_device.h"
 #include "fdb_kernels.h"
@@ -341,24 +342,30 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
     // a block that touches the end of a sequence or the causal diagonal masks its elements one by one
     const bool edge = xw0 + 31 >= Lb || y0 + kBwdStep > Lb ||
                       (p.causal && (kDQ ? y0 + kBwdStep - 1 > xw0 : xw0 + 31 > y0));
+    // one branch for the block, not one per element: the common block carries no mask at all
+    auto probabilities = [&](auto edge_tag) __attribute__((always_inline)) {
+      constexpr bool EDGE = decltype(edge_tag)::value;
 #pragma unroll
-    for (int q4 = 0; q4 < 4; ++q4) {
-      f32x4 lse4 = {lse_x, lse_x, lse_x, lse_x};
-      if (!kDQ) lse4 = *(const f32x4*)(lse_s + 8 * q4 + 4 * g);
+      for (int q4 = 0; q4 < 4; ++q4) {
+        f32x4 lse4 = {lse_x, lse_x, lse_x, lse_x};
+        if (!kDQ) lse4 = *(const f32x4*)(lse_s + 8 * q4 + 4 * g);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int v = 4 * q4 + e;
-        float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[v], c_log2, -lse4[e]));
-        if (edge) {
-          const int yr = y0 + 8 * q4 + 4 * g + e;
-          const int i = kDQ ? xr : yr, j = kDQ ? yr : xr;
-          if (!(x_ok && yr < Lb && (!p.causal || j <= i))) pv = 0.f;
+        for (int e = 0; e < 4; ++e) {
+          const int v = 4 * q4 + e;
+          float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[v], c_log2, -lse4[e]));
+          if (EDGE) {
+            const int yr = y0 + 8 * q4 + 4 * g + e;
+            const int i = kDQ ? xr : yr, j = kDQ ? yr : xr;
+            if (!(x_ok && yr < Lb && (!p.causal || j <= i))) pv = 0.f;
+          }
+          pr[v] = pv;
+          ds[v] = pv * dpacc[v];
+          g_sum += ds[v];
         }
-        pr[v] = pv;
-        ds[v] = pv * dpacc[v];
-        g_sum += ds[v];
       }
-    }
+    };
+    if (edge) probabilities(std::true_type{});
+    else probabilities(std::false_type{});
     if (kGrad) {
       // LDS float atomics are served a lane at a time on this hardware (160 clocks per instruction), so the adds are
       // plain reads and writes: the lanes of a half-wave own different rows, and the two halves (which share rows)
