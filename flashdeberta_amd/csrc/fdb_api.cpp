@@ -475,7 +475,9 @@ int fdb_attn_bwd(const fdb_attn_bwd_args* a, void* stream) {
   // score gradients leave in aligned groups of four entries
   const uintptr_t group_bytes = 4u * (uintptr_t)qk_elem_size(a->dtype);  // one store: four entries
   if (has_pos && ((a->att_span & 1) || (a->bias_stride_b & 3) || (a->bias_stride_t & 3) || (a->bias_stride_h & 3) ||
-                  reinterpret_cast<uintptr_t>(a->d_c2p_bias) % group_bytes || reinterpret_cast<uintptr_t>(a->d_p2c_bias) % group_bytes))
+                  reinterpret_cast<uintptr_t>(a->d_c2p_bias) % group_bytes || reinterpret_cast<uintptr_t>(a->d_p2c_bias) % group_bytes ||
+                  // ... and the scores arrive in aligned 32-bit words (two 16-bit entries)
+                  reinterpret_cast<uintptr_t>(a->c2p_bias) % 4 || reinterpret_cast<uintptr_t>(a->p2c_bias) % 4))
     return FDB_ERR_ALIGN;
   const int sz = qk_elem_size(a->dtype);
   const void* ptrs[] = {a->q, a->k, a->v, a->dout, a->dq, a->dk, a->dv, a->out};

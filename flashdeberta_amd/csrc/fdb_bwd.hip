@@ -26,6 +26,10 @@
 // do not depend on the order workgroups run in.
 // A step whose relative positions all lie beyond the table radius has one table row: its position scores are
 // one load per row and its score gradients enter the ring as one row sum per lane.
+// In a near block the loop side's scores are one load per element (a wave instruction reads neighbouring entries of one
+// or two rows); the lane side's, where every lane has its own row (64 cache lines per instruction), come as one 12-byte
+// load per group of four neighbouring loop rows -- six consecutive entries that hold the group's four table rows
+// whenever the table moves by at most one row per position -- and the element is picked from the three registers.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -109,6 +113,11 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
   if (m0 >= Lb) return;
   if (C2P || P2C)
     for (int x = tid; x < 2 * p.R + 1; x += kBwdThreads) lut_s[x] = p.lut[x];
+  // grp_ok: four consecutive relative positions never span more than four table rows (steps of 0 or 1, the usual
+  // case): the lane side's scores of four neighbouring loop rows then sit within six consecutive entries of the lane's
+  // row and are fetched as one 12-byte load (see request_near).  Every wave checks the table for itself once it is
+  // in LDS.
+  bool grp_ok = false;
 
   auto base = [&](const char* ptr, int64_t sb, int64_t st, int64_t sh) {
     return ptr + (b * sb + (int64_t)tok0 * st + (int64_t)h * sh) * QT::SZ;
@@ -260,22 +269,62 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
       if (kLoopT) raw_loop[0] = loop_t[loop_off(y0 + li) + (uint32_t)dfar_n];
     }
   };
+  // The loop over the other side, written once and compiled twice: GRP says whether the lane side's near scores are
+  // fetched in groups (see grp_ok); the two copies keep their own registers.
+  auto run = [&](auto grp_tag) __attribute__((always_inline)) {
+  constexpr bool GRP = decltype(grp_tag)::value;
   // The table rows of a near block's 16 elements stay with the lane until the block's score gradients are added: as
   // offsets (0..31) from the first entry of the lane row's window, four to a register.
   int d_lo = 0;
   uint32_t off4[4] = {0u, 0u, 0u, 0u};
+  typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
+  u32x3 raw3[4];         // grouped form of the lane side's scores: six consecutive 16-bit entries per group of four elements
+  uint32_t goff = 0u;    // ... and where in them the group's lowest table row sits (0..5), four bits per group
+#pragma unroll
+  for (int q4 = 0; q4 < 4; ++q4) raw3[q4] = u32x3{0u, 0u, 0u};
+  const uint32_t x_last = x_off + (uint32_t)(2 * p.S) - 6u;   // last even start whose six entries stay inside the row
   auto request_near = [&](int y0) __attribute__((always_inline)) {
     if (!kBias || far_n) return;
     d_lo = delta_of(kDQ ? xr - (y0 + kBwdStep - 1) : y0 - xr);
     off4[0] = off4[1] = off4[2] = off4[3] = 0u;
+    if constexpr (kLaneT && sizeof(BT) == 2) {
+      if (GRP) {
+      goff = 0u;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int yr = y0 + 8 * (v >> 2) + 4 * g + (v & 3);
-      const int dl = delta_of(kDQ ? xr - yr : yr - xr);
-      off4[v >> 2] |= (uint32_t)(dl - d_lo) << (8 * (v & 3));
-      if (kLaneT) raw_lane[v] = lane_t[x_off + (uint32_t)dl];
-      if (kLoopT) raw_loop[v] = loop_t[loop_off(yr) + (uint32_t)dl];
+      for (int q4 = 0; q4 < 4; ++q4) {
+        int dmin = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int v = 4 * q4 + e;
+          const int yr = y0 + 8 * q4 + 4 * g + e;
+          const int dl = delta_of(kDQ ? xr - yr : yr - xr);
+          off4[q4] |= (uint32_t)(dl - d_lo) << (8 * e);
+          if (e == (kDQ ? 3 : 0)) dmin = dl;   // the table row falls (dQ role) or rises (dK/dV role) with the loop row
+          if (kLoopT) raw_loop[v] = loop_t[loop_off(yr) + (uint32_t)dl];
+        }
+        const uint32_t first = x_off + (uint32_t)dmin;
+        const uint32_t start = min(first & ~1u, x_last);
+        goff |= (first - start) << (4 * q4);
+        raw3[q4] = *(const u32x3*)(lane_t + start);
+      }
+      return;
+      }
     }
+    {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int yr = y0 + 8 * (v >> 2) + 4 * g + (v & 3);
+        const int dl = delta_of(kDQ ? xr - yr : yr - xr);
+        off4[v >> 2] |= (uint32_t)(dl - d_lo) << (8 * (v & 3));
+        if (kLaneT) raw_lane[v] = lane_t[x_off + (uint32_t)dl];
+        if (kLoopT) raw_loop[v] = loop_t[loop_off(yr) + (uint32_t)dl];
+      }
+    }
+  };
+  // entry `idx` (0..5) of six consecutive 16-bit entries held in three registers
+  auto entry16 = [&](const u32x3& w, uint32_t idx) __attribute__((always_inline)) -> uint16_t {
+    const uint32_t lo = idx < 2u ? w[0] : (idx < 4u ? w[1] : w[2]);
+    return (uint16_t)((idx & 1u) ? lo >> 16 : lo);
   };
   if (y_lo < y_hi) {
     tiles_dma(y_lo, 0);
@@ -294,6 +343,7 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
   // waits for where it uses them.
   constexpr int kAsked = (kLaneT ? 1 : 0) + (kLoopT ? 1 : 0);
   if (far_n) wait_vmcnt<kAsked>();
+  else if (kLaneT && GRP) wait_vmcnt<4 + (kLoopT ? 16 : 0)>();
   else wait_vmcnt<16 * kAsked>();
   __syncthreads();   // ... and everybody's; every wave is done with the other buffer (and the table is in LDS)
   const bool next_tiles = yt + C::TROWS < y_hi;
@@ -318,8 +368,19 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
     if (kBias && far) {
       sacc = rank1_start<QT>(kLaneT ? (float)raw_lane[0] : 0.f, kLoopT ? (float)raw_loop[0] : 0.f, g);
     } else {
+      bool grouped = false;
+      if constexpr (kLaneT && sizeof(BT) == 2) grouped = GRP;
+      if (grouped) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) sacc[v] = (float)raw_lane[v] + (float)raw_loop[v];
+        for (int v = 0; v < 16; ++v) {
+          const uint32_t o4 = off4[v >> 2];
+          const uint32_t idx = ((goff >> (4 * (v >> 2))) & 7u) + ((o4 >> (8 * (v & 3))) & 255u) - ((o4 >> (kDQ ? 24 : 0)) & 255u);
+          if constexpr (sizeof(BT) == 2) sacc[v] = QT::scratch_to_f32(entry16(raw3[v >> 2], idx)) + (float)raw_loop[v];
+        }
+      } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) sacc[v] = (float)raw_lane[v] + (float)raw_loop[v];
+      }
     }
     if (has_next) request_far(y0 + kBwdStep);
 #pragma unroll
@@ -460,6 +521,16 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
   }
   if (next_tiles) stats_store(buf ^ 1);
   }
+
+  };
+  if (kBias && sizeof(typename QT::scratch_t) == 2) {
+    __syncthreads();  // the table is in LDS
+    bool wide = false;
+    for (int x = lane; x + 3 < 2 * p.R + 1; x += 64) wide |= lut_s[x + 3] - lut_s[x] > 3 || lut_s[x + 3] < lut_s[x];
+    grp_ok = __builtin_amdgcn_ballot_w64(wide) == 0;
+  }
+  if (grp_ok) run(std::true_type{});
+  else run(std::false_type{});
 
   if (!x_ok) return;
   auto write = [&](char* ptr, int64_t sb, int64_t st, int64_t sh, const f32x16 (&acc)[DBLKS]) {

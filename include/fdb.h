@@ -181,7 +181,7 @@ int fdb_attn_fwd_noalloc(const fdb_attn_args* a, void* stream);
  * is stored once, by plain stores in aligned groups of four, if any score maps to its group, and not touched
  * otherwise.  The four tensors share one layout: element (b, l, h, delta) at b * bias_stride_b + l * bias_stride_t
  * + h * bias_stride_h + delta (strides in elements, multiples of 4; 2S a multiple of 4; the gradient tensors
- * aligned to four elements; l * bias_stride_t + delta must stay below 2^31).  Head-major [H, B, L, 2S] is what a batched
+ * aligned to four elements, the score tensors to four bytes; l * bias_stride_t + delta must stay below 2^31).  Head-major [H, B, L, 2S] is what a batched
  * GEMM over the heads writes and reads without a transpose.  The chain through K_r / Q_r and into q / k is the
  * caller's GEMMs.
  * dq, dk, dv hold only the content part,

@@ -506,6 +506,7 @@ def test_backward_argument_validation_codes():
     a = _good_bwd_args(); a.att_span = 255; a.bias_stride_t = 512; assert call(a) == -4   # 2S must be a multiple of 4
     a = _good_bwd_args(); a.bias_stride_h = 2 * 512 * 512 + 2; assert call(a) == -4
     a = _good_bwd_args(); a.d_p2c_bias = 0x4004; assert call(a) == -4      # a store group is four elements
+    a = _good_bwd_args(); a.c2p_bias = 0x3002; assert call(a) == -4        # the scores are read as aligned 32-bit words
     a = _good_bwd_args(); a.d_p2c_bias = 0x4008; a.seqlen = 0; assert call(a) == -5       # (8-byte alignment is enough for 16-bit types)
     a = _good_bwd_args(); a.bias_stride_t = 500; assert call(a) == -5      # rows shorter than 2S
     a = _good_bwd_args(); a.seqlen, a.bias_stride_t = 1 << 20, 1 << 12; assert call(a) == -5  # 32-bit offsets

@@ -1222,6 +1222,8 @@ BWD_CASES = [
     (1, 150, 2, 128, 32, 64, True, True, False, None),
     (1, 600, 1, 64, 0, 300, True, True, False, None),     # no buckets: 600 table rows, every block linear
     (1, 1100, 2, 64, 256, 512, True, True, False, None),  # v3 buckets past the radius: far steps on both sides of every zone
+    (2, 200, 2, 64, 32, 22, True, True, False, None),     # a steep table (four neighbouring positions span up to ten rows):
+    (1, 150, 2, 64, 16, 16, True, True, True, None),      # ... the lane side's near scores are then fetched one by one
 ]
 
 
