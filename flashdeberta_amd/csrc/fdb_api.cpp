@@ -140,12 +140,15 @@ int far_parts_wanted(const fdb_attn_args* a) {
 int near_parts_wanted(const fdb_attn_args* a) {
   if (!(a->pos_key || a->pos_query) || !a->lse || !steps32_supported(a->dtype, a->head_dim)) return 1;
   if (a->near_splits > 0) return a->near_splits;
-  if (a->cu_seqlens) return 1;
+  // A packed batch has its lengths on the device: the host goes by the mean length and by the most query tiles the
+  // token count allows (the kernel divides each query tile's own steps among the shares, whatever they are).
+  const int32_t typical = a->cu_seqlens ? a->total_tokens / a->batch : a->max_seqlen;
   const int64_t wgs = query_tiles(a) * a->heads, slots = 2 * (int64_t)cu_count();
-  const int steps_all = (a->max_seqlen + 31) / 32, steps_near = (FDB_BM + 2 * a->lut_radius + 3 * (FDB_BN - 1)) / 32;
+  const int steps_all = (typical + 31) / 32, steps_near = (FDB_BM + 2 * a->lut_radius + 3 * (FDB_BN - 1)) / 32;
   const int steps = steps_all < steps_near ? steps_all : steps_near;
   int best = 1;
-  for (int n = 2; n <= FDB_MAX_FAR_PARTS && (wgs * n <= slots || (n == 2 && wgs * 10 <= slots * 7)); ++n) {
+  // (packed batches only share when all shares fit in one round: three sequences of 1000 lose 10 % to two shares)
+  for (int n = 2; n <= FDB_MAX_FAR_PARTS && (wgs * n <= slots || (n == 2 && !a->cu_seqlens && wgs * 10 <= slots * 7)); ++n) {
     const int per = steps / n;
     if (per >= 16 || (per >= 8 && wgs * n <= slots / 2)) best = n;
   }

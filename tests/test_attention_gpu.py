@@ -303,6 +303,22 @@ def test_far_keys_shared_packed_and_padded():
         off += n
 
 
+def test_packed_batch_of_one_short_sequence_shares_near_steps_by_itself():
+    """A packed batch whose token count leaves most of the GPU idle shares the near steps of a query tile among
+    workgroups by the library's own choice (no near_splits): same result as unshared, both match the oracle."""
+    pb, mr, H, D, L = 256, 512, 12, 64, 1024
+    q, k, v, pk, pq = _inputs(1, L, H, D, pb, mr, torch.bfloat16, 612, 1.0)
+    cu = torch.tensor([0, L], dtype=torch.int32).cuda()
+    kw = dict(position_buckets=pb, max_relative_positions=mr, cu_seqlens=cu, max_seqlen=L)
+    args = [_dev(q[0]), _dev(k[0]), _dev(v[0]), _dev(pk), _dev(pq)]
+    auto = ops.disentangled_attention_fwd(*args, **kw)
+    one = ops.disentangled_attention_fwd(*args, near_splits=1, far_splits=1, **kw)
+    ref = _oracle_blhd(q, k, v, pk, pq, pb, mr)
+    _check(auto[None], ref, TOL[torch.bfloat16], "library's choice")
+    _check(one[None], ref, TOL[torch.bfloat16], "unshared")
+    assert (auto.float() - one.float()).abs().max().item() <= TOL[torch.bfloat16]
+
+
 @pytest.mark.parametrize("B,L,splits,near", [(2, 700, 0, 1), (1, 1500, 2, 0), (1, 1500, 2, 3)])
 def test_operator_replays_from_a_hip_graph(B, L, splits, near):
     """The operator enqueues only kernels on the current stream and allocates through torch, so it can be
