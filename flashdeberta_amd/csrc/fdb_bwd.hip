@@ -65,7 +65,7 @@ struct BCfg {
   static constexpr int TILE = TROWS * RS;                    // a multiple of 1024: RS is a multiple of 16
   static constexpr int REGION = 2 * TILE;                    // [Y1 tile | Y2 tile] of one buffer
   // two buffers, loop-row statistics, ring windows, groups to store; the table follows
-  static constexpr int fixed_lds_bytes() { return 2 * REGION + 4 * TROWS * 4 + FDB_BM * kRingStrideMax * 4 + FDB_BM * 8; }
+  static constexpr int fixed_lds_bytes() { return 2 * REGION + 4 * 64 * 4 + FDB_BM * kRingStrideMax * 4 + FDB_BM * 8; }
   static int lds_bytes(int radius) { return fixed_lds_bytes() + (((2 * radius + 1) * 2 + 15) & ~15); }
 };
 
@@ -98,8 +98,8 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
   constexpr int kRingStride = ring_stride(kDQ);
   extern __shared__ __attribute__((aligned(16))) char smem[];
   char* Ys = smem;                                    // two buffers of [K | V] (dQ role) / [Q | dO] (dK/dV role)
-  float* stat_s = (float*)(Ys + 2 * C::REGION);       // dK/dV role: per buffer, log-sum-exp (base 2) and Delta of the staged loop rows
-  float* ring_s = stat_s + 4 * C::TROWS;              // [128 lane-side rows][kRingStride] score-gradient windows
+  float* stat_s = (float*)(Ys + 2 * C::REGION);       // dK/dV role: per buffer, log-sum-exp and Delta of the staged loop rows (64 floats each)
+  float* ring_s = stat_s + 4 * 64;              // [128 lane-side rows][kRingStride] score-gradient windows
   int2* inf_s = (int2*)(ring_s + FDB_BM * kRingStrideMax);  // [4 waves][32] (first group, groups) to store per row
   LDS_AS int16_t* lut_s = (LDS_AS int16_t*)(inf_s + FDB_BM);  // the whole table (the launcher sizes the allocation for it)
 
@@ -223,19 +223,15 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
       }
     }
   };
-  float st_reg[2] = {0.f, 0.f};
-  auto stats_load = [&](int r0) __attribute__((always_inline)) {
-    if (!kDQ && tid < C::TROWS) {
-      const int row = min(r0 + tid, Lb - 1);
-      const int64_t t = ((int64_t)b * p.L + tok0 + row) * p.H + h;
-      st_reg[0] = p.lse[t];   // used (scaled to base 2) only when stored: a use here would wait for the loads at once
-      st_reg[1] = p.delta[t];
-    }
-  };
-  auto stats_store = [&](int buf) __attribute__((always_inline)) {
-    if (!kDQ && tid < C::TROWS) {
-      stat_s[buf * 2 * C::TROWS + tid] = st_reg[0] * 1.4426950408889634f;
-      stat_s[buf * 2 * C::TROWS + C::TROWS + tid] = st_reg[1];
+  // The statistics of the staged loop rows (dK/dV role) travel like the tiles, from global memory straight into LDS:
+  // wave 0 fetches the log-sum-exps, wave 1 the Deltas, one row per lane, and the wait and the barrier that cover
+  // the tiles cover them.  (Through registers, the wave that fetched them waited at its store for every load it had
+  // issued since, the next block's position scores among them, and the other waves waited for it at the barrier.)
+  auto stats_dma = [&](int r0, int buf) __attribute__((always_inline)) {
+    if (!kDQ && wave < 2) {
+      const int row = min(r0 + lane, Lb - 1);
+      const float* src = (wave == 0 ? p.lse : p.delta) + (((int64_t)b * p.L + tok0 + row) * p.H + h);
+      dma4(src, lds0 + (uint32_t)((const char*)stat_s - smem) + (uint32_t)((buf * 2 + wave) * 64 * 4));
     }
   };
   // Position scores of a step are requested one step ahead (their addresses depend on indices only), so that their
@@ -328,12 +324,11 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
   };
   if (y_lo < y_hi) {
     tiles_dma(y_lo, 0);
-    stats_load(y_lo);
+    stats_dma(y_lo, 0);
     __syncthreads();  // the table is in LDS
     if (kGrad) g_next = delta_of(kDQ ? xr - y_lo : y_lo - xr) >> 2;
     request_far(y_lo);
     request_near(y_lo);
-    stats_store(0);
   }
 
   int buf = 0;
@@ -349,7 +344,7 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
   const bool next_tiles = yt + C::TROWS < y_hi;
   if (next_tiles) {
     tiles_dma(yt + C::TROWS, buf ^ 1);
-    stats_load(yt + C::TROWS);
+    stats_dma(yt + C::TROWS, buf ^ 1);
   }
 #pragma unroll 1
   for (int sub = 0; sub < C::TROWS / kBwdStep; ++sub) {
@@ -358,8 +353,8 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
     const bool has_next = y0 + kBwdStep < y_hi;
     const char* Y1s = Ys + buf * C::REGION + sub * kBwdStep * C::RS;
     const char* Y2s = Y1s + C::TILE;
-    const float* lse_s = stat_s + buf * 2 * C::TROWS + sub * kBwdStep;
-    const float* del_s = lse_s + C::TROWS;
+    const float* lse_s = stat_s + buf * 2 * 64 + sub * kBwdStep;
+    const float* del_s = lse_s + 64;
     // ---- position scores (requested during the step before) ---------------------------------------------------
     // element v of lane (g, li): loop row yr = y0 + 8*(v/4) + 4g + v%4, lane row xr; i - j = +-(xr - yr)
     const bool far = far_n;
@@ -409,7 +404,7 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
         f32x4 lse4 = {lse_x, lse_x, lse_x, lse_x};
-        if (!kDQ) lse4 = *(const f32x4*)(lse_s + 8 * q4 + 4 * g);
+        if (!kDQ) lse4 = *(const f32x4*)(lse_s + 8 * q4 + 4 * g) * 1.4426950408889634f;   // to base 2, like lse_x
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int v = 4 * q4 + e;
@@ -519,7 +514,6 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
       }
     }
   }
-  if (next_tiles) stats_store(buf ^ 1);
   }
 
   };

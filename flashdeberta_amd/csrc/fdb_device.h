@@ -300,6 +300,13 @@ __device__ __forceinline__ void dma16(const void* g, uint32_t lds_base) {
   asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0"
                : "=&s"(keep) : "v"(g), "s"(base) : "memory");
 }
+// One dword per lane, global memory -> LDS at lds_base + 4 * lane.
+__device__ __forceinline__ void dma4(const void* g, uint32_t lds_base) {
+  const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);
+  uint32_t keep;
+  asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %1, off\n\ts_mov_b32 m0, %0"
+               : "=&s"(keep) : "v"(g), "s"(base) : "memory");
+}
 // The same with the address split into a base that is the same in every lane (it travels in scalar
 // registers) and this lane's 32-bit byte offset from it.
 __device__ __forceinline__ void dma16s(const void* base, uint32_t lane_off, uint32_t lds_base) {
