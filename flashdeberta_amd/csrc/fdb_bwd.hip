@@ -22,7 +22,8 @@
 // which 32 consecutive relative positions span more than 61 rows (steps of 0 or 1, the usual case, span at most 32):
 // a 64-entry ring per row in LDS takes the adds, and the entries the window has left behind are stored
 // once, in aligned groups of four (eight lanes per row, one 16- or 8-byte store each), and cleared.  The tensors have
-// the element type of q and arrive zeroed; entries no element maps to are written as zeros or not at all.  Results
+// the element type of q; the entries of a real token's row that no element maps to are written as zeros (in the loop or after it),
+// rows of padding are not touched.  Results
 // do not depend on the order workgroups run in.
 // A step whose relative positions all lie beyond the table radius has one table row: its position scores are
 // one load per row and its score gradients enter the ring as one row sum per lane.
@@ -525,6 +526,26 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
   }
   if (grp_ok) run(std::true_type{});
   else run(std::false_type{});
+
+  // The groups of a row that the loop never reached (table rows beyond the ones its relative positions map to: rows
+  // near the ends of a sequence, and half of every row of a causal call) are written as zeros here, so that every
+  // entry of a real token's row is stored exactly once and the caller need not clear the tensor.
+  if (kGrad) {
+    const int g_first = delta_of(kDQ ? xr - y_lo : y_lo - xr) >> 2;        // where the loop began; g_next: one past where it ended
+    const int lo = kDir < 0 ? g_next + 1 : g_first, hi = kDir < 0 ? g_first : g_next - 1;
+    const int n_groups = (2 * p.S) >> 2;
+    if (g == 0) inf_w[li] = x_ok ? int2{lo, hi} : int2{0, n_groups - 1};   // rows past the end: nothing to write
+    wave_lds_fence();
+#pragma unroll 1
+    for (int it = 0; it < 4; ++it) {
+      const int rho = 8 * it + (lane >> 3);
+      const int2 inf = inf_w[rho];
+      if (__builtin_amdgcn_ballot_w64(inf.x > 0 || inf.y < n_groups - 1) == 0) continue;
+      for (int m = lane & 7; m < n_groups; m += 8)
+        if (m < inf.x || m > inf.y)
+          QT::store4(gw + ((uint32_t)(xw0 + rho) * row_elems + (uint32_t)(4 * m)) * QT::SZ, 0.f, 0.f, 0.f, 0.f);
+    }
+  }
 
   if (!x_ok) return;
   auto write = [&](char* ptr, int64_t sb, int64_t st, int64_t sh, const f32x16 (&acc)[DBLKS]) {

@@ -64,7 +64,7 @@ struct FdbBwdParams {
   const char* out;      // the forward's output or NULL
   const char* c2p;      // q_i . K_r[delta] or NULL; element type of q, like the gradient tensors below
   const char* p2c;      // k_j . Q_r[delta] or NULL
-  char* d_c2p;          // element type of q; zero-initialised by the caller; touched entries are stored once
+  char* d_c2p;          // element type of q; every entry of a real token's row is stored once, rows of padding are not touched
   char* d_p2c;
   const int32_t* seq_start;
   const int32_t* seq_len;

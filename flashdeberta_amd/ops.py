@@ -251,7 +251,8 @@ def attention_bwd_kernels(q, k, v, dout, lse, *, out=None, delta=None, c2p=None,
                           position_buckets=0, max_relative_positions=0, causal=False, seq_start=None, seq_len=None):
     """The two backward launches (fdb_attn_bwd) on tensors the caller made: q, k, v, dout [B, L, H, D]; lse [B*L, H];
     either `out` (the forward's output; the call then computes delta itself) or `delta` [B*L, H] fp32; the position
-    scores c2p = q . K_r^T / p2c = k . Q_r^T and their zeroed gradient tensors as views of logical shape
+    scores c2p = q . K_r^T / p2c = k . Q_r^T and their gradient tensors (cleared by the caller if the batch is padded: the
+    kernels store every entry of a real token's row and leave rows of padding alone) as views of logical shape
     [B, L, H, 2S] with a unit stride on the last axis and any memory layout behind it (all four the same, in q's
     element type).  Returns dq, dk, dv (content part) and leaves the score gradients in d_c2p / d_p2c."""
     B, L, H, D = q.shape
@@ -334,6 +335,8 @@ def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=
     # writes and reads as it stands (a token-major tensor would cost a transposing copy of it each way).
     heads_first = lambda x: x.permute(2, 0, 1, 3).reshape(H, B * L, D)  # a view of [B, L, H, D] when that is contiguous
     both = pos_key is not None and pos_query is not None
+    # the kernels store every entry of a real token's row of the score gradients; only rows of padding need clearing
+    like = torch.zeros_like if (seq_start is not None or seq_len is not None) else torch.empty_like
     if both:
         # both terms: their tensors stacked, [2H, B*L, ...], so that each GEMM around the kernel is one call over 2H
         # matrices instead of two over H (a third less time at 4 k tokens; the reduction over tokens, which has few
@@ -341,14 +344,14 @@ def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=
         x2 = torch.stack([heads_first(q), heads_first(k)]).view(2 * H, B * L, D)
         pos2 = torch.stack([pos_key[:, :2 * span], pos_query[:, :2 * span]]).view(2 * H, 2 * span, D).to(q.dtype)
         scores2 = torch.bmm(x2, pos2.transpose(1, 2))        # [2H, B*L, 2S] = (q . K_r^T, k . Q_r^T), in the inputs' type like the reference's
-        d_scores2 = torch.zeros_like(scores2)
+        d_scores2 = like(scores2)
         c2p, p2c, d_c2p, d_p2c = scores2[:H], scores2[H:], d_scores2[:H], d_scores2[H:]
     elif pos_key is not None:
         c2p = torch.bmm(heads_first(q), pos_key[:, :2 * span].transpose(1, 2).to(q.dtype))
-        d_c2p = torch.zeros_like(c2p)
+        d_c2p = like(c2p)
     elif pos_query is not None:
         p2c = torch.bmm(heads_first(k), pos_query[:, :2 * span].transpose(1, 2).to(k.dtype))
-        d_p2c = torch.zeros_like(p2c)
+        d_p2c = like(p2c)
     blhs = lambda x: None if x is None else x.view(H, B, L, 2 * span).permute(1, 2, 0, 3)  # the logical [B, L, H, 2S] view
     dq, dk, dv = attention_bwd_kernels(q, k, v, dout, lse, out=out, delta=delta, c2p=blhs(c2p), p2c=blhs(p2c), d_c2p=blhs(d_c2p),
                                        d_p2c=blhs(d_p2c), sm_scale=sm_scale, position_buckets=position_buckets,

@@ -177,9 +177,10 @@ int fdb_attn_fwd_noalloc(const fdb_attn_args* a, void* stream);
  * FlashAttentionDisentangled.backward (:1066-1086).  Same division of labour as there: the position scores come
  * in as tensors, c2p_bias[b,l,h,delta] = q . K_r[delta] and p2c_bias[b,l,h,delta] = k . Q_r[delta], and the
  * gradients with respect to them leave in d_c2p_bias / d_p2c_bias; all four have the element type of `dtype`,
- * like the reference's ([B,H,L,2S] in the input dtype).  The gradient tensors are ZEROED BY THE CALLER: an entry
- * is stored once, by plain stores in aligned groups of four, if any score maps to its group, and not touched
- * otherwise.  The four tensors share one layout: element (b, l, h, delta) at b * bias_stride_b + l * bias_stride_t
+ * like the reference's ([B,H,L,2S] in the input dtype).  Every entry of the gradient tensors that belongs to a
+ * real token (batch row b, seq_start[b] <= l < seq_start[b] + seq_len[b]) is stored exactly once, by plain stores in
+ * aligned groups of four (zeros where no score maps to it); rows of padding are not touched, so a caller with a padded
+ * batch clears the tensors first.  The four tensors share one layout: element (b, l, h, delta) at b * bias_stride_b + l * bias_stride_t
  * + h * bias_stride_h + delta (strides in elements, multiples of 4; 2S a multiple of 4; the gradient tensors
  * aligned to four elements, the score tensors to four bytes; l * bias_stride_t + delta must stay below 2^31).  Head-major [H, B, L, 2S] is what a batched
  * GEMM over the heads writes and reads without a transpose.  The chain through K_r / Q_r and into q / k is the

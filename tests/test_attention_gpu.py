@@ -1761,6 +1761,40 @@ def test_backward_kernels_take_any_layout_of_the_score_tensors(dtype):
                                   d_c2p=torch.zeros_like(c2p), d_p2c=torch.zeros_like(p2c), sm_scale=0.07, **kw)
 
 
+@pytest.mark.parametrize("L,pb,mr,causal,lens", [
+    (300, 32, 64, False, None),      # rows near either end reach only part of the table
+    (40, 8, 16, True, None),         # causal: half of every row is never reached
+    (700, 256, 512, False, None),    # v3 buckets, shorter than the table radius
+    (1100, 256, 512, True, None),
+    (333, 32, 64, False, [333, 150]),  # padded batch: rows of padding stay as the caller left them
+])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_backward_stores_every_entry_of_a_real_tokens_row(L, pb, mr, causal, lens, dtype):
+    """The score-gradient tensors need no clearing: handed in full of NaN, every entry of a real token's row comes back
+    as it does from cleared tensors, bit for bit (zeros where no score maps to it), and rows of padding are not touched."""
+    B, H, D = (2 if lens else 1), 2, 64
+    q, k, v, pk, pq = [x.cuda() for x in _inputs(B, L, H, D, pb, mr, dtype, 4500 + L, 1.0, True, True)]
+    dout = torch.randn(B, L, H, D, generator=torch.Generator().manual_seed(4501)).to(dtype).cuda()
+    kw = dict(position_buckets=pb, max_relative_positions=mr, causal=causal)
+    if lens:
+        kw["seq_len"] = torch.tensor(lens, dtype=torch.int32).cuda()
+    out, lse = ops.disentangled_attention_fwd(q, k, v, pk, pq, return_lse=True, **kw)
+    heads_first = lambda x: x.permute(2, 0, 1, 3).reshape(H, B * L, D)
+    view = lambda x: x.view(H, B, L, -1).permute(1, 2, 0, 3)
+    c2p = view(torch.bmm(heads_first(q), pk.transpose(1, 2)))
+    p2c = view(torch.bmm(heads_first(k), pq.transpose(1, 2)))
+    got = []
+    for fill in (0.0, float("nan")):
+        dc, dp = [view(torch.full((H, B * L, c2p.shape[-1]), fill, dtype=dtype, device="cuda")) for _ in range(2)]
+        ops.attention_bwd_kernels(q, k, v, dout, lse, out=out, c2p=c2p, p2c=p2c, d_c2p=dc, d_p2c=dp, sm_scale=1.0 / np.sqrt(3 * D), **kw)
+        got.append((dc, dp))
+    for b in range(B):
+        n = lens[b] if lens else L
+        for cleared, dirty in zip(got[0], got[1]):
+            assert torch.equal(cleared[b, :n], dirty[b, :n])
+            assert torch.isnan(dirty[b, n:]).all()
+
+
 @pytest.mark.parametrize("what", ["no_alloc_forward", "backward"])
 def test_more_replays_from_a_hip_graph(what):
     """The entry point that allocates nothing (the case it exists for) and the backward operator (two launches and
