@@ -472,9 +472,9 @@ int fdb_attn_bwd(const fdb_attn_bwd_args* a, void* stream) {
   if (has_pos && (a->att_span < 1 || a->lut_radius < 1 || !a->delta_lut)) return FDB_ERR_SPAN;
   // the ring that collects a row's score gradients holds the table rows of one 32-row step plus a partly stored group
   if (has_pos && (a->lut_window < 0 || a->lut_window > FDB_BWD_MAX_WINDOW)) return FDB_ERR_SPAN;
-  // the kernels address a sequence's rows of the position-score tensors with 32-bit element offsets
+  // the kernels address a sequence's rows of the position-score tensors with 32-bit byte offsets
   if (has_pos && (a->bias_stride_t < 2 * a->att_span || a->bias_stride_b < 0 || a->bias_stride_h < 0 ||
-                  (int64_t)a->seqlen * a->bias_stride_t > 0x7fffffffll)) return FDB_ERR_SHAPE;
+                  (int64_t)a->seqlen * a->bias_stride_t * qk_elem_size(a->dtype) > 0xffffffffll)) return FDB_ERR_SHAPE;
   // score gradients leave in aligned groups of four entries
   const uintptr_t group_bytes = 4u * (uintptr_t)qk_elem_size(a->dtype);  // one store: four entries
   if (has_pos && ((a->att_span & 1) || (a->bias_stride_b & 3) || (a->bias_stride_t & 3) || (a->bias_stride_h & 3) ||

@@ -30,7 +30,10 @@
 // In a near block the loop side's scores are one load per element (a wave instruction reads neighbouring entries of one
 // or two rows); the lane side's, where every lane has its own row (64 cache lines per instruction), come as one 12-byte
 // load per group of four neighbouring loop rows -- six consecutive entries that hold the group's four table rows
-// whenever the table moves by at most one row per position -- and the element is picked from the three registers.
+// whenever the table moves by at most one row per position -- and the element is picked from the three registers
+// (one byte permutation per element where the six entries start at the group's first table row or one before it).
+// The table sits in LDS with 64 copies of its end entries on either side, so that the lookups of a near block are one
+// address per step plus a constant per element, without a clamp.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -54,6 +57,9 @@ static_assert(kRing == 64 && FDB_BWD_MAX_WINDOW + 4 <= kRing, "ring slots are ta
 // dK/dV role: -): with stride 65 resp. 67 that is bank 2 * lane, no two lanes alike.
 constexpr int ring_stride(bool dq) { return dq ? kRing + 1 : kRing + 3; }
 constexpr int kRingStrideMax = kRing + 3;
+// The table in LDS carries this many copies of its first and of its last entry before and after it: the relative
+// positions of a near block reach at most 62 beyond the radius, so its lookups need no clamp.
+constexpr int kLutPad = 64;
 
 template <class QT, int D>
 struct BCfg {
@@ -67,7 +73,7 @@ struct BCfg {
   static constexpr int REGION = 2 * TILE;                    // [Y1 tile | Y2 tile] of one buffer
   // two buffers, loop-row statistics, ring windows, groups to store; the table follows
   static constexpr int fixed_lds_bytes() { return 2 * REGION + 4 * 64 * 4 + FDB_BM * kRingStrideMax * 4 + FDB_BM * 8; }
-  static int lds_bytes(int radius) { return fixed_lds_bytes() + (((2 * radius + 1) * 2 + 15) & ~15); }
+  static int lds_bytes(int radius) { return fixed_lds_bytes() + (((2 * radius + 1 + 2 * kLutPad) * 2 + 15) & ~15); }
 };
 
 // acc[m][n] = a_lane(n) + b_loop(m) as one MFMA: the start of S' in a block with a single table row, where the
@@ -102,7 +108,8 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
   float* stat_s = (float*)(Ys + 2 * C::REGION);       // dK/dV role: per buffer, log-sum-exp and Delta of the staged loop rows (64 floats each)
   float* ring_s = stat_s + 4 * 64;              // [128 lane-side rows][kRingStride] score-gradient windows
   int2* inf_s = (int2*)(ring_s + FDB_BM * kRingStrideMax);  // [4 waves][32] (first group, groups) to store per row
-  LDS_AS int16_t* lut_s = (LDS_AS int16_t*)(inf_s + FDB_BM);  // the whole table (the launcher sizes the allocation for it)
+  LDS_AS int16_t* lut_pad = (LDS_AS int16_t*)(inf_s + FDB_BM);  // the whole table, padded (the launcher sizes the allocation for it)
+  LDS_AS int16_t* lut_s = lut_pad + kLutPad;
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -113,7 +120,7 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
   const int Lb = p.seq_len ? min(max(p.seq_len[b], 0), p.L - tok0) : p.L;
   if (m0 >= Lb) return;
   if (C2P || P2C)
-    for (int x = tid; x < 2 * p.R + 1; x += kBwdThreads) lut_s[x] = p.lut[x];
+    for (int x = tid; x < 2 * p.R + 1 + 2 * kLutPad; x += kBwdThreads) lut_pad[x] = p.lut[min(max(x - kLutPad, 0), 2 * p.R)];
   // grp_ok: four consecutive relative positions never span more than four table rows (steps of 0 or 1, the usual
   // case): the lane side's scores of four neighbouring loop rows then sit within six consecutive entries of the lane's
   // row and are fetched as one 12-byte load (see request_near).  Every wave checks the table for itself once it is
@@ -254,7 +261,7 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
     return (uint32_t)min(yr, Lb - 1) * row_elems;
   };
   // Classifies the wave's block of the step at y0 and, if it is far, asks for its two values right away (they cost two
-  // registers); the 32 values of a near block are asked for later in the step by request_near (they would sit in 32).
+  // registers); the values of a near block are asked for by request_near right after (28 registers in the grouped form).
   auto request_far = [&](int y0) __attribute__((always_inline)) {
     if (!kBias) return;
     const int r_min = kDQ ? xw0 - (y0 + kBwdStep - 1) : y0 - (xw0 + 31);      // over the wave's 32 x 32 block
@@ -272,18 +279,27 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
   constexpr bool GRP = decltype(grp_tag)::value;
   // The table rows of a near block's 16 elements stay with the lane until the block's score gradients are added: as
   // offsets (0..31) from the first entry of the lane row's window, four to a register.
-  int d_lo = 0;
-  uint32_t off4[4] = {0u, 0u, 0u, 0u};
+  int d_lo = 0, d_lo_n = 0;            // ... of the current step and of the one asked for
+  uint32_t off4[4] = {0u, 0u, 0u, 0u}, off4_n[4] = {0u, 0u, 0u, 0u};
   typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
   u32x3 raw3[4];         // grouped form of the lane side's scores: six consecutive 16-bit entries per group of four elements
   uint32_t goff = 0u;    // ... and where in them the group's lowest table row sits (0..5), four bits per group
 #pragma unroll
   for (int q4 = 0; q4 < 4; ++q4) raw3[q4] = u32x3{0u, 0u, 0u};
   const uint32_t x_last = x_off + (uint32_t)(2 * p.S) - 6u;   // last even start whose six entries stay inside the row
+  // Table row of element (q4, e) of this lane in the step at y0: relative position xr - yr (dQ role) or yr - xr with
+  // yr = y0 + 8 q4 + 4 g + e, looked up in the padded table at one address per step plus a constant per element.
+  const int lut_lane = kDQ ? xr - 4 * g + p.R - 27 : p.R + 4 * g - xr;
   auto request_near = [&](int y0) __attribute__((always_inline)) {
     if (!kBias || far_n) return;
-    d_lo = delta_of(kDQ ? xr - (y0 + kBwdStep - 1) : y0 - xr);
-    off4[0] = off4[1] = off4[2] = off4[3] = 0u;
+    volatile LDS_AS const int16_t* lut_e = lut_s + (kDQ ? lut_lane - y0 : lut_lane + y0);  // volatile: merged into 8-byte reads at 2-byte alignment they would be served lane by lane
+    const uint32_t row_bytes = row_elems * (uint32_t)sizeof(BT), last_row = (uint32_t)(Lb - 1) * row_bytes;
+    const uint32_t rowb = (uint32_t)(y0 + 4 * g) * row_bytes;   // byte offset of the loop row of element 0; rows past the end re-read the last one
+    int dls[16];   // all lookups first: the reads are volatile and stay in this order, so none waits for a use before it
+#pragma unroll
+    for (int v = 0; v < 16; ++v) dls[v] = (int)lut_e[kDQ ? 27 - (8 * (v >> 2) + (v & 3)) : 8 * (v >> 2) + (v & 3)];
+    d_lo_n = (int)lut_e[kDQ ? 4 * g - 4 : -4 * g];   // the step's lowest table row of this lane's row: loop row y0 + 31 (dQ role) or y0
+    off4_n[0] = off4_n[1] = off4_n[2] = off4_n[3] = 0u;
     if constexpr (kLaneT && sizeof(BT) == 2) {
       if (GRP) {
       goff = 0u;
@@ -292,12 +308,11 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
         int dmin = 0;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const int v = 4 * q4 + e;
-          const int yr = y0 + 8 * q4 + 4 * g + e;
-          const int dl = delta_of(kDQ ? xr - yr : yr - xr);
-          off4[q4] |= (uint32_t)(dl - d_lo) << (8 * e);
+          const int v = 8 * q4 + e;
+          const int dl = dls[4 * q4 + e];
+          off4_n[q4] |= (uint32_t)(dl - d_lo_n) << (8 * e);
           if (e == (kDQ ? 3 : 0)) dmin = dl;   // the table row falls (dQ role) or rises (dK/dV role) with the loop row
-          if (kLoopT) raw_loop[v] = loop_t[loop_off(yr) + (uint32_t)dl];
+          if (kLoopT) raw_loop[4 * q4 + e] = *(const BT*)((const char*)loop_t + (min(rowb + (uint32_t)v * row_bytes, last_row) + (uint32_t)dl * (uint32_t)sizeof(BT)));
         }
         const uint32_t first = x_off + (uint32_t)dmin;
         const uint32_t start = min(first & ~1u, x_last);
@@ -310,11 +325,11 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
     {
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int yr = y0 + 8 * (v >> 2) + 4 * g + (v & 3);
-        const int dl = delta_of(kDQ ? xr - yr : yr - xr);
-        off4[v >> 2] |= (uint32_t)(dl - d_lo) << (8 * (v & 3));
+        const int ve = 8 * (v >> 2) + (v & 3);
+        const int dl = dls[v];
+        off4_n[v >> 2] |= (uint32_t)(dl - d_lo_n) << (8 * (v & 3));
         if (kLaneT) raw_lane[v] = lane_t[x_off + (uint32_t)dl];
-        if (kLoopT) raw_loop[v] = loop_t[loop_off(yr) + (uint32_t)dl];
+        if (kLoopT) raw_loop[v] = *(const BT*)((const char*)loop_t + (min(rowb + (uint32_t)ve * row_bytes, last_row) + (uint32_t)dl * (uint32_t)sizeof(BT)));
       }
     }
   };
@@ -334,9 +349,10 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
 
   int buf = 0;
   for (int yt = y_lo; yt < y_hi; yt += C::TROWS, buf ^= 1) {
-  // This wave's share of the buffer has landed: loads complete in issue order, and the only younger ones are the
-  // position scores the last step asked for (two per lane for a far block, up to 32 for a near one), which the step
-  // waits for where it uses them.
+  // This wave's share of the buffer has landed: memory operations complete in issue order, and the younger ones are
+  // the position scores the last step asked for (two per lane for a far block, up to 32 for a near one), which the
+  // step waits for where it uses them, and the window stores issued after them (counting only the former waits for
+  // as many of them as there were stores, no more than the step is about to wait for anyway).
   constexpr int kAsked = (kLaneT ? 1 : 0) + (kLoopT ? 1 : 0);
   if (far_n) wait_vmcnt<kAsked>();
   else if (kLaneT && GRP) wait_vmcnt<4 + (kLoopT ? 16 : 0)>();
@@ -360,6 +376,8 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
     // element v of lane (g, li): loop row yr = y0 + 8*(v/4) + 4g + v%4, lane row xr; i - j = +-(xr - yr)
     const bool far = far_n;
     const int d_far = dfar_n;
+    d_lo = d_lo_n;
+    off4[0] = off4_n[0], off4[1] = off4_n[1], off4[2] = off4_n[2], off4[3] = off4_n[3];
     f32x16 sacc, dpacc;   // S' starts from the position scores, dP' from -Delta: the products add on top
     if (kBias && far) {
       sacc = rank1_start<QT>(kLaneT ? (float)raw_lane[0] : 0.f, kLoopT ? (float)raw_loop[0] : 0.f, g);
@@ -367,11 +385,29 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
       bool grouped = false;
       if constexpr (kLaneT && sizeof(BT) == 2) grouped = GRP;
       if (grouped) {
+        // Where no lane's six entries were moved back to stay inside its row, a group's first entry is entry 0 or 1 and
+        // element e lies at most |e - e_min| further on: entries 0..3 for three of the elements, which one byte
+        // permutation picks out of the first two registers, and 0..4 for the fourth.
+        if (__builtin_amdgcn_ballot_w64((goff & 0xEEEEu) != 0u) == 0) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const uint32_t o4 = off4[v >> 2];
-          const uint32_t idx = ((goff >> (4 * (v >> 2))) & 7u) + ((o4 >> (8 * (v & 3))) & 255u) - ((o4 >> (kDQ ? 24 : 0)) & 255u);
-          if constexpr (sizeof(BT) == 2) sacc[v] = QT::scratch_to_f32(entry16(raw3[v >> 2], idx)) + (float)raw_loop[v];
+          for (int v = 0; v < 16; ++v) {
+            if constexpr (sizeof(BT) == 2) {
+              const uint32_t o4 = off4[v >> 2];
+              const u32x3 w = raw3[v >> 2];
+              const uint32_t idx = ((goff >> (4 * (v >> 2))) & 1u) + ((o4 >> (8 * (v & 3))) & 255u) - ((o4 >> (kDQ ? 24 : 0)) & 255u);
+              // bytes 2 idx, 2 idx + 1 of {w[1], w[0]} into the low half of the result, zeros above
+              uint32_t u = __builtin_amdgcn_perm(w[1], w[0], __umul24(idx, 0x0202u) + 0x0c0c0100u);
+              if ((v & 3) == (kDQ ? 0 : 3)) u = idx == 4u ? (w[2] & 0xffffu) : u;
+              sacc[v] = QT::scratch_to_f32((uint16_t)u) + (float)raw_loop[v];
+            }
+          }
+        } else {
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const uint32_t o4 = off4[v >> 2];
+            const uint32_t idx = ((goff >> (4 * (v >> 2))) & 7u) + ((o4 >> (8 * (v & 3))) & 255u) - ((o4 >> (kDQ ? 24 : 0)) & 255u);
+            if constexpr (sizeof(BT) == 2) sacc[v] = QT::scratch_to_f32(entry16(raw3[v >> 2], idx)) + (float)raw_loop[v];
+          }
         }
       } else {
 #pragma unroll
@@ -379,6 +415,8 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
       }
     }
     if (has_next) request_far(y0 + kBwdStep);
+    if (has_next) request_near(y0 + kBwdStep);   // as early as the registers are free: the round trip runs behind the whole step
+                                                 // (in four parts between the parts of the step it was slower)
 #pragma unroll
     for (int q4 = 0; q4 < 4; ++q4) {
       f32x4 del4 = {del_x, del_x, del_x, del_x};
@@ -497,7 +535,6 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
         n_g -= n_now;
       }
     }
-    if (has_next) request_near(y0 + kBwdStep);  // here rather than earlier: the requested values occupy 32 registers until used
     // ---- outputs: contraction over the loop rows, which are the accumulator registers ------------------------------
 #pragma unroll
     for (int c = 0; c < 2; ++c) {

@@ -510,6 +510,7 @@ def test_backward_argument_validation_codes():
     a = _good_bwd_args(); a.d_p2c_bias = 0x4008; a.seqlen = 0; assert call(a) == -5       # (8-byte alignment is enough for 16-bit types)
     a = _good_bwd_args(); a.bias_stride_t = 500; assert call(a) == -5      # rows shorter than 2S
     a = _good_bwd_args(); a.seqlen, a.bias_stride_t = 1 << 20, 1 << 12; assert call(a) == -5  # 32-bit offsets
+    a = _good_bwd_args(); a.dtype, a.seqlen, a.bias_stride_t = _lib.FDB_F32, 1 << 19, 1 << 11; assert call(a) == -5  # ... in bytes
     a = _good_bwd_args(); a.delta_lut = None; assert call(a) == -6
     a = _good_bwd_args(); a.lut_radius = 0; assert call(a) == -6
     a = _good_bwd_args(); a.lut_window = 61; assert call(a) == -6           # more table rows per step than the ring holds
