@@ -248,13 +248,16 @@ def _scores_f32(x, pos_t):
 
 
 def attention_bwd_kernels(q, k, v, dout, lse, *, out=None, delta=None, c2p=None, p2c=None, d_c2p=None, d_p2c=None, sm_scale,
-                          position_buckets=0, max_relative_positions=0, causal=False, seq_start=None, seq_len=None):
+                          position_buckets=0, max_relative_positions=0, causal=False, seq_start=None, seq_len=None,
+                          dq_out=None, dk_out=None):
     """The two backward launches (fdb_attn_bwd) on tensors the caller made: q, k, v, dout [B, L, H, D]; lse [B*L, H];
     either `out` (the forward's output; the call then computes delta itself) or `delta` [B*L, H] fp32; the position
     scores c2p = q . K_r^T / p2c = k . Q_r^T and their gradient tensors (cleared by the caller if the batch is padded: the
     kernels store every entry of a real token's row and leave rows of padding alone) as views of logical shape
     [B, L, H, 2S] with a unit stride on the last axis and any memory layout behind it (all four the same, in q's
-    element type).  Returns dq, dk, dv (content part) and leaves the score gradients in d_c2p / d_p2c."""
+    element type).  Returns dq, dk, dv (content part) and leaves the score gradients in d_c2p / d_p2c.
+    dq_out / dk_out: where to write dq / dk instead of a fresh tensor, views of logical shape [B, L, H, D] in q's type with
+    a unit stride on the last axis and rows aligned to 16 bytes (cleared by the caller if the batch is padded)."""
     B, L, H, D = q.shape
     span = att_span(position_buckets, max_relative_positions)
     q, k, v, dout = [x if x.stride(-1) == 1 else x.contiguous() for x in (q, k, v, dout)]
@@ -288,7 +291,10 @@ def attention_bwd_kernels(q, k, v, dout, lse, *, out=None, delta=None, c2p=None,
     lse = lse.contiguous()
     padded = seq_start is not None or seq_len is not None
     alloc = torch.zeros if padded else torch.empty
-    dq, dk, dv = [alloc((B, L, H, D), dtype=q.dtype, device=q.device) for _ in range(3)]
+    for name, x in (("dq_out", dq_out), ("dk_out", dk_out)):
+        if x is not None and (tuple(x.shape) != (B, L, H, D) or x.stride(3) != 1 or x.dtype != q.dtype or x.device != q.device):
+            raise ValueError("%s: a view of shape [B, L, H, D] = %s in q's element type with a unit last stride" % (name, (B, L, H, D)))
+    dq, dk, dv = [x if x is not None else alloc((B, L, H, D), dtype=q.dtype, device=q.device) for x in (dq_out, dk_out, None)]
     a.q, a.k, a.v, a.dout = q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr()
     a.dq, a.dk, a.dv, a.lse, a.delta = dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), lse.data_ptr(), delta.data_ptr()
     a.out = None if out is None else out.data_ptr()
@@ -319,7 +325,8 @@ def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=
     flash_attn_v2_bwd_dise the position-score tensors and gets their gradients back; as there, those tensors
     are two GEMMs around the kernel (here head-major [H, B*L, 2S]) and the chain through K_r / Q_r and back into
     q / k is four more.  delta: (dout * out).sum(-1) as fp32 [B*L, H] if the caller has it (then `out` is not
-    read); by default the first launch computes it."""
+    read); by default the first launch computes it.  dq / dk of a side with a position term come back as the
+    [B, L, H, D] view of head-major memory (see below), the others contiguous."""
     B, L, H, D = q.shape
     if q.dtype not in _DTYPES:
         raise ValueError("unsupported dtype %s" % q.dtype)
@@ -353,13 +360,20 @@ def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=
         p2c = torch.bmm(heads_first(k), pos_query[:, :2 * span].transpose(1, 2).to(k.dtype))
         d_p2c = like(p2c)
     blhs = lambda x: None if x is None else x.view(H, B, L, 2 * span).permute(1, 2, 0, 3)  # the logical [B, L, H, 2S] view
+    # dq / dk of a side with a position term are written head-major, [H, B*L, D], the layout in which the GEMM that
+    # carries the score gradients back through K_r / Q_r adds its product onto them in place (fp32 accumulation over the
+    # kernel's content part, one rounding; no fp32 copy of the product and no passes to add and convert it).  The
+    # caller gets the logical [B, L, H, D] view of that memory.
+    new_x = torch.zeros if like is torch.zeros_like else torch.empty
+    x_hm = new_x((2 if both else 1, H, B * L, D), dtype=q.dtype, device=q.device) if (pos_key is not None or pos_query is not None) else None
+    blhd = lambda x: x.view(H, B, L, D).permute(1, 2, 0, 3)
+    dq_out = blhd(x_hm[0]) if pos_key is not None else None
+    dk_out = blhd(x_hm[1 if both else 0]) if pos_query is not None else None
     dq, dk, dv = attention_bwd_kernels(q, k, v, dout, lse, out=out, delta=delta, c2p=blhs(c2p), p2c=blhs(p2c), d_c2p=blhs(d_c2p),
                                        d_p2c=blhs(d_p2c), sm_scale=sm_scale, position_buckets=position_buckets,
-                                       max_relative_positions=max_relative_positions, causal=causal, seq_start=seq_start, seq_len=seq_len)
+                                       max_relative_positions=max_relative_positions, causal=causal, seq_start=seq_start, seq_len=seq_len,
+                                       dq_out=dq_out, dk_out=dk_out)
     dpk = dpq = None
-
-    def into_x(dx, extra):  # the content part in the inputs' type plus the position part in fp32, [H', B*L, D] head-major
-        return extra.view(H, B, L, D).permute(1, 2, 0, 3).add_(dx).to(dx.dtype, memory_format=torch.contiguous_format)
 
     def into_pos(d_scores, xh, pos):  # [H', B*L, 2S]^T . [H', B*L, D] -> [H', 2S, D]: a reduction over the tokens
         n_mat, n_tok = d_scores.shape[0], d_scores.shape[1]
@@ -379,15 +393,14 @@ def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=
 
     # score = x . pos[delta]: both factors get their share
     if both:
-        extra2 = _scores_f32(d_scores2, pos2)                  # [2H, B*L, D]
-        dq, dk = into_x(dq, extra2[:H]), into_x(dk, extra2[H:])
+        x_hm.view(2 * H, B * L, D).baddbmm_(d_scores2, pos2)  # (dq, dk) += (d c2p . K_r, d p2c . Q_r)
         dpos2 = into_pos(d_scores2, x2, None)
         dpk, dpq = pad_rows(dpos2[:H], pos_key), pad_rows(dpos2[H:], pos_query)
     elif pos_key is not None:
-        dq = into_x(dq, _scores_f32(d_c2p, pos_key[:, :2 * span]))
+        x_hm[0].baddbmm_(d_c2p, pos_key[:, :2 * span].to(q.dtype))
         dpk = pad_rows(into_pos(d_c2p, heads_first(q), None), pos_key)
     elif pos_query is not None:
-        dk = into_x(dk, _scores_f32(d_p2c, pos_query[:, :2 * span]))
+        x_hm[0].baddbmm_(d_p2c, pos_query[:, :2 * span].to(k.dtype))
         dpq = pad_rows(into_pos(d_p2c, heads_first(k), None), pos_query)
     return dq, dk, dv, dpk, dpq
 
