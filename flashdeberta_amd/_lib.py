@@ -45,7 +45,7 @@ class FdbAttnBwdArgs(ctypes.Structure):
 
 
 EXPORTS = (
-    "fdb_version", "fdb_attn_args_size", "fdb_strerror", "fdb_attn_check", "fdb_attn_fwd", "fdb_attn_fwd_part", "fdb_attn_fwd_noalloc", "fdb_attn_bwd", "fdb_attn_bwd_args_size", "fdb_attn_workspace_bytes",
+    "fdb_version", "fdb_attn_args_size", "fdb_strerror", "fdb_attn_check", "fdb_attn_fwd", "fdb_attn_fwd_part", "fdb_attn_fwd_noalloc", "fdb_attn_bwd", "fdb_attn_bwd_chain", "fdb_attn_bwd_args_size", "fdb_attn_workspace_bytes",
     "fdb_worklist_ints",
     "fdb_worklist_max_tiles", "fdb_tile_rows", "fdb_build_worklist", "fdb_delta_lut_radius", "fdb_delta_lut", "fdb_delta_lut_window",
     "fdb_quant_e4m3_per_head", "fdb_quant_e4m3_per_head_pair", "fdb_dequant_e4m3_per_head",
@@ -83,6 +83,8 @@ def _load():
                           "rebuild it" % (LIB_PATH, lib.fdb_attn_bwd_args_size(), ctypes.sizeof(FdbAttnBwdArgs)))
     lib.fdb_attn_bwd.restype = ctypes.c_int
     lib.fdb_attn_bwd.argtypes = [ctypes.POINTER(FdbAttnBwdArgs), vp]
+    lib.fdb_attn_bwd_chain.restype = ctypes.c_int
+    lib.fdb_attn_bwd_chain.argtypes = [vp, vp, vp, vp, vp, i32, i64, i32, i32, i32, i32, vp]
     lib.fdb_attn_workspace_bytes.restype = i64
     lib.fdb_attn_workspace_bytes.argtypes = [ctypes.POINTER(FdbAttnArgs)]
     lib.fdb_worklist_ints.restype = i64

@@ -13,7 +13,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 PKG = os.path.dirname(HERE)
 LIB = os.path.join(PKG, "libfdb_hip.so")
-SOURCES = ["fdb_api.cpp", "fdb_attn.hip", "fdb_near.hip", "fdb_fp8.hip", "fdb_aux.hip", "fdb_bwd.hip"]
+SOURCES = ["fdb_api.cpp", "fdb_attn.hip", "fdb_near.hip", "fdb_fp8.hip", "fdb_aux.hip", "fdb_bwd.hip", "fdb_chain.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-x", "hip",

@@ -87,6 +87,18 @@ struct FdbBwdParams {
 };
 int fdb_launch_bwd(const FdbBwdParams& p, int dtype, int head_dim, void* stream);
 
+// The chain through the position tables (fdb_chain.hip): contiguous tensors, head_dim 64, 2S = 512.
+struct FdbChainParams {
+  const char* g;       // [matrices][rows][2S] score gradients
+  const char* x;       // [matrices][rows][D] the token rows of the other factor (q or k)
+  const char* pos;     // [matrices][2S][D] the tables
+  char* dx;            // [matrices][rows][D] in and out: += g . pos
+  float* parts_out;    // [parts][matrices][2S][D] partial sums of g^T . x
+  int64_t rows;
+  int32_t matrices, parts, tiles_per_part;
+};
+int fdb_launch_chain(const FdbChainParams& p, int dtype, void* stream);
+
 // Workspace slot `slot`: its output rows and its log-sum-exps (row_bytes = head_dim * element size).
 #if defined(__HIPCC__)
 __device__ __forceinline__ char* ws_slot_out(const FdbKParams& p, int slot, int row_bytes) {

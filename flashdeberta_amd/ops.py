@@ -317,8 +317,33 @@ def attention_bwd_kernels(q, k, v, dout, lse, *, out=None, delta=None, c2p=None,
     return dq, dk, dv
 
 
+def chain_through_tables(d_scores, x, pos, dx):
+    """dx += d_scores . pos in place and returns d_scores^T . x (fp32), both from one pass over d_scores
+    (fdb_attn_bwd_chain): d_scores [M, N, 2S], x and dx [M, N, D], pos [M, 2S, D], contiguous, one 16-bit element type.
+    M: (head, term) pairs, N: token rows.  Counterpart of the autograd backward of the reference's bias GEMMs
+    (model.py:189-192).  chain_through_tables_ok says whether the kernel is built for a shape."""
+    M, N, two_s = d_scores.shape
+    D = x.shape[2]
+    for t, shape in ((d_scores, (M, N, two_s)), (x, (M, N, D)), (pos, (M, two_s, D)), (dx, (M, N, D))):
+        if tuple(t.shape) != shape or not t.is_contiguous() or t.dtype != d_scores.dtype or t.device != d_scores.device:
+            raise ValueError("chain_through_tables: contiguous tensors [M, N, 2S], [M, N, D], [M, 2S, D], [M, N, D] of one type on one device")
+    if not chain_through_tables_ok(d_scores.dtype, D, two_s // 2, N):
+        raise ValueError("chain_through_tables: built for 16-bit types, head_dim 64, 2S = 512 and a multiple of 32 rows")
+    cus = torch.cuda.get_device_properties(d_scores.device).multi_processor_count
+    parts = max(1, min(N // 32, cus // M))   # one workgroup per CU: as many shares of the rows as fill the GPU once
+    dpos_parts = torch.empty((parts, M, two_s, D), dtype=torch.float32, device=d_scores.device)
+    with torch.cuda.device(d_scores.device):
+        check(lib.fdb_attn_bwd_chain(d_scores.data_ptr(), x.data_ptr(), pos.data_ptr(), dx.data_ptr(), dpos_parts.data_ptr(),
+                                     M, N, two_s // 2, D, _DTYPES[d_scores.dtype], parts, _stream_ptr(d_scores.device)), "fdb_attn_bwd_chain")
+    return dpos_parts.sum(0) if parts > 1 else dpos_parts[0]
+
+
+def chain_through_tables_ok(dtype, head_dim, span, rows):
+    return dtype in (torch.bfloat16, torch.float16) and head_dim == 64 and span == 256 and rows >= 32 and rows % 32 == 0
+
+
 def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=None, *, sm_scale=None, position_buckets=0,
-                               max_relative_positions=0, causal=False, seq_start=None, seq_len=None, delta=None):
+                               max_relative_positions=0, causal=False, seq_start=None, seq_len=None, delta=None, fused_chain=None):
     """Backward of the fixed layout: q, k, v, out, dout [B, L, H, D], lse [B*L, H] as the forward returns it,
     pos_key = K_r / pos_query = Q_r [H, 2S, D] or None  ->  (dq, dk, dv, d pos_key, d pos_query).
     Counterpart of FlashAttentionDisentangled.backward (reference flash_attention.py:1066-1086), which hands
@@ -326,7 +351,8 @@ def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=
     are two GEMMs around the kernel (here head-major [H, B*L, 2S]) and the chain through K_r / Q_r and back into
     q / k is four more.  delta: (dout * out).sum(-1) as fp32 [B*L, H] if the caller has it (then `out` is not
     read); by default the first launch computes it.  dq / dk of a side with a position term come back as the
-    [B, L, H, D] view of head-major memory (see below), the others contiguous."""
+    [B, L, H, D] view of head-major memory (see below), the others contiguous.  fused_chain: None takes the one-pass
+    chain kernel (chain_through_tables) where it is built for the shape, False the two GEMMs, True insists on the kernel."""
     B, L, H, D = q.shape
     if q.dtype not in _DTYPES:
         raise ValueError("unsupported dtype %s" % q.dtype)
@@ -391,17 +417,25 @@ def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=
             dpos = torch.cat([dpos, dpos.new_zeros(H, pos.shape[1] - 2 * span, D)], dim=1)
         return dpos
 
-    # score = x . pos[delta]: both factors get their share
+    # score = x . pos[delta]: both factors get their share -- in one pass over the score gradients where the chain
+    # kernel is built for the shape, else as two GEMMs (the first adds onto dq / dk in place)
+    fused = chain_through_tables_ok(q.dtype, D, span, B * L) if fused_chain is None else bool(fused_chain)
     if both:
-        x_hm.view(2 * H, B * L, D).baddbmm_(d_scores2, pos2)  # (dq, dk) += (d c2p . K_r, d p2c . Q_r)
-        dpos2 = into_pos(d_scores2, x2, None)
+        if fused:
+            dpos2 = chain_through_tables(d_scores2, x2, pos2, x_hm.view(2 * H, B * L, D))
+        else:
+            x_hm.view(2 * H, B * L, D).baddbmm_(d_scores2, pos2)  # (dq, dk) += (d c2p . K_r, d p2c . Q_r)
+            dpos2 = into_pos(d_scores2, x2, None)
         dpk, dpq = pad_rows(dpos2[:H], pos_key), pad_rows(dpos2[H:], pos_query)
-    elif pos_key is not None:
-        x_hm[0].baddbmm_(d_c2p, pos_key[:, :2 * span].to(q.dtype))
-        dpk = pad_rows(into_pos(d_c2p, heads_first(q), None), pos_key)
-    elif pos_query is not None:
-        x_hm[0].baddbmm_(d_p2c, pos_query[:, :2 * span].to(k.dtype))
-        dpq = pad_rows(into_pos(d_p2c, heads_first(k), None), pos_query)
+    elif pos_key is not None or pos_query is not None:
+        pos, x, d_s = (pos_key, q, d_c2p) if pos_key is not None else (pos_query, k, d_p2c)
+        pos_t = pos[:, :2 * span].to(q.dtype)
+        if fused:
+            dpos = chain_through_tables(d_s, heads_first(x).contiguous(), pos_t.contiguous(), x_hm[0])
+        else:
+            x_hm[0].baddbmm_(d_s, pos_t)
+            dpos = into_pos(d_s, heads_first(x), None)
+        dpk, dpq = (pad_rows(dpos, pos_key), None) if pos_key is not None else (None, pad_rows(dpos, pos_query))
     return dq, dk, dv, dpk, dpq
 
 

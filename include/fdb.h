@@ -24,6 +24,10 @@
  *                             followed by clamp(. + S, 0, 2S-1) (:318, :336); host-side, integers out.
  *   fdb_attn_bwd           <- flash_attn_v2_bwd_dise (flash_attention.py:942-1030) with _bwd_preprocess,
  *                             _bwd_kv_dise_kernel and _bwd_q_dise_kernel (:62-141, :581-941).
+ *   fdb_attn_bwd_chain     <- the backward of the two bias GEMMs the reference's module runs in front of its
+ *                             kernels (src/flashdeberta/model.py:189-192: pos_key = q . K_r^T, pos_query = k . Q_r^T),
+ *                             which the reference leaves to autograd: d q += d pos_key . K_r, d K_r = d pos_key^T . q
+ *                             (and the same for k / Q_r), here both in one pass over the score gradients.
  *   fdb_quant_e4m3_per_head, fdb_quant_e4m3_per_head_pair, fdb_dequant_e4m3_per_head   no reference counterpart
  *                             (FP8 Q/K variant).
  */
@@ -241,6 +245,22 @@ typedef struct fdb_attn_bwd_args {
 
 size_t fdb_attn_bwd_args_size(void);
 int fdb_attn_bwd(const fdb_attn_bwd_args* a, void* stream);
+
+/*
+ * The chain of the backward through the position tables, for `matrices` (head, term) pairs at once: with
+ * g = d_scores [matrices][rows][2 * att_span] (what fdb_attn_bwd left in d_c2p_bias / d_p2c_bias, head-major),
+ * x [matrices][rows][head_dim] (the q rows for a c2p matrix, the k rows for a p2c matrix) and
+ * pos [matrices][2 * att_span][head_dim] (K_r resp. Q_r), all contiguous and of element type `dtype`:
+ *     dx [matrices][rows][head_dim]                      += g . pos     (in place, fp32 accumulation, one rounding)
+ *     dpos_parts [parts][matrices][2 * att_span][head_dim] = partial sums of g^T . x over `parts` shares of the rows
+ *                                                           (fp32; the caller adds the parts up)
+ * Built for head_dim 64, att_span 256, FDB_BF16 / FDB_F16, rows a multiple of 32, 1 <= parts <= rows / 32, pointers
+ * aligned to 16 bytes; anything else is refused (FDB_ERR_HEAD_DIM / _SPAN / _DTYPE / _SHAPE / _ALIGN) and the caller
+ * takes the two matrix products instead.  Reference: the autograd backward of model.py:189-192 (see the list above).
+ */
+int fdb_attn_bwd_chain(const void* d_scores, const void* x, const void* pos, void* dx, float* dpos_parts,
+                       int32_t matrices, int64_t rows, int32_t att_span, int32_t head_dim, int32_t dtype, int32_t parts,
+                       void* stream);
 
 /*
  * Bytes of workspace the call would use (0: none), for the device that is current.  A launch whose

@@ -493,6 +493,18 @@ def _good_bwd_args():
     return a
 
 
+def test_chain_argument_validation_codes():
+    """fdb_attn_bwd_chain refuses what its kernel is not built for before anything touches the GPU."""
+    f = lambda g=0x1000, x=0x2000, pos=0x3000, dx=0x4000, parts_out=0x5000, m=24, rows=4096, span=256, d=64, dt=_lib.FDB_BF16, parts=10: \
+        lib.fdb_attn_bwd_chain(g, x, pos, dx, parts_out, m, rows, span, d, dt, parts, None)
+    assert f(g=None) == -1 and f(parts_out=None) == -1
+    assert f(dt=_lib.FDB_F32) == -2 and f(dt=_lib.FDB_FP8_E4M3) == -2
+    assert f(d=32) == -3 and f(d=128) == -3
+    assert f(x=0x2008) == -4 and f(dx=0x4004) == -4
+    assert f(rows=4100) == -5 and f(rows=0) == -5 and f(parts=0) == -5 and f(parts=129) == -5 and f(m=0) == -5
+    assert f(span=128) == -6
+
+
 def test_backward_argument_validation_codes():
     """Every refusal of fdb_attn_bwd comes before anything touches the GPU, so it can be checked without one."""
     call = lambda a: lib.fdb_attn_bwd(ctypes.byref(a), None)

@@ -1277,6 +1277,45 @@ def test_backward_matches_oracle(case, dtype):
         assert not np.isnan(got).any() and err <= tol * max(np.abs(r).max(), 1e-3), "%s: err %.3e, ref max %.3e" % (n, err, np.abs(r).max())
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("M,N", [(1, 32), (2, 96), (24, 1024), (5, 4000 // 32 * 32), (300, 64)])
+def test_chain_through_tables_matches_the_two_matrix_products(M, N, dtype):
+    """fdb_attn_bwd_chain (both products of the score gradients in one pass) against the two products in fp32 on the same
+    16-bit operands: dx in place within one rounding of the element type, the table gradient to fp32 summation order."""
+    g = torch.Generator().manual_seed(91 + M + N)
+    d_scores = torch.randn(M, N, 512, generator=g).to(dtype).cuda()
+    d_scores[:, :, 100:140] = 0                                  # entries the backward kernels wrote as zeros
+    x = torch.randn(M, N, 64, generator=g).to(dtype).cuda()
+    pos = torch.randn(M, 512, 64, generator=g).to(dtype).cuda()
+    dx0 = torch.randn(M, N, 64, generator=g).to(dtype).cuda()
+    dx = dx0.clone()
+    dpos = ops.chain_through_tables(d_scores, x, pos, dx)
+    ref_dx = dx0.float() + torch.bmm(d_scores.float(), pos.float())
+    ref_dpos = torch.bmm(d_scores.float().transpose(1, 2), x.float())
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    assert dpos.dtype == torch.float32 and tuple(dpos.shape) == (M, 512, 64)
+    assert (dx.float() - ref_dx).abs().max().item() <= 1.01 * ulp * ref_dx.abs().max().item()
+    assert (dpos - ref_dpos).abs().max().item() <= 1e-4 * max(1.0, ref_dpos.abs().max().item())
+
+
+@pytest.mark.parametrize("terms", [(True, True), (True, False), (False, True)], ids=["both", "c2p", "p2c"])
+def test_backward_with_and_without_the_chain_kernel(terms):
+    """The whole backward operator with the one-pass chain kernel and with the two GEMMs in its place: the same gradients
+    to the rounding of the element type (v3 buckets, the only table size the kernel is built for)."""
+    B, L, H, D, pb, mr = 2, 512, 3, 64, 256, 512
+    q, k, v, pk, pq = _inputs(B, L, H, D, pb, mr, torch.bfloat16, 4242, 1.0, *terms)
+    q, k, v, pk, pq = [None if x is None else x.cuda() for x in (q, k, v, pk, pq)]
+    dout = torch.randn(B, L, H, D, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16).cuda()
+    kw = dict(position_buckets=pb, max_relative_positions=mr)
+    out, lse = ops.disentangled_attention_fwd(q, k, v, pk, pq, return_lse=True, **kw)
+    a = ops.disentangled_attention_bwd(q, k, v, out, lse, dout, pk, pq, fused_chain=True, **kw)
+    b = ops.disentangled_attention_bwd(q, k, v, out, lse, dout, pk, pq, fused_chain=False, **kw)
+    for name, x, y in zip(("dq", "dk", "dv", "dK_r", "dQ_r"), a, b):
+        assert (x is None) == (y is None), name
+        if x is not None:
+            assert (x.float() - y.float()).abs().max().item() <= 2.0 ** -7 * y.float().abs().max().item(), name
+
+
 @pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "g_*.npz"))), ids=os.path.basename)
 def test_module_backward_matches_golden_gradients(path):
     """The drop-in module under autograd against the gradients torch.autograd wrote through the eager class:
