@@ -9,7 +9,7 @@
 // the score tensors are made) -- two reads of the largest tensor of the backward.  Here a workgroup walks a share of
 // a matrix's rows 32 at a time: the 32 x 2S tile of G goes from global memory straight into one of two LDS buffers
 // (the next tile on its way while this one is used) and feeds both products from there; pos stays in LDS for the
-// life of the workgroup, the tile of x passes through registers.  dx is read, added to in fp32 and written back in
+// life of the workgroup, the tile of x (rows of any stride: q and k are read where they lie) passes through registers.  dx is read, added to in fp32 and written back in
 // the element type (one rounding over the kernels' content part, as a GEMM with beta = 1 would); every workgroup
 // keeps its share of dpos in registers (fp32, 32 KB of accumulators per wave) and writes it once, as one of `parts`
 // partial sums the caller adds up.
@@ -67,7 +67,8 @@ __global__ __launch_bounds__(kChainThreads, 1) void fdb_chain_kernel(const FdbCh
   const int64_t t0 = (int64_t)part * p.tiles_per_part;
   const int64_t t1 = t0 + p.tiles_per_part < tiles ? t0 + p.tiles_per_part : tiles;
   const char* gm = p.g + (int64_t)m * p.rows * (kChainS2 * 2);
-  const char* xm = p.x + (int64_t)m * p.rows * (kChainD * 2);
+  const char* xm = (m < p.split ? p.x + (int64_t)m * p.x_sm * 2 : p.x2 + (int64_t)(m - p.split) * p.x_sm * 2);
+  const int64_t x_row = p.x_sr * 2;   // bytes between the rows of x
   char* dxm = p.dx + (int64_t)m * p.rows * (kChainD * 2);
   const char* pm = p.pos + (int64_t)m * (kChainS2 * kChainD * 2);
 
@@ -98,7 +99,7 @@ __global__ __launch_bounds__(kChainThreads, 1) void fdb_chain_kernel(const FdbCh
   // the tile of x: 32 rows of eight chunks, one chunk per thread, through a register into the padded rows
   u32x4 xreg = {0u, 0u, 0u, 0u};
   auto x_load = [&](int64_t t) __attribute__((always_inline)) {
-    xreg = *(const u32x4*)(xm + (t * kChainRows + (tid >> 3)) * (kChainD * 2) + (tid & 7) * 16);
+    xreg = *(const u32x4*)(xm + (t * kChainRows + (tid >> 3)) * x_row + (tid & 7) * 16);
   };
   // Waves 0 and 1 complete the rows of dx of a tile one tile late: their own half of the table rows (kept in
   // registers) plus the half that wave + 2 left in LDS, added onto the rows in memory and rounded once.

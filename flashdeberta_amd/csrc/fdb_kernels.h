@@ -90,12 +90,13 @@ int fdb_launch_bwd(const FdbBwdParams& p, int dtype, int head_dim, void* stream)
 // The chain through the position tables (fdb_chain.hip): contiguous tensors, head_dim 64, 2S = 512.
 struct FdbChainParams {
   const char* g;       // [matrices][rows][2S] score gradients
-  const char* x;       // [matrices][rows][D] the token rows of the other factor (q or k)
+  const char* x;       // the token rows of the other factor (q or k) of matrices [0, split): matrix stride x_sm, row stride x_sr (elements)
+  const char* x2;      // ... of matrices [split, matrices), numbered from 0 again; same strides
   const char* pos;     // [matrices][2S][D] the tables
   char* dx;            // [matrices][rows][D] in and out: += g . pos
   float* parts_out;    // [parts][matrices][2S][D] partial sums of g^T . x
-  int64_t rows;
-  int32_t matrices, parts, tiles_per_part;
+  int64_t rows, x_sm, x_sr;
+  int32_t matrices, split, parts, tiles_per_part;
 };
 int fdb_launch_chain(const FdbChainParams& p, int dtype, void* stream);
 

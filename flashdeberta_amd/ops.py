@@ -317,24 +317,34 @@ def attention_bwd_kernels(q, k, v, dout, lse, *, out=None, delta=None, c2p=None,
     return dq, dk, dv
 
 
-def chain_through_tables(d_scores, x, pos, dx):
+def chain_through_tables(d_scores, x, pos, dx, x_second=None):
     """dx += d_scores . pos in place and returns d_scores^T . x (fp32), both from one pass over d_scores
-    (fdb_attn_bwd_chain): d_scores [M, N, 2S], x and dx [M, N, D], pos [M, 2S, D], contiguous, one 16-bit element type.
-    M: (head, term) pairs, N: token rows.  Counterpart of the autograd backward of the reference's bias GEMMs
-    (model.py:189-192).  chain_through_tables_ok says whether the kernel is built for a shape."""
+    (fdb_attn_bwd_chain): d_scores [M, N, 2S], dx [M, N, D] and pos [M, 2S, D] contiguous; the token rows x [M, N, D]
+    with any matrix and row stride and a unit last stride -- or x [M1, N, D] and x_second [M - M1, N, D] with the same
+    strides, so that q and k are read where they lie.  One 16-bit element type.  M: (head, term) pairs, N: token rows.
+    Counterpart of the autograd backward of the reference's bias GEMMs (model.py:189-192).  chain_through_tables_ok
+    says whether the kernel is built for a shape."""
     M, N, two_s = d_scores.shape
-    D = x.shape[2]
-    for t, shape in ((d_scores, (M, N, two_s)), (x, (M, N, D)), (pos, (M, two_s, D)), (dx, (M, N, D))):
+    D = dx.shape[2]
+    m1 = x.shape[0]
+    for t, shape in ((d_scores, (M, N, two_s)), (pos, (M, two_s, D)), (dx, (M, N, D))):
         if tuple(t.shape) != shape or not t.is_contiguous() or t.dtype != d_scores.dtype or t.device != d_scores.device:
-            raise ValueError("chain_through_tables: contiguous tensors [M, N, 2S], [M, N, D], [M, 2S, D], [M, N, D] of one type on one device")
+            raise ValueError("chain_through_tables: contiguous d_scores [M, N, 2S], pos [M, 2S, D], dx [M, N, D] of one type on one device")
+    xs = [x] if x_second is None else [x, x_second]
+    if sum(t.shape[0] for t in xs) != M or any(tuple(t.shape[1:]) != (N, D) or t.dtype != d_scores.dtype or t.device != d_scores.device for t in xs):
+        raise ValueError("chain_through_tables: x (and x_second) hold M matrices of [N, D] in the type of d_scores")
+    if any(t.stride(2) != 1 or t.stride() != x.stride() or (t.stride(0) * t.element_size()) % 16 or (t.stride(1) * t.element_size()) % 16
+           or t.data_ptr() % 16 for t in xs):
+        xs = [t.contiguous() for t in xs]   # one layout for both, rows and matrices at multiples of 16 bytes
     if not chain_through_tables_ok(d_scores.dtype, D, two_s // 2, N):
         raise ValueError("chain_through_tables: built for 16-bit types, head_dim 64, 2S = 512 and a multiple of 32 rows")
     cus = torch.cuda.get_device_properties(d_scores.device).multi_processor_count
     parts = max(1, min(N // 32, cus // M))   # one workgroup per CU: as many shares of the rows as fill the GPU once
     dpos_parts = torch.empty((parts, M, two_s, D), dtype=torch.float32, device=d_scores.device)
     with torch.cuda.device(d_scores.device):
-        check(lib.fdb_attn_bwd_chain(d_scores.data_ptr(), x.data_ptr(), pos.data_ptr(), dx.data_ptr(), dpos_parts.data_ptr(),
-                                     M, N, two_s // 2, D, _DTYPES[d_scores.dtype], parts, _stream_ptr(d_scores.device)), "fdb_attn_bwd_chain")
+        check(lib.fdb_attn_bwd_chain(d_scores.data_ptr(), xs[0].data_ptr(), xs[1].data_ptr() if len(xs) > 1 else None, pos.data_ptr(),
+                                     dx.data_ptr(), dpos_parts.data_ptr(), M, m1, N, xs[0].stride(0), xs[0].stride(1), two_s // 2, D,
+                                     _DTYPES[d_scores.dtype], parts, _stream_ptr(d_scores.device)), "fdb_attn_bwd_chain")
     return dpos_parts.sum(0) if parts > 1 else dpos_parts[0]
 
 
@@ -371,12 +381,13 @@ def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=
     # the kernels store every entry of a real token's row of the score gradients; only rows of padding need clearing
     like = torch.zeros_like if (seq_start is not None or seq_len is not None) else torch.empty_like
     if both:
-        # both terms: their tensors stacked, [2H, B*L, ...], so that each GEMM around the kernel is one call over 2H
-        # matrices instead of two over H (a third less time at 4 k tokens; the reduction over tokens, which has few
-        # output tiles, gains most)
-        x2 = torch.stack([heads_first(q), heads_first(k)]).view(2 * H, B * L, D)
+        # both terms: their score tensors stacked, [2H, B*L, 2S], so that the chain back through the tables is one call
+        # over 2H matrices; the scores themselves are two GEMMs that read q and k where they lie (a stacked copy of
+        # q and k plus one GEMM over 2H matrices took 339 against 236 us at the bench shape)
         pos2 = torch.stack([pos_key[:, :2 * span], pos_query[:, :2 * span]]).view(2 * H, 2 * span, D).to(q.dtype)
-        scores2 = torch.bmm(x2, pos2.transpose(1, 2))        # [2H, B*L, 2S] = (q . K_r^T, k . Q_r^T), in the inputs' type like the reference's
+        scores2 = torch.empty((2 * H, B * L, 2 * span), dtype=q.dtype, device=q.device)   # (q . K_r^T, k . Q_r^T), in the inputs' type like the reference's
+        torch.bmm(heads_first(q), pos2[:H].transpose(1, 2), out=scores2[:H])
+        torch.bmm(heads_first(k), pos2[H:].transpose(1, 2), out=scores2[H:])
         d_scores2 = like(scores2)
         c2p, p2c, d_c2p, d_p2c = scores2[:H], scores2[H:], d_scores2[:H], d_scores2[H:]
     elif pos_key is not None:
@@ -422,16 +433,17 @@ def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=
     fused = chain_through_tables_ok(q.dtype, D, span, B * L) if fused_chain is None else bool(fused_chain)
     if both:
         if fused:
-            dpos2 = chain_through_tables(d_scores2, x2, pos2, x_hm.view(2 * H, B * L, D))
+            dpos2 = chain_through_tables(d_scores2, heads_first(q), pos2, x_hm.view(2 * H, B * L, D), x_second=heads_first(k))
         else:
             x_hm.view(2 * H, B * L, D).baddbmm_(d_scores2, pos2)  # (dq, dk) += (d c2p . K_r, d p2c . Q_r)
-            dpos2 = into_pos(d_scores2, x2, None)
+            # the reduction over the tokens has few output tiles: one call over 2H matrices, on a stacked copy of q and k
+            dpos2 = into_pos(d_scores2, torch.stack([heads_first(q), heads_first(k)]).view(2 * H, B * L, D), None)
         dpk, dpq = pad_rows(dpos2[:H], pos_key), pad_rows(dpos2[H:], pos_query)
     elif pos_key is not None or pos_query is not None:
         pos, x, d_s = (pos_key, q, d_c2p) if pos_key is not None else (pos_query, k, d_p2c)
         pos_t = pos[:, :2 * span].to(q.dtype)
         if fused:
-            dpos = chain_through_tables(d_s, heads_first(x).contiguous(), pos_t.contiguous(), x_hm[0])
+            dpos = chain_through_tables(d_s, heads_first(x), pos_t.contiguous(), x_hm[0])
         else:
             x_hm[0].baddbmm_(d_s, pos_t)
             dpos = into_pos(d_s, heads_first(x), None)

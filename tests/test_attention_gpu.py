@@ -1289,7 +1289,13 @@ def test_chain_through_tables_matches_the_two_matrix_products(M, N, dtype):
     pos = torch.randn(M, 512, 64, generator=g).to(dtype).cuda()
     dx0 = torch.randn(M, N, 64, generator=g).to(dtype).cuda()
     dx = dx0.clone()
-    dpos = ops.chain_through_tables(d_scores, x, pos, dx)
+    if M % 2 == 0:
+        # the token rows as two strided views of token-major tensors, the way q and k reach the operator
+        xa, xb = [torch.empty(N, M // 2, 64, dtype=dtype, device="cuda") for _ in range(2)]
+        xa.copy_(x[:M // 2].transpose(0, 1)); xb.copy_(x[M // 2:].transpose(0, 1))
+        dpos = ops.chain_through_tables(d_scores, xa.transpose(0, 1), pos, dx, x_second=xb.transpose(0, 1))
+    else:
+        dpos = ops.chain_through_tables(d_scores, x, pos, dx)
     ref_dx = dx0.float() + torch.bmm(d_scores.float(), pos.float())
     ref_dpos = torch.bmm(d_scores.float().transpose(1, 2), x.float())
     ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
