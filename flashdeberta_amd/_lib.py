@@ -84,7 +84,7 @@ def _load():
     lib.fdb_attn_bwd.restype = ctypes.c_int
     lib.fdb_attn_bwd.argtypes = [ctypes.POINTER(FdbAttnBwdArgs), vp]
     lib.fdb_attn_bwd_chain.restype = ctypes.c_int
-    lib.fdb_attn_bwd_chain.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, i64, i64, i64, i32, i32, i32, i32, vp]
+    lib.fdb_attn_bwd_chain.argtypes = [vp, vp, vp, vp, vp, vp, vp, i32, i32, i64, i64, i64, i64, i64, i32, i32, i32, i32, vp]
     lib.fdb_attn_workspace_bytes.restype = i64
     lib.fdb_attn_workspace_bytes.argtypes = [ctypes.POINTER(FdbAttnArgs)]
     lib.fdb_worklist_ints.restype = i64

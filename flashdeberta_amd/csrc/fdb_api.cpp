@@ -461,23 +461,27 @@ int fdb_attn_fwd_noalloc(const fdb_attn_args* a, void* stream) {
 
 size_t fdb_attn_bwd_args_size(void) { return sizeof(fdb_attn_bwd_args); }
 
-int fdb_attn_bwd_chain(const void* d_scores, const void* x, const void* x_second, const void* pos, void* dx, float* dpos_parts,
-                       int32_t matrices, int32_t first_matrices, int64_t rows, int64_t x_stride_matrix, int64_t x_stride_row,
-                       int32_t att_span, int32_t head_dim, int32_t dtype, int32_t parts, void* stream) {
+int fdb_attn_bwd_chain(const void* d_scores, const void* x, const void* x_second, const void* pos, void* dx, void* dx_second,
+                       float* dpos_parts, int32_t matrices, int32_t first_matrices, int64_t rows, int64_t x_stride_matrix,
+                       int64_t x_stride_row, int64_t dx_stride_matrix, int64_t dx_stride_row, int32_t att_span, int32_t head_dim,
+                       int32_t dtype, int32_t parts, void* stream) {
   if (!d_scores || !x || !pos || !dx || !dpos_parts) return FDB_ERR_NULL;
-  if (matrices >= 1 && first_matrices < matrices && !x_second) return FDB_ERR_NULL;
+  if (matrices >= 1 && first_matrices < matrices && (!x_second || !dx_second)) return FDB_ERR_NULL;
   if (dtype != FDB_BF16 && dtype != FDB_F16) return FDB_ERR_DTYPE;
   if (head_dim != 64) return FDB_ERR_HEAD_DIM;
   if (att_span != 256) return FDB_ERR_SPAN;
   if (matrices < 1 || matrices > 65535 || first_matrices < 1 || first_matrices > matrices || rows < 32 || rows % 32 != 0 ||
-      parts < 1 || parts > rows / 32 || x_stride_matrix < 0 || x_stride_row < 64) return FDB_ERR_SHAPE;
+      parts < 1 || parts > rows / 32 || x_stride_matrix < 0 || x_stride_row < 64 || dx_stride_matrix < 64 || dx_stride_row < 64)
+    return FDB_ERR_SHAPE;
   if (!aligned16(d_scores) || !aligned16(x) || (x_second && !aligned16(x_second)) || !aligned16(pos) || !aligned16(dx) ||
-      !aligned16(dpos_parts) || (x_stride_matrix * 2) % 16 != 0 || (x_stride_row * 2) % 16 != 0) return FDB_ERR_ALIGN;
+      (dx_second && !aligned16(dx_second)) || !aligned16(dpos_parts) || (x_stride_matrix * 2) % 16 != 0 ||
+      (x_stride_row * 2) % 16 != 0 || (dx_stride_matrix * 2) % 16 != 0 || (dx_stride_row * 2) % 16 != 0) return FDB_ERR_ALIGN;
   FdbChainParams p;
   memset(&p, 0, sizeof(p));
   p.g = (const char*)d_scores; p.x = (const char*)x; p.x2 = (const char*)x_second; p.pos = (const char*)pos; p.dx = (char*)dx;
-  p.parts_out = dpos_parts;
-  p.rows = rows; p.x_sm = x_stride_matrix; p.x_sr = x_stride_row; p.matrices = matrices; p.split = first_matrices; p.parts = parts;
+  p.dx2 = (char*)dx_second; p.parts_out = dpos_parts;
+  p.rows = rows; p.x_sm = x_stride_matrix; p.x_sr = x_stride_row; p.dx_sm = dx_stride_matrix; p.dx_sr = dx_stride_row;
+  p.matrices = matrices; p.split = first_matrices; p.parts = parts;
   const int64_t tiles = rows / 32;
   p.tiles_per_part = (int32_t)((tiles + parts - 1) / parts);
   return fdb_launch_chain(p, dtype, stream);

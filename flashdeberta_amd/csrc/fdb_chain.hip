@@ -136,7 +136,8 @@ __global__ __launch_bounds__(kChainThreads, 1) void fdb_chain_kernel(const FdbCh
   } else {
     // ---- dx^T += pos^T G^T: wave u = wave - 4 takes block u % 2 of d and half u / 2 of the table rows ---------------
     const int u = wave - 4;
-    char* dxm = p.dx + (int64_t)m * p.rows * (kChainD * 2);
+    char* dxm = (m < p.split ? p.dx + (int64_t)m * p.dx_sm * 2 : p.dx2 + (int64_t)(m - p.split) * p.dx_sm * 2);
+    const int64_t dx_row = p.dx_sr * 2;   // bytes between the rows of dx
     const char* pm = p.pos + (int64_t)m * (kChainS2 * kChainD * 2);
     // This wave's share of the table, transposed, as the sixteen A operands of its product: column 32 (u % 2) + li,
     // table rows 256 (u / 2) + 16 c + 8 g + 0..7.  64 registers for the life of the workgroup, gathered once.
@@ -160,7 +161,7 @@ __global__ __launch_bounds__(kChainThreads, 1) void fdb_chain_kernel(const FdbCh
     for (int q4 = 0; q4 < 4; ++q4) dx_old[q4] = st4{(ST)0.f, (ST)0.f, (ST)0.f, (ST)0.f};
     bool have_prev = false;
     auto dx_ptr = [&](int64_t t, int q4) __attribute__((always_inline)) -> char* {
-      return dxm + ((t * kChainRows + li) * kChainD + 32 * u + 8 * q4 + 4 * g) * 2;
+      return dxm + (t * kChainRows + li) * dx_row + (32 * u + 8 * q4 + 4 * g) * 2;
     };
     auto request_dx = [&](int64_t t) __attribute__((always_inline)) {
       if (u >= 2) return;

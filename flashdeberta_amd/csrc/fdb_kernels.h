@@ -93,9 +93,10 @@ struct FdbChainParams {
   const char* x;       // the token rows of the other factor (q or k) of matrices [0, split): matrix stride x_sm, row stride x_sr (elements)
   const char* x2;      // ... of matrices [split, matrices), numbered from 0 again; same strides
   const char* pos;     // [matrices][2S][D] the tables
-  char* dx;            // [matrices][rows][D] in and out: += g . pos
+  char* dx;            // in and out: += g . pos; rows laid out like those of x, with strides dx_sm, dx_sr, for matrices [0, split)
+  char* dx2;           // ... and for matrices [split, matrices)
   float* parts_out;    // [parts][matrices][2S][D] partial sums of g^T . x
-  int64_t rows, x_sm, x_sr;
+  int64_t rows, x_sm, x_sr, dx_sm, dx_sr;
   int32_t matrices, split, parts, tiles_per_part;
 };
 int fdb_launch_chain(const FdbChainParams& p, int dtype, void* stream);

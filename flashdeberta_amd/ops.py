@@ -317,34 +317,41 @@ def attention_bwd_kernels(q, k, v, dout, lse, *, out=None, delta=None, c2p=None,
     return dq, dk, dv
 
 
-def chain_through_tables(d_scores, x, pos, dx, x_second=None):
+def chain_through_tables(d_scores, x, pos, dx, x_second=None, dx_second=None):
     """dx += d_scores . pos in place and returns d_scores^T . x (fp32), both from one pass over d_scores
-    (fdb_attn_bwd_chain): d_scores [M, N, 2S], dx [M, N, D] and pos [M, 2S, D] contiguous; the token rows x [M, N, D]
-    with any matrix and row stride and a unit last stride -- or x [M1, N, D] and x_second [M - M1, N, D] with the same
-    strides, so that q and k are read where they lie.  One 16-bit element type.  M: (head, term) pairs, N: token rows.
-    Counterpart of the autograd backward of the reference's bias GEMMs (model.py:189-192).  chain_through_tables_ok
-    says whether the kernel is built for a shape."""
+    (fdb_attn_bwd_chain): d_scores [M, N, 2S] and pos [M, 2S, D] contiguous; the token rows x [M, N, D] and the rows dx
+    [M, N, D] they belong to with any matrix and row stride and a unit last stride -- or x / dx [M1, N, D] and
+    x_second / dx_second [M - M1, N, D] with the same strides, so that q, k, dq and dk are read and updated where they
+    lie.  One 16-bit element type.  M: (head, term) pairs, N: token rows.  Counterpart of the autograd backward of the
+    reference's bias GEMMs (model.py:189-192).  chain_through_tables_ok says whether the kernel is built for a shape."""
     M, N, two_s = d_scores.shape
     D = dx.shape[2]
     m1 = x.shape[0]
-    for t, shape in ((d_scores, (M, N, two_s)), (pos, (M, two_s, D)), (dx, (M, N, D))):
+    for t, shape in ((d_scores, (M, N, two_s)), (pos, (M, two_s, D))):
         if tuple(t.shape) != shape or not t.is_contiguous() or t.dtype != d_scores.dtype or t.device != d_scores.device:
-            raise ValueError("chain_through_tables: contiguous d_scores [M, N, 2S], pos [M, 2S, D], dx [M, N, D] of one type on one device")
+            raise ValueError("chain_through_tables: contiguous d_scores [M, N, 2S] and pos [M, 2S, D] of one type on one device")
     xs = [x] if x_second is None else [x, x_second]
-    if sum(t.shape[0] for t in xs) != M or any(tuple(t.shape[1:]) != (N, D) or t.dtype != d_scores.dtype or t.device != d_scores.device for t in xs):
-        raise ValueError("chain_through_tables: x (and x_second) hold M matrices of [N, D] in the type of d_scores")
-    if any(t.stride(2) != 1 or t.stride() != x.stride() or (t.stride(0) * t.element_size()) % 16 or (t.stride(1) * t.element_size()) % 16
-           or t.data_ptr() % 16 for t in xs):
+    dxs = [dx] if dx_second is None else [dx, dx_second]
+    for name, ts in (("x", xs), ("dx", dxs)):
+        if (len(ts) != len(xs) or [t.shape[0] for t in ts] != [t.shape[0] for t in xs] or sum(t.shape[0] for t in ts) != M
+                or any(tuple(t.shape[1:]) != (N, D) or t.dtype != d_scores.dtype or t.device != d_scores.device for t in ts)):
+            raise ValueError("chain_through_tables: %s (and %s_second) hold the M matrices of [N, D] in the type of d_scores" % (name, name))
+    aligned = lambda ts: not any(t.stride(2) != 1 or t.stride() != ts[0].stride() or (t.stride(0) * t.element_size()) % 16
+                                 or (t.stride(1) * t.element_size()) % 16 or t.data_ptr() % 16 for t in ts)
+    if not aligned(xs):
         xs = [t.contiguous() for t in xs]   # one layout for both, rows and matrices at multiples of 16 bytes
+    if not aligned(dxs):
+        raise ValueError("chain_through_tables: dx (and dx_second) share one layout with a unit last stride, rows and matrices at multiples of 16 bytes")
     if not chain_through_tables_ok(d_scores.dtype, D, two_s // 2, N):
         raise ValueError("chain_through_tables: built for 16-bit types, head_dim 64, 2S = 512 and a multiple of 32 rows")
     cus = torch.cuda.get_device_properties(d_scores.device).multi_processor_count
     parts = max(1, min(N // 32, cus // M))   # one workgroup per CU: as many shares of the rows as fill the GPU once
     dpos_parts = torch.empty((parts, M, two_s, D), dtype=torch.float32, device=d_scores.device)
+    second = lambda ts: ts[1].data_ptr() if len(ts) > 1 else None
     with torch.cuda.device(d_scores.device):
-        check(lib.fdb_attn_bwd_chain(d_scores.data_ptr(), xs[0].data_ptr(), xs[1].data_ptr() if len(xs) > 1 else None, pos.data_ptr(),
-                                     dx.data_ptr(), dpos_parts.data_ptr(), M, m1, N, xs[0].stride(0), xs[0].stride(1), two_s // 2, D,
-                                     _DTYPES[d_scores.dtype], parts, _stream_ptr(d_scores.device)), "fdb_attn_bwd_chain")
+        check(lib.fdb_attn_bwd_chain(d_scores.data_ptr(), xs[0].data_ptr(), second(xs), pos.data_ptr(), dxs[0].data_ptr(), second(dxs),
+                                     dpos_parts.data_ptr(), M, m1, N, xs[0].stride(0), xs[0].stride(1), dxs[0].stride(0), dxs[0].stride(1),
+                                     two_s // 2, D, _DTYPES[d_scores.dtype], parts, _stream_ptr(d_scores.device)), "fdb_attn_bwd_chain")
     return dpos_parts.sum(0) if parts > 1 else dpos_parts[0]
 
 
@@ -360,8 +367,8 @@ def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=
     flash_attn_v2_bwd_dise the position-score tensors and gets their gradients back; as there, those tensors
     are two GEMMs around the kernel (here head-major [H, B*L, 2S]) and the chain through K_r / Q_r and back into
     q / k is four more.  delta: (dout * out).sum(-1) as fp32 [B*L, H] if the caller has it (then `out` is not
-    read); by default the first launch computes it.  dq / dk of a side with a position term come back as the
-    [B, L, H, D] view of head-major memory (see below), the others contiguous.  fused_chain: None takes the one-pass
+    read); by default the first launch computes it.  Where the chain kernel does not serve the shape, dq / dk of a side
+    with a position term come back as the [B, L, H, D] view of head-major memory (see below); otherwise contiguous.  fused_chain: None takes the one-pass
     chain kernel (chain_through_tables) where it is built for the shape, False the two GEMMs, True insists on the kernel."""
     B, L, H, D = q.shape
     if q.dtype not in _DTYPES:
@@ -397,15 +404,18 @@ def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=
         p2c = torch.bmm(heads_first(k), pos_query[:, :2 * span].transpose(1, 2).to(k.dtype))
         d_p2c = like(p2c)
     blhs = lambda x: None if x is None else x.view(H, B, L, 2 * span).permute(1, 2, 0, 3)  # the logical [B, L, H, 2S] view
-    # dq / dk of a side with a position term are written head-major, [H, B*L, D], the layout in which the GEMM that
-    # carries the score gradients back through K_r / Q_r adds its product onto them in place (fp32 accumulation over the
-    # kernel's content part, one rounding; no fp32 copy of the product and no passes to add and convert it).  The
-    # caller gets the logical [B, L, H, D] view of that memory.
-    new_x = torch.zeros if like is torch.zeros_like else torch.empty
-    x_hm = new_x((2 if both else 1, H, B * L, D), dtype=q.dtype, device=q.device) if (pos_key is not None or pos_query is not None) else None
-    blhd = lambda x: x.view(H, B, L, D).permute(1, 2, 0, 3)
-    dq_out = blhd(x_hm[0]) if pos_key is not None else None
-    dk_out = blhd(x_hm[1 if both else 0]) if pos_query is not None else None
+    # The chain of the score gradients back through K_r / Q_r adds its product onto dq / dk in place (fp32 accumulation
+    # over the kernel's content part, one rounding; no fp32 copy of the product and no passes to add and convert it):
+    # the chain kernel where they lie, the GEMM that stands in for it on a head-major [H, B*L, D] copy-free layout of
+    # its own, which the backward launches write and of which the caller gets the logical [B, L, H, D] view.
+    fused = chain_through_tables_ok(q.dtype, D, span, B * L) if fused_chain is None else bool(fused_chain)
+    x_hm = dq_out = dk_out = None
+    if not fused and (pos_key is not None or pos_query is not None):
+        new_x = torch.zeros if like is torch.zeros_like else torch.empty
+        x_hm = new_x((2 if both else 1, H, B * L, D), dtype=q.dtype, device=q.device)
+        blhd = lambda x: x.view(H, B, L, D).permute(1, 2, 0, 3)
+        dq_out = blhd(x_hm[0]) if pos_key is not None else None
+        dk_out = blhd(x_hm[1 if both else 0]) if pos_query is not None else None
     dq, dk, dv = attention_bwd_kernels(q, k, v, dout, lse, out=out, delta=delta, c2p=blhs(c2p), p2c=blhs(p2c), d_c2p=blhs(d_c2p),
                                        d_p2c=blhs(d_p2c), sm_scale=sm_scale, position_buckets=position_buckets,
                                        max_relative_positions=max_relative_positions, causal=causal, seq_start=seq_start, seq_len=seq_len,
@@ -430,20 +440,20 @@ def disentangled_attention_bwd(q, k, v, out, lse, dout, pos_key=None, pos_query=
 
     # score = x . pos[delta]: both factors get their share -- in one pass over the score gradients where the chain
     # kernel is built for the shape, else as two GEMMs (the first adds onto dq / dk in place)
-    fused = chain_through_tables_ok(q.dtype, D, span, B * L) if fused_chain is None else bool(fused_chain)
     if both:
         if fused:
-            dpos2 = chain_through_tables(d_scores2, heads_first(q), pos2, x_hm.view(2 * H, B * L, D), x_second=heads_first(k))
+            in_place = lambda x: x.permute(2, 0, 1, 3).view(H, B * L, D)   # a view or an error, never a copy: the kernel writes through it
+            dpos2 = chain_through_tables(d_scores2, heads_first(q), pos2, in_place(dq), x_second=heads_first(k), dx_second=in_place(dk))
         else:
             x_hm.view(2 * H, B * L, D).baddbmm_(d_scores2, pos2)  # (dq, dk) += (d c2p . K_r, d p2c . Q_r)
             # the reduction over the tokens has few output tiles: one call over 2H matrices, on a stacked copy of q and k
             dpos2 = into_pos(d_scores2, torch.stack([heads_first(q), heads_first(k)]).view(2 * H, B * L, D), None)
         dpk, dpq = pad_rows(dpos2[:H], pos_key), pad_rows(dpos2[H:], pos_query)
     elif pos_key is not None or pos_query is not None:
-        pos, x, d_s = (pos_key, q, d_c2p) if pos_key is not None else (pos_query, k, d_p2c)
+        pos, x, dx, d_s = (pos_key, q, dq, d_c2p) if pos_key is not None else (pos_query, k, dk, d_p2c)
         pos_t = pos[:, :2 * span].to(q.dtype)
         if fused:
-            dpos = chain_through_tables(d_s, heads_first(x), pos_t.contiguous(), x_hm[0])
+            dpos = chain_through_tables(d_s, heads_first(x), pos_t.contiguous(), dx.permute(2, 0, 1, 3).view(H, B * L, D))
         else:
             x_hm[0].baddbmm_(d_s, pos_t)
             dpos = into_pos(d_s, heads_first(x), None)

@@ -253,17 +253,19 @@ int fdb_attn_bwd(const fdb_attn_bwd_args* a, void* stream);
  * x + m * x_stride_matrix + r * x_stride_row for m < first_matrices, at x_second + (m - first_matrices) *
  * x_stride_matrix + r * x_stride_row beyond, in elements, head_dim contiguous elements each -- q and k are read
  * where they lie; x_second may be NULL when first_matrices == matrices) and
- * pos [matrices][2 * att_span][head_dim] (K_r resp. Q_r), g, pos and dx contiguous, all of element type `dtype`:
- *     dx [matrices][rows][head_dim]                      += g . pos     (in place, fp32 accumulation, one rounding)
+ * pos [matrices][2 * att_span][head_dim] (K_r resp. Q_r), g and pos contiguous, all of element type `dtype`:
+ *     dx (rows addressed like those of x, through dx / dx_second and dx_stride_matrix / dx_stride_row: dq and dk are
+ *         updated where they lie)                        += g . pos     (in place, fp32 accumulation, one rounding)
  *     dpos_parts [parts][matrices][2 * att_span][head_dim] = partial sums of g^T . x over `parts` shares of the rows
  *                                                           (fp32; the caller adds the parts up)
  * Built for head_dim 64, att_span 256, FDB_BF16 / FDB_F16, rows a multiple of 32, 1 <= parts <= rows / 32, pointers
- * and the strides of x (in bytes) aligned to 16 bytes; anything else is refused (FDB_ERR_HEAD_DIM / _SPAN / _DTYPE / _SHAPE / _ALIGN) and the caller
+ * and the strides of x and dx (in bytes) aligned to 16 bytes; anything else is refused (FDB_ERR_HEAD_DIM / _SPAN / _DTYPE / _SHAPE / _ALIGN) and the caller
  * takes the two matrix products instead.  Reference: the autograd backward of model.py:189-192 (see the list above).
  */
-int fdb_attn_bwd_chain(const void* d_scores, const void* x, const void* x_second, const void* pos, void* dx, float* dpos_parts,
-                       int32_t matrices, int32_t first_matrices, int64_t rows, int64_t x_stride_matrix, int64_t x_stride_row,
-                       int32_t att_span, int32_t head_dim, int32_t dtype, int32_t parts, void* stream);
+int fdb_attn_bwd_chain(const void* d_scores, const void* x, const void* x_second, const void* pos, void* dx, void* dx_second,
+                       float* dpos_parts, int32_t matrices, int32_t first_matrices, int64_t rows, int64_t x_stride_matrix,
+                       int64_t x_stride_row, int64_t dx_stride_matrix, int64_t dx_stride_row, int32_t att_span, int32_t head_dim,
+                       int32_t dtype, int32_t parts, void* stream);
 
 /*
  * Bytes of workspace the call would use (0: none), for the device that is current.  A launch whose

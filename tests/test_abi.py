@@ -495,11 +495,13 @@ def _good_bwd_args():
 
 def test_chain_argument_validation_codes():
     """fdb_attn_bwd_chain refuses what its kernel is not built for before anything touches the GPU."""
-    f = lambda g=0x1000, x=0x2000, x2=0x2800, pos=0x3000, dx=0x4000, parts_out=0x5000, m=24, m1=12, rows=4096, sm=64, sr=768, span=256, d=64, \
-        dt=_lib.FDB_BF16, parts=10: lib.fdb_attn_bwd_chain(g, x, x2, pos, dx, parts_out, m, m1, rows, sm, sr, span, d, dt, parts, None)
-    assert f(g=None) == -1 and f(parts_out=None) == -1 and f(x2=None) == -1   # matrices beyond the first tensor's need the second
-    assert f(m1=0) == -5 and f(m1=25) == -5 and f(sr=32) == -5
-    assert f(sm=4) == -4 and f(sr=772) == -4 and f(x2=0x2804) == -4
+    f = lambda g=0x1000, x=0x2000, x2=0x2800, pos=0x3000, dx=0x4000, dx2=0x4800, parts_out=0x5000, m=24, m1=12, rows=4096, sm=64, sr=768, \
+        dsm=64, dsr=768, span=256, d=64, dt=_lib.FDB_BF16, parts=10: \
+        lib.fdb_attn_bwd_chain(g, x, x2, pos, dx, dx2, parts_out, m, m1, rows, sm, sr, dsm, dsr, span, d, dt, parts, None)
+    assert f(g=None) == -1 and f(parts_out=None) == -1
+    assert f(x2=None) == -1 and f(dx2=None) == -1   # matrices beyond the first tensor's need the second
+    assert f(m1=0) == -5 and f(m1=25) == -5 and f(sr=32) == -5 and f(dsm=32) == -5 and f(dsr=0) == -5
+    assert f(sm=4) == -4 and f(sr=772) == -4 and f(x2=0x2804) == -4 and f(dsr=772) == -4 and f(dx2=0x4808) == -4
     assert f(dt=_lib.FDB_F32) == -2 and f(dt=_lib.FDB_FP8_E4M3) == -2
     assert f(d=32) == -3 and f(d=128) == -3
     assert f(x=0x2008) == -4 and f(dx=0x4004) == -4

@@ -1293,7 +1293,10 @@ def test_chain_through_tables_matches_the_two_matrix_products(M, N, dtype):
         # the token rows as two strided views of token-major tensors, the way q and k reach the operator
         xa, xb = [torch.empty(N, M // 2, 64, dtype=dtype, device="cuda") for _ in range(2)]
         xa.copy_(x[:M // 2].transpose(0, 1)); xb.copy_(x[M // 2:].transpose(0, 1))
-        dpos = ops.chain_through_tables(d_scores, xa.transpose(0, 1), pos, dx, x_second=xb.transpose(0, 1))
+        da, db = [torch.empty(N, M // 2, 64, dtype=dtype, device="cuda") for _ in range(2)]
+        da.copy_(dx0[:M // 2].transpose(0, 1)); db.copy_(dx0[M // 2:].transpose(0, 1))
+        dpos = ops.chain_through_tables(d_scores, xa.transpose(0, 1), pos, da.transpose(0, 1), x_second=xb.transpose(0, 1), dx_second=db.transpose(0, 1))
+        dx = torch.cat([da.transpose(0, 1), db.transpose(0, 1)])
     else:
         dpos = ops.chain_through_tables(d_scores, x, pos, dx)
     ref_dx = dx0.float() + torch.bmm(d_scores.float(), pos.float())
