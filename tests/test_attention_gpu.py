@@ -1843,12 +1843,13 @@ def test_backward_stores_every_entry_of_a_real_tokens_row(L, pb, mr, causal, len
             assert torch.isnan(dirty[b, n:]).all()
 
 
-@pytest.mark.parametrize("what", ["no_alloc_forward", "backward"])
+@pytest.mark.parametrize("what", ["no_alloc_forward", "backward", "backward_chain_kernel"])
 def test_more_replays_from_a_hip_graph(what):
     """The entry point that allocates nothing (the case it exists for) and the backward operator (two launches and
-    torch's fills and GEMMs around them) captured into a HIP graph: three replays on fresh input values, with eager
-    work and synchronisations in between, each equal to the eager result on the same values."""
-    B, L, H, D, pb, mr = 2, 700, 2, 64, 32, 64
+    torch's fills and GEMMs around them; with v3 buckets and a multiple of 32 rows, the chain kernel and the sum of its
+    partial table gradients in place of two of the GEMMs) captured into a HIP graph: three replays on fresh input
+    values, with eager work and synchronisations in between, each equal to the eager result on the same values."""
+    B, L, H, D, pb, mr = (2, 704, 2, 64, 256, 512) if what == "backward_chain_kernel" else (2, 700, 2, 64, 32, 64)
     kw = dict(position_buckets=pb, max_relative_positions=mr)
     q, k, v, pk, pq = [_dev(x) for x in _inputs(B, L, H, D, pb, mr, torch.bfloat16, 910, 1.0)]
     dout = torch.randn(B, L, H, D, generator=torch.Generator().manual_seed(911)).to(torch.bfloat16).cuda()
