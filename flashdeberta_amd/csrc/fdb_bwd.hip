@@ -114,8 +114,28 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63, li = lane & 31, g = lane >> 5;
-  const int h = blockIdx.y, b = blockIdx.z;
-  const int m0 = blockIdx.x * FDB_BM;
+  // Linear workgroup id -> (tile of lane-side rows, head, batch row).  The hardware deals workgroups to the 8 XCDs
+  // round-robin by linear id and each XCD has its own L2: where the launcher asks for it (p.pairs_per_xcd: the (batch
+  // row, head) pairs are a multiple of 8 and the launch is more than two rounds of workgroups), pairs are dealt to
+  // XCDs whole, so that all tiles of a pair stream the same loop-side rows (tiles and position scores) through one L2,
+  // one after the other in dispatch order.  A causal dQ launch deals a pair's tiles last first: those see the most keys.
+  const int tiles_x = (p.L + FDB_BM - 1) / FDB_BM;
+  int h, b, tile_x;
+  {
+    const int n = blockIdx.x;
+    if (p.pairs_per_xcd) {
+      const int slot = n >> 3, pair = (n & 7) + 8 * (slot / tiles_x);
+      tile_x = slot % tiles_x;
+      b = pair / p.H;
+      h = pair % p.H;
+    } else {
+      tile_x = n % tiles_x;
+      h = (n / tiles_x) % p.H;
+      b = n / (tiles_x * p.H);
+    }
+    if (kDQ && p.causal) tile_x = tiles_x - 1 - tile_x;
+  }
+  const int m0 = tile_x * FDB_BM;
   const int tok0 = p.seq_start ? min(max(p.seq_start[b], 0), p.L) : 0;
   const int Lb = p.seq_len ? min(max(p.seq_len[b], 0), p.L - tok0) : p.L;
   if (m0 >= Lb) return;
@@ -615,7 +635,7 @@ int launch_bwd_one(const FdbBwdParams& p, hipStream_t stream) {
   hipError_t e = fdb_set_lds_once((const void*)kern, 160 * 1024, lds_set);
   if (e != hipSuccess) return (int)e;
   const unsigned tiles = (unsigned)((p.L + FDB_BM - 1) / FDB_BM);
-  hipLaunchKernelGGL(kern, dim3(tiles, (unsigned)p.H, (unsigned)p.B), dim3(kBwdThreads), lds, stream, p);
+  hipLaunchKernelGGL(kern, dim3(tiles * (unsigned)p.H * (unsigned)p.B), dim3(kBwdThreads), lds, stream, p);
   return (int)hipGetLastError();
 }
 

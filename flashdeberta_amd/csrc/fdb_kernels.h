@@ -82,6 +82,7 @@ struct FdbBwdParams {
   int32_t S;        // att_span
   int32_t R;        // table radius
   int32_t causal;
+  int32_t pairs_per_xcd;  // workgroup ids map to (tile, head, batch row) with whole (batch row, head) pairs per XCD
   float scale_log2; // sm_scale * log2(e)
   float sm_scale;
 };
