@@ -548,6 +548,8 @@ int fdb_attn_bwd(const fdb_attn_bwd_args* a, void* stream) {
   const int64_t tiles = ((int64_t)a->seqlen + FDB_BM - 1) / FDB_BM, pairs = (int64_t)a->batch * a->heads;
   if (tiles * pairs > INT32_MAX) return FDB_ERR_SHAPE;
   p.pairs_per_xcd = (pairs % 8 == 0 && tiles * pairs > 4 * (int64_t)cu_count()) ? 1 : 0;
+  // the ring holds a step's window, a partly stored group and, with chunked stores, up to seven or three more complete groups
+  p.store_chunks = !has_pos ? 1 : a->lut_window + 4 + 28 <= FDB_BWD_RING ? 8 : a->lut_window + 4 + 12 <= FDB_BWD_RING ? 4 : 1;
   return fdb_launch_bwd(p, a->dtype, a->head_dim, stream);
 }
 

@@ -522,7 +522,15 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
       int n_g = 0;
       if (!settled) {
         const int d_edge = delta_of(has_next ? (kDQ ? xr - (y0 + kBwdStep) : y0 + kBwdStep - xr) : (kDQ ? xr - (y_hi - 1) : y_hi - 1 - xr));
-        n_g = !x_ok ? 0 : kDir * ((d_edge >> 2) - g_next) + (has_next ? 0 : 1);
+        int g_edge = d_edge >> 2;
+        // Where the ring has the room (p.store_chunks = 8 or 4 groups; 1: none), what leaves before the last step leaves
+        // in whole chunks, 64 or 32 bytes at a multiple of as much: every such sector of the tensor is then written
+        // once, not in two pieces.
+        if (has_next) {
+          const int cm = p.store_chunks - 1;
+          g_edge = kDir > 0 ? (g_edge & ~cm) : ((g_edge + cm + 1) & ~cm) - 1;
+        }
+        n_g = !x_ok ? 0 : kDir * (g_edge - g_next) + (has_next ? 0 : 1);
       }
       while (__builtin_amdgcn_ballot_w64(n_g > 0) != 0) {
         const int n_now = max(0, min(n_g, 8));

@@ -83,6 +83,7 @@ struct FdbBwdParams {
   int32_t R;        // table radius
   int32_t causal;
   int32_t pairs_per_xcd;  // workgroup ids map to (tile, head, batch row) with whole (batch row, head) pairs per XCD
+  int32_t store_chunks;   // score gradients leave the ring in aligned chunks of this many groups of four entries: 8, 4 or 1 (as the table's window leaves room)
   float scale_log2; // sm_scale * log2(e)
   float sm_scale;
 };

@@ -441,6 +441,41 @@ def test_backward_window_of_every_accepted_table():
     assert ops.delta_lut_window(256, 512) <= 31
 
 
+def test_backward_ring_holds_the_chunked_stores():
+    """Score gradients leave the 64-entry ring of a row in aligned chunks of 8, 4 or 1 groups of four entries, as the
+    table's window leaves room (fdb_attn_bwd: lut_window + 4 + 28, + 12 or + 0 within the ring).  Replay of the kernel's
+    bookkeeping on the host for every accepted table of the grid, both directions and every phase of the 32-row steps
+    against the table: the entries between the oldest one not yet stored and the newest one touched never exceed the ring."""
+    ring = 64
+    grid = [(pb, mr) for pb in (0, 4, 8, 16, 32, 64, 100, 128, 256, 512) for mr in (3, 8, 16, 24, 40, 64, 100, 128, 200, 256, 300, 512, 600, 1024)]
+    checked = 0
+    for pb, mr in grid:
+        if lib.fdb_delta_lut_radius(pb, mr) < 1:
+            continue
+        w = ops.delta_lut_window(pb, mr)
+        if w > _lib.FDB_BWD_MAX_WINDOW:
+            continue
+        chunk = 8 if w + 4 + 28 <= ring else 4 if w + 4 + 12 <= ring else 1
+        lut, radius = ops.delta_lut_host(pb, mr)
+        lut = lut.astype(np.int64)
+        delta = lambda r: int(lut[min(max(r, -radius), radius) + radius])
+        for r0 in range(-radius - 40, radius + 41, 1 if radius <= 64 else 3):
+            # dK/dV role: the relative position grows with the loop row, the window moves up
+            g_next = delta(r0) >> 2
+            for k in range((2 * radius + 160) // 32):
+                lo_r = r0 + 32 * k
+                assert delta(lo_r + 31) - 4 * g_next + 1 <= ring, (pb, mr, r0, k)
+                g_next = max(g_next, (delta(lo_r + 32) >> 2) & ~(chunk - 1))
+            # dQ role: it falls, the window moves down
+            g_next = delta(r0) >> 2
+            for k in range((2 * radius + 160) // 32):
+                hi_r = r0 - 32 * k
+                assert 4 * g_next + 3 - delta(hi_r - 31) + 1 <= ring, (pb, mr, r0, k)
+                g_next = min(g_next, (((delta(hi_r - 32) >> 2) + chunk) & ~(chunk - 1)) - 1)
+        checked += 1
+    assert checked > 60
+
+
 def _header_struct_fields(name):
     """(field name, C type) pairs of `typedef struct <name> { ... } <name>;` in include/fdb.h, in order."""
     text = open(os.path.join(ROOT, "include", "fdb.h")).read()
