@@ -541,13 +541,13 @@ int fdb_attn_bwd(const fdb_attn_bwd_args* a, void* stream) {
   p.causal = a->causal ? 1 : 0;
   p.sm_scale = a->sm_scale;
   p.scale_log2 = a->sm_scale * 1.4426950408889634f;
-  // One workgroup per 128 rows, head and batch row, in a one-dimensional grid.  With the (batch row, head) pairs a
-  // multiple of 8 and more than two rounds of workgroups (two per CU), whole pairs go to one XCD each: the tiles of a
+  // One workgroup per 128 rows, head and batch row, in a one-dimensional grid.  With at least eight (batch row, head)
+  // pairs and more than two rounds of workgroups (two per CU), whole pairs go to one XCD each, eight at a time: the tiles of a
   // pair then share the loop-side rows through that XCD's L2 (B = 8, L = 4096: 3.30 -> 3.12 ms for the two launches,
   // causal 2.83 -> 2.03); a launch of at most two rounds is a little faster with the tiles of a pair spread out.
   const int64_t tiles = ((int64_t)a->seqlen + FDB_BM - 1) / FDB_BM, pairs = (int64_t)a->batch * a->heads;
   if (tiles * pairs > INT32_MAX) return FDB_ERR_SHAPE;
-  p.pairs_per_xcd = (pairs % 8 == 0 && tiles * pairs > 4 * (int64_t)cu_count()) ? 1 : 0;
+  p.pairs_per_xcd = (pairs >= 8 && tiles * pairs > 4 * (int64_t)cu_count()) ? 1 : 0;
   // the ring holds a step's window, a partly stored group and, with chunked stores, up to seven or three more complete groups
   p.store_chunks = !has_pos ? 1 : a->lut_window + 4 + 28 <= FDB_BWD_RING ? 8 : a->lut_window + 4 + 12 <= FDB_BWD_RING ? 4 : 1;
   return fdb_launch_bwd(p, a->dtype, a->head_dim, stream);

@@ -115,17 +115,23 @@ __global__ __launch_bounds__(kBwdThreads, (D * QT::SZ <= 128 ? 2 : 1)) void fdb_
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63, li = lane & 31, g = lane >> 5;
   // Linear workgroup id -> (tile of lane-side rows, head, batch row).  The hardware deals workgroups to the 8 XCDs
-  // round-robin by linear id and each XCD has its own L2: where the launcher asks for it (p.pairs_per_xcd: the (batch
-  // row, head) pairs are a multiple of 8 and the launch is more than two rounds of workgroups), pairs are dealt to
-  // XCDs whole, so that all tiles of a pair stream the same loop-side rows (tiles and position scores) through one L2,
+  // round-robin by linear id and each XCD has its own L2: where the launcher asks for it (p.pairs_per_xcd: at least
+  // eight (batch row, head) pairs and more than two rounds of workgroups), pairs are dealt to XCDs whole, eight at a
+  // time, so that all tiles of a pair stream the same loop-side rows (tiles and position scores) through one L2,
   // one after the other in dispatch order.  A causal dQ launch deals a pair's tiles last first: those see the most keys.
   const int tiles_x = (p.L + FDB_BM - 1) / FDB_BM;
   int h, b, tile_x;
   {
     const int n = blockIdx.x;
-    if (p.pairs_per_xcd) {
+    const int whole = (p.B * p.H) & ~7;   // pairs dealt to XCDs whole; the rest follow in the plain order
+    if (p.pairs_per_xcd && n < whole * tiles_x) {
       const int slot = n >> 3, pair = (n & 7) + 8 * (slot / tiles_x);
       tile_x = slot % tiles_x;
+      b = pair / p.H;
+      h = pair % p.H;
+    } else if (p.pairs_per_xcd) {
+      const int rest = n - whole * tiles_x, pair = whole + rest / tiles_x;
+      tile_x = rest % tiles_x;
       b = pair / p.H;
       h = pair % p.H;
     } else {
