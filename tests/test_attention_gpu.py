@@ -1507,6 +1507,22 @@ def test_backward_at_the_benchmark_length():
     runs = [ops.disentangled_attention_bwd(q, k, v, out, lse, dout, pk, pq, position_buckets=pb, max_relative_positions=mr) for _ in range(2)]
     for n, a, b in zip(("dq", "dk", "dv", "dK_r", "dQ_r"), *runs):
         assert not torch.isnan(a).any() and torch.equal(a, b), n
+    # The workgroups of such a launch are dealt to the XCDs by (batch row, head) pair, eight pairs at a time and the rest
+    # in the plain order; a batch row on its own (twelve pairs in one round of workgroups) takes the plain order throughout,
+    # which the oracle has just checked.  Same bits for dq, dk, dv of a batch row either way, causal (where the dQ launch
+    # also reverses the order of a pair's tiles) or not, with a number of pairs that is a multiple of 8 or not.
+    for Bn, causal, rows in ((8, False, (0, 5)), (3, False, (2,)), (3, True, (0, 2))):
+        kw = dict(position_buckets=pb, max_relative_positions=mr, causal=causal)
+        sl = lambda x: x[:Bn]
+        out, lse = ops.disentangled_attention_fwd(sl(q), sl(k), sl(v), pk, pq, return_lse=True, **kw)
+        whole = ops.disentangled_attention_bwd(sl(q), sl(k), sl(v), out, lse, sl(dout), pk, pq, **kw)
+        for b in rows:
+            one = lambda x: x[b:b + 1].contiguous()
+            # (the forward's output and log-sum-exp of the whole batch: a batch row alone shares its far keys among
+            # workgroups and rounds differently)
+            alone = ops.disentangled_attention_bwd(one(q), one(k), one(v), one(out), lse[b * L:(b + 1) * L].contiguous(), one(dout), pk, pq, **kw)
+            for n, a, w in zip(("dq", "dk", "dv"), alone, whole):
+                assert torch.equal(a, w[b:b + 1]), "B=%d causal=%s row %d: %s" % (Bn, causal, b, n)
 
 
 def test_backward_refuses_an_odd_span():
