@@ -251,7 +251,7 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
   const int lane = tid & 63, li = lane & 31, g = lane >> 5;
   int xq, h;
   block_map((int)blockIdx.x, p.grid_x, p.H, p.tiles_per_seq, p.cu == nullptr,
-            MODE == kFarOnly ? kEdgesFirst : (MODE == kNearRing ? kMiddleFirst : kNatural), xq, h);
+            MODE == kFarOnly ? (p.causal ? kLastFirst : kEdgesFirst) : (MODE == kNearRing ? kMiddleFirst : kNatural), xq, h);
 
   int b, m0, tok0, Lb;
   int64_t qo, ko, vo, oo;

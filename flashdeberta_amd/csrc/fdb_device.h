@@ -261,8 +261,9 @@ __device__ __forceinline__ float scratch_add_hi<float>(float acc, uint32_t) { re
 // whole: all query tiles of a group then stream the same K and V through one L2.
 // Within a group the query tiles are dealt in the order `order` asks for, so that the workgroups
 // with the most key tiles start first and the launch ends on the short ones: kEdgesFirst for the far
-// tiles (a query tile at either end of the sequence has the most), kMiddleFirst for the near tiles.
-enum { kNatural = 0, kEdgesFirst = 1, kMiddleFirst = 2 };
+// tiles (a query tile at either end of the sequence has the most), kMiddleFirst for the near tiles, kLastFirst for
+// the far tiles of a causal call (a query tile sees the keys before it: the last one has the most).
+enum { kNatural = 0, kEdgesFirst = 1, kMiddleFirst = 2, kLastFirst = 3 };
 __device__ __forceinline__ void block_map(int n, int nx, int heads, int tiles_per_seq, bool fixed, int order, int& xq,
                                           int& h) {
   const int groups = fixed ? (nx / tiles_per_seq) * heads : 1;
@@ -270,7 +271,9 @@ __device__ __forceinline__ void block_map(int n, int nx, int heads, int tiles_pe
     const int xcd = n & 7, slot = n >> 3;
     const int grp = xcd + 8 * (slot / tiles_per_seq);
     int t = slot % tiles_per_seq;
-    if (order != kNatural) {
+    if (order == kLastFirst) {
+      t = tiles_per_seq - 1 - t;
+    } else if (order != kNatural) {
       if (order == kMiddleFirst) t = tiles_per_seq - 1 - t;
       t = (t & 1) ? tiles_per_seq - 1 - (t >> 1) : (t >> 1);  // 0, T-1, 1, T-2, ...
     }

@@ -87,7 +87,7 @@ __global__ __launch_bounds__(kThreads, 3) void fdb_far8_kernel(const FdbKParams 
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63, li = lane & 31, g = lane >> 5;
   int xq, h;
-  block_map((int)blockIdx.x, p.grid_x, p.H, p.tiles_per_seq, p.cu == nullptr, kEdgesFirst, xq, h);
+  block_map((int)blockIdx.x, p.grid_x, p.H, p.tiles_per_seq, p.cu == nullptr, p.causal ? kLastFirst : kEdgesFirst, xq, h);
 
   int b, m0, tok0, Lb;
   int64_t qo, ko, vo, oo;
