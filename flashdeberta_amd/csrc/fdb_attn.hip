@@ -546,9 +546,8 @@ __global__ __launch_bounds__(kThreads, (min_blocks<QT, VT, D, C2P, P2C, MODE>())
     }
   };
   // Tiles that need no mask: entirely inside the sequence and, when causal, entirely below the
-  // diagonal of every row of the workgroup, i.e. ending at or before its first row m0 (causal runs keep
-  // it simple beyond that: all near tiles are masked; without a position term there are no near tiles).
-  const int n_full = p.causal ? min(min(Lb / FDB_BN, t_near0), m0 / FDB_BN) : Lb / FDB_BN;
+  // diagonal of every row of the workgroup, i.e. ending at or before its first row m0.
+  const int n_full = p.causal ? min(Lb, m0) / FDB_BN : Lb / FDB_BN;
   auto far_loop = [&](auto mask_tag, int t0, int t1) __attribute__((always_inline)) {
     constexpr bool MASK = decltype(mask_tag)::value;
     for (int t = t0; t < t1; ++t) {

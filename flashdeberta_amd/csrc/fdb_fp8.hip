@@ -471,7 +471,7 @@ __global__ __launch_bounds__(kThreads, 3) void fdb_near8_kernel(const FdbKParams
     s0 = s0 + (int)((int64_t)all * part / p.near_parts);
   }
   const int n_steps = s1 - s0;
-  const int n_full = p.causal ? 0 : max(0, min(n_steps, Lb / kStep - s0));
+  const int n_full = max(0, min(n_steps, (p.causal ? min(Lb, m0) : Lb) / kStep - s0));
   // u = r_hi0 - r counts downwards from the first step's largest r; batch = u / 32, ring slot = batch mod 5 (E_K) or 6 (E_Q).  Wave w's
   // block bk at step k is batch k + 4 - w - bk, MFMA row m its row 31 - m: r = iw0 - 32 s - 32 + 32 bk + m.
   const int r_hi0 = m0 + FDB_BM - 1 - s0 * kStep;

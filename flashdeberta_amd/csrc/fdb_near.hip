@@ -178,7 +178,7 @@ __global__ __launch_bounds__(kNThreads, 2) void fdb_near_kernel(const FdbKParams
     s0 = s0 + (int)((int64_t)all * part / p.near_parts);
   }
   const int n_steps = s1 - s0;
-  const int n_full = p.causal ? 0 : max(0, min(n_steps, Lb / kStep - s0));  // steps k < n_full need no mask
+  const int n_full = max(0, min(n_steps, (p.causal ? min(Lb, m0) : Lb) / kStep - s0));  // steps k < n_full need no mask
 
   // relative positions of the workgroup at step k = s - s0: r in [r_hi0 - 32k - 159, r_hi0 - 32k];
   // u = r_hi0 - r counts downwards from the first step's largest r; batch = u / 32, ring slot = batch mod 5.
